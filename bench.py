@@ -1,0 +1,238 @@
+"""Benchmark of the embedding-cache hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5] [--mode fast|exact]
+
+One step = lookup + cached_fetch of the query rows, combine of the per-query gradients, and the
+sparse Adagrad update of every distinct row, on one batch of synthetic Zipf ids that is already
+resident in HBM.  Prints ONE JSON line: whole-step throughput in query rows/s, the roofline of the
+dominant kernel (algorithmic bytes / HIP-event time of its launches inside the timed region) and
+the same step timed on the host cores with the CPU oracle.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+PCIE_PEAK_GBS = 64.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
+    ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
+    ap.add_argument("--batches", type=int, default=4, help="distinct pre-generated id batches")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    return ap.parse_args()
+
+
+class Workload:
+    """Tables, hot set and pre-generated batches of one configuration, resident on the device
+    (cold table in pinned host memory for cfg3)."""
+
+    def __init__(self, name, nbatches, device):
+        import torch
+        from hades_amd import synth
+        from hades_amd.sparse_optim import SparseAdagrad
+        cfg = synth.CONFIGS[name]
+        self.name, self.cfg = name, cfg
+        N, D, H = cfg["num_rows"], cfg["dim"], cfg["num_hot"]
+        self.N, self.D, self.H = N, D, H
+        self.trainers = cfg.get("trainers", 1)
+        self.n = cfg["batch"] * self.trainers
+        self.host_cold = name == "cfg3"
+        seed = 1234 + int(name[3:])
+        if self.host_cold:
+            table = torch.empty((N, D), dtype=torch.float32, pin_memory=True)
+        else:
+            table = torch.empty((N, D), dtype=torch.float32, device=device)
+        synth.fill_normal_(table, 0.01, seed)
+        hot_ids = synth.hot_ids(N, H, device) if H else torch.empty(0, dtype=torch.int64, device=device)
+        self.opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=device)
+        sampler = synth.ZipfSampler(N, cfg["zipf_s"], device)
+        self.ids, self.grads = [], []
+        for b in range(nbatches):
+            parts = [synth.make_ids(sampler, N, cfg["batch"], seed * 1000 + b * 16 + t)
+                     for t in range(self.trainers)]
+            self.ids.append(torch.cat(parts).contiguous())
+            self.grads.append(synth.make_grads(self.n, D, seed * 2000 + b, device))
+        del sampler
+        self.rows_out = torch.empty((self.n, D), dtype=torch.float32, device=device)
+        self.comb_out = (torch.empty(self.n, dtype=torch.int64, device=device),
+                         torch.empty((self.n, D), dtype=torch.float32, device=device),
+                         torch.empty(self.n, dtype=torch.int64, device=device),
+                         torch.empty(1, dtype=torch.int64, device=device))
+
+    def describe(self):
+        return ("%s: %d x %d fp32 table (%s), hot %d rows in HBM, %d ids/step zipf s=%.2f%s" %
+                (self.name, self.N, self.D, "cold rows in pinned host memory" if self.host_cold
+                 else "all in HBM", self.H, self.n, self.cfg["zipf_s"],
+                 ", %d trainer batches concatenated" % self.trainers if self.trainers > 1 else ""))
+
+
+def run_gpu(args):
+    import torch
+    from hades_amd import ops
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    wl = Workload(args.workload, args.batches, dev)
+    opt = wl.opt
+    mode = ops.COMBINE_FAST if args.mode == "fast" else ops.COMBINE_EXACT
+    ws = ops.Workspace(dev)
+    nb = len(wl.ids)
+    phases = ("fetch", "combine", "update")
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+
+    def step(i, events=None):
+        q, g = wl.ids[i % nb], wl.grads[i % nb]
+        if events: events[0].record()
+        ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_ids, out=wl.rows_out)
+        if events: events[1].record()
+        uids, sums, cnts, nu = ops.combine_padded(q, g, id_bound=wl.N, mode=mode, workspace=ws,
+                                                  out=wl.comb_out)
+        if events: events[2].record()
+        opt.update(uids, sums, nu)
+        if events: events[3].record()
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, ev[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    phase_ms = {p: sum(ev[i][k].elapsed_time(ev[i][k + 1]) for i in range(args.steps)) / args.steps
+                for k, p in enumerate(phases)}
+    # distinct ids per step and hot-hit statistics of the batches actually used
+    uniq, hot_hit, uniq_hot = [], [], []
+    for q in wl.ids:
+        u = torch.unique(q)
+        uniq.append(u.numel())
+        if wl.H:
+            hot_hit.append(float((ops.lookup(q, opt.hot_ids) >= 0).float().mean()))
+            uniq_hot.append(int((ops.lookup(u, opt.hot_ids) >= 0).sum()))
+        else:
+            hot_hit.append(0.0)
+            uniq_hot.append(0)
+    U = sum(uniq) / len(uniq)
+    U_hot = sum(uniq_hot) / len(uniq_hot)
+    hit = sum(hot_hit) / len(hot_hit)
+    n, D = wl.n, wl.D
+    # algorithmic bytes per launch of each phase (fp32): fetch 16 + 8D per query row;
+    # combine n(8+4D) read + U(16+4D) written; Adagrad 8 + 20D per distinct row
+    alg_bytes = {"fetch": n * (16 + 8 * D), "combine": n * (8 + 4 * D) + U * (16 + 4 * D),
+                 "update": U * (8 + 20 * D)}
+    dominant = max(phases, key=lambda p: phase_ms[p])
+    kernel_of = {"fetch": "row_move_kernel<AddrFetchSorted>", "combine": "hades_combine (sort + runs + seg_chunk_kernel + seg_fixup_kernel)",
+                 "update": "adagrad_kernel"}
+    achieved = alg_bytes[dominant] / (phase_ms[dominant] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": kernel_of[dominant], "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": None}
+    per_phase = {p: {"ms": round(phase_ms[p], 4),
+                     "GB/s": round(alg_bytes[p] / (phase_ms[p] * 1e-3) / 1e9, 1),
+                     "frac_hbm": round(alg_bytes[p] / (phase_ms[p] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                 for p in phases}
+    total_bytes = sum(alg_bytes.values())
+    extra = {"phases": per_phase, "step_alg_GB": round(total_bytes / 1e9, 4),
+             "step_GB/s": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+             "step_frac_hbm": round(total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+             "unique_per_step": round(U, 1), "unique_hot_per_step": round(U_hot, 1),
+             "hot_hit": round(hit, 4)}
+    if wl.host_cold:
+        cold_q = n * (1 - hit)
+        cold_u = U - U_hot
+        extra["pcie"] = {
+            "fetch_GB/s": round(cold_q * 4 * D / (phase_ms["fetch"] * 1e-3) / 1e9, 2),
+            "update_read_GB/s": round(cold_u * 8 * D / (phase_ms["update"] * 1e-3) / 1e9, 2),
+            "update_write_GB/s": round(cold_u * 8 * D / (phase_ms["update"] * 1e-3) / 1e9, 2),
+            "peak_per_direction": PCIE_PEAK_GBS}
+    return wl, ms_per_step, roofline, extra
+
+
+def run_cpu_baseline(wl_name, seconds):
+    """The same step with the CPU oracle (torch CPU ops, all host threads), on a bounded sample:
+    the benchmark's own batches at full table size when that fits the host, repeated for about
+    `seconds`."""
+    import torch
+    from hades_amd import synth
+    from oracle import hades_oracle as O
+    cfg = synth.CONFIGS[wl_name]
+    N, D, H = cfg["num_rows"], cfg["dim"], cfg["num_hot"]
+    sample = "full %s step" % wl_name
+    if N * D * 4 > 8 << 30:            # bound host memory: shrink the table, keep batch and skew
+        scale = (8 << 30) / (N * D * 4)
+        N, H = int(N * scale), int(H * scale)
+        sample = "%s batch and skew on a table cut to %d rows" % (wl_name, N)
+    seed = 1234 + int(wl_name[3:])
+    n = cfg["batch"] * cfg.get("trainers", 1)
+    cold_w = torch.empty((N, D))
+    synth.fill_normal_(cold_w, 0.01, seed)
+    cold_s = torch.zeros((N, D))
+    hot_ids = synth.hot_ids(N, H) if H else torch.empty(0, dtype=torch.int64)
+    hot_w, hot_s = cold_w[hot_ids].clone(), torch.zeros((hot_ids.numel(), D))
+    sampler = synth.ZipfSampler(N, cfg["zipf_s"])
+    q = synth.make_ids(sampler, N, n, seed * 1000)
+    g = synth.make_grads(n, D, seed * 2000)
+    O.torch_step(cold_w, cold_s, hot_w, hot_s, hot_ids, q, g, 0.01, 1e-10)   # warm-up
+    times = []
+    t_end = time.perf_counter() + seconds
+    while time.perf_counter() < t_end or len(times) < 3:
+        t0 = time.perf_counter()
+        O.torch_step(cold_w, cold_s, hot_w, hot_s, hot_ids, q, g, 0.01, 1e-10)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(n / med, 1), "unit": "rows/s", "cores": torch.get_num_threads(),
+            "kind": "port", "ms_per_step": round(med * 1e3, 3),
+            "sample": "%s, %d repetitions, median; torch CPU ops (searchsorted, index, unique + "
+                      "index_add_, addcmul/addcdiv)" % (sample, len(times))}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the all-to-all "
+              "gradient exchange is out of scope); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    wl, ms_per_step, roofline, extra = run_gpu(args)
+    n = wl.n
+    line = {
+        "metric": "embedding rows/s (fetch+combine+update)",
+        "value": round(n / (ms_per_step * 1e-3), 1),
+        "unit": "rows/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "step_us": round(ms_per_step * 1e3, 1),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": wl.describe(), "combine_mode": args.mode,
+                   "optimizer": "sparse Adagrad lr=0.01 eps=1e-10"},
+        "roofline": roofline,
+    }
+    line.update(extra)
+    del wl
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = run_cpu_baseline(args.workload, args.cpu_seconds)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,22 @@
+"""hades_amd - the HADES per-GPU embedding-cache hot path on MI355X (gfx950).
+
+    hades_amd.EmbCacheLib   drop-in for the reference's extension module (same operator names)
+    hades_amd.ops           fused operators: lookup, split, cached_fetch/set, combine, optimizers
+    hades_amd.cache         EmbCache: hot-row cache keyed by the sorted hot-ID set
+    hades_amd.sparse_optim  only_unique_grads / unique_grads / SparseAdagrad / SparseAdam
+
+All device work is done by csrc/libhades_hip.so (hand-written HIP, C ABI in include/hades_hip.h),
+built in-tree with `python -m hades_amd.build`.  There is no CPU fallback: without the library
+every operator raises.
+"""
+import sys
+
+__version__ = "0.1.0"
+
+
+def install_as_embcachelib():
+    """Registers hades_amd.EmbCacheLib under the name `EmbCacheLib`, so that unmodified reference
+    code (`import EmbCacheLib`, python/EmbCache/cache.py:2) binds to this implementation."""
+    from . import EmbCacheLib
+    sys.modules["EmbCacheLib"] = EmbCacheLib
+    return EmbCacheLib

@@ -1,0 +1,146 @@
+// Shared host/device helpers for libhades_hip.so (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/hades_hip.h"
+
+namespace hades {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// ---- error reporting: thread-local message, never exit() -------------------
+int set_error(int code, const char* fmt, ...);
+
+#define HADES_HIP_TRY(expr)                                                          \
+  do {                                                                               \
+    hipError_t _e = (expr);                                                          \
+    if (_e != hipSuccess) {                                                          \
+      (void)hipGetLastError();                                                       \
+      return ::hades::set_error(HADES_ERR_HIP, "%s:%d: %s failed: %s", __FILE__,     \
+                                __LINE__, #expr, hipGetErrorString(_e));             \
+    }                                                                                \
+  } while (0)
+
+#define HADES_REQUIRE(cond, ...)                                                     \
+  do {                                                                               \
+    if (!(cond)) return ::hades::set_error(HADES_ERR_ARG, __VA_ARGS__);              \
+  } while (0)
+
+// Launch-error check after every <<<>>> (the reference never checks its launches).
+#define HADES_LAUNCH_CHECK() HADES_HIP_TRY(hipGetLastError())
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+inline int ilog2_ceil(uint64_t x) {  // smallest b with 2^b >= x
+  int b = 0;
+  while (b < 64 && (uint64_t(1) << b) < x) ++b;
+  return b;
+}
+inline uintptr_t align_of_ptr(const void* p) { return reinterpret_cast<uintptr_t>(p); }
+
+// Carve aligned sub-buffers out of a caller-provided workspace.
+struct Carver {
+  char* base;
+  size_t off = 0;
+  explicit Carver(void* p) : base(static_cast<char*>(p)) {}
+  template <typename T>
+  T* take(size_t count) {
+    off = (off + 255) & ~size_t(255);
+    T* r = base ? reinterpret_cast<T*>(base + off) : nullptr;
+    off += count * sizeof(T);
+    return r;
+  }
+  size_t total() const { return (off + 255) & ~size_t(255); }
+};
+
+// ---- device helpers ---------------------------------------------------------
+#if defined(__HIPCC__)
+
+__device__ __forceinline__ int lane_id() { return __lane_id(); }
+
+// number of entries of ascending a[0..n) that are <= v  (std::upper_bound index)
+template <typename T>
+__device__ __forceinline__ int64_t upper_bound_dev(const T* __restrict__ a, int64_t n, T v) {
+  int64_t lo = 0, len = n;
+  while (len > 0) {
+    int64_t half = len >> 1;
+    T x = a[lo + half];
+    if (x <= v) {
+      lo += half + 1;
+      len -= half + 1;
+    } else {
+      len = half;
+    }
+  }
+  return lo;
+}
+
+// slot of v in the ascending duplicate-free set a[0..n), or -1
+__device__ __forceinline__ int64_t lookup_slot_dev(const int64_t* __restrict__ a, int64_t n,
+                                                   int64_t v) {
+  int64_t pos = upper_bound_dev<int64_t>(a, n, v);
+  return (pos > 0 && a[pos - 1] == v) ? pos - 1 : int64_t(-1);
+}
+
+// wave64 inclusive prefix sum of a 32-bit value over the lanes of a wavefront
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t v) {
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    uint32_t t = __shfl_up(v, d, kWave);
+    if (lane_id() >= d) v += t;
+  }
+  return v;
+}
+
+// lanes below mine whose ballot bit is set
+__device__ __forceinline__ uint32_t ballot_rank(uint64_t ballot) {
+  return __builtin_amdgcn_mbcnt_hi(uint32_t(ballot >> 32),
+                                   __builtin_amdgcn_mbcnt_lo(uint32_t(ballot), 0u));
+}
+
+#endif  // __HIPCC__
+
+}  // namespace hades
+
+#if defined(__HIPCC__)
+namespace hades {
+
+// Exclusive prefix sum of one value per thread over a block of kBlock threads (kBlock a multiple
+// of 64, at most 1024).  Returns the exclusive prefix; *total receives the block sum.  `smem`
+// must hold kBlock/64 + 1 elements of T.  Contains __syncthreads(): call from all threads.
+template <typename T, int kBlock>
+__device__ __forceinline__ T block_exclusive_sum(T v, T* smem, T* total) {
+  constexpr int kWaves = kBlock / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  T inc = v;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    T t = __shfl_up(inc, d, kWave);
+    if (lane >= d) inc += t;
+  }
+  if (lane == kWave - 1) smem[wave] = inc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    T run = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      T t = smem[w];
+      smem[w] = run;
+      run += t;
+    }
+    smem[kWaves] = run;
+  }
+  __syncthreads();
+  T res = smem[wave] + inc - v;
+  *total = smem[kWaves];
+  __syncthreads();  // smem may be reused by the caller
+  return res;
+}
+
+}  // namespace hades
+#endif

@@ -1,0 +1,27 @@
+// Building blocks shared between translation units of libhades_hip.so (not part of the C ABI).
+#pragma once
+
+#include "common.h"
+
+namespace hades {
+
+// index.hip: ascending positions i with keys[i] != -1, and their number (device).
+// pos_out needs capacity n.
+size_t compact_live_workspace_bytes(int64_t n);
+int compact_live_keys(const int64_t* keys, int64_t n, int64_t* pos_out, int64_t* count_out,
+                      void* workspace, size_t workspace_bytes, hipStream_t st);
+
+// combine.hip: stable radix sort of (id, position) over the bits id_bound leaves significant.
+// On return *perm_out[j] is the position in `ids` of the j-th smallest id and *sorted_keys the
+// sorted keys in the sort's own key type (*key64 tells which: uint64 with the sign bit flipped,
+// or uint32).  Both live in the workspace.
+struct SortResult {
+  const void* sorted_keys;
+  const uint32_t* perm;
+  bool key64;
+};
+size_t sort_ids_workspace_bytes(int64_t n);
+int sort_ids(const int64_t* ids, int64_t n, int64_t id_bound, void* workspace,
+             size_t workspace_bytes, hipStream_t st, SortResult* out);
+
+}  // namespace hades

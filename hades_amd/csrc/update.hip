@@ -1,0 +1,257 @@
+// Sparse row optimizers with the lookup, the state/weight gather and the scatter-back fused into
+// one kernel: sparse Adagrad, and the SparseAdam of the reference
+// (python/EmbCache/sparse_optim.py:590-685; state gather/scatter python/EmbCache/cache.py:66-131).
+//
+// A block owns kRows consecutive unique rows.  Phase 1: one thread per row searches the sorted hot
+// set and records where the row lives (hot slot in HBM, or the id itself for the cold tables,
+// which may be pinned host memory).  Phase 2: the block walks its rows as a flat list of float4
+// chunks (scalar when dim is not a multiple of 4): read g, state, w; write state, w.
+// This translation unit is compiled with fused multiply-add contraction off: every operation
+// rounds to fp32 on its own, like the CPU restatement it is checked against.
+#include "common.h"
+
+namespace hades {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kRows = 64;
+constexpr int kUnroll = 4;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int VEC>
+struct Vf;
+template <>
+struct Vf<4> {
+  typedef f32x4 type;
+};
+template <>
+struct Vf<1> {
+  typedef float type;
+};
+
+__device__ __forceinline__ float vsqrt(float x) { return __fsqrt_rn(x); }
+__device__ __forceinline__ f32x4 vsqrt(f32x4 x) {
+  return f32x4{__fsqrt_rn(x.x), __fsqrt_rn(x.y), __fsqrt_rn(x.z), __fsqrt_rn(x.w)};
+}
+__device__ __forceinline__ float vdiv(float a, float b) { return __fdiv_rn(a, b); }
+__device__ __forceinline__ f32x4 vdiv(f32x4 a, f32x4 b) {
+  return f32x4{__fdiv_rn(a.x, b.x), __fdiv_rn(a.y, b.y), __fdiv_rn(a.z, b.z), __fdiv_rn(a.w, b.w)};
+}
+
+struct RowArgs {
+  const int64_t* uids;
+  const float* grad;
+  const int64_t* num_unique;
+  int64_t max_rows;
+  int64_t dim;
+  const int64_t* sorted_hot;
+  int64_t num_hot;
+};
+
+struct AdagradArgs {
+  RowArgs r;
+  float* hot_w; float* hot_s; float* cold_w; float* cold_s;
+  float lr, eps;
+};
+
+struct AdamArgs {
+  RowArgs r;
+  float* hot_w; float* hot_step; float* hot_m; float* hot_v;
+  float* cold_w; float* cold_step; float* cold_m; float* cold_v;
+  float lr, beta1, beta2, one_minus_beta1, one_minus_beta2, eps;
+};
+
+// phase 1 shared by both optimizers: s_row[r] = element offset of the row in its table,
+// s_hot[r] = 1 if that table is the hot one.  Returns the number of live rows of this block.
+__device__ __forceinline__ int resolve_rows(const RowArgs& a, int64_t* s_row, uint8_t* s_hot) {
+  const int64_t U = a.num_unique ? a.num_unique[0] : a.max_rows;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRows;
+  const int64_t left = (U < a.max_rows ? U : a.max_rows) - row0;
+  const int rows_here = left >= kRows ? kRows : (left > 0 ? static_cast<int>(left) : 0);
+  for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+    const int64_t id = a.uids[row0 + r];
+    const int64_t loc = lookup_slot_dev(a.sorted_hot, a.num_hot, id);
+    s_row[r] = loc >= 0 ? loc : id;
+    s_hot[r] = loc >= 0 ? 1 : 0;
+  }
+  return rows_here;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void adagrad_kernel(AdagradArgs a) {
+  typedef typename Vf<VEC>::type V;
+  __shared__ int64_t s_row[kRows];
+  __shared__ uint8_t s_hot[kRows];
+  const int rows_here = resolve_rows(a.r, s_row, s_hot);
+  __syncthreads();
+  if (rows_here == 0) return;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRows;
+  const int cpr = static_cast<int>(a.r.dim / VEC);
+  const int total = rows_here * cpr;
+  for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
+    V g[kUnroll], s[kUnroll], w[kUnroll];
+    V* sp[kUnroll];
+    V* wp[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int c = base + k * kThreads;
+      if (c < total) {
+        const int r = c / cpr;
+        const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
+        const int64_t off = s_row[r] * a.r.dim + col;
+        sp[k] = reinterpret_cast<V*>((s_hot[r] ? a.hot_s : a.cold_s) + off);
+        wp[k] = reinterpret_cast<V*>((s_hot[r] ? a.hot_w : a.cold_w) + off);
+        g[k] = *reinterpret_cast<const V*>(a.r.grad + (row0 + r) * a.r.dim + col);
+        s[k] = *sp[k];
+        w[k] = *wp[k];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int c = base + k * kThreads;
+      if (c < total) {
+        const V s1 = s[k] + g[k] * g[k];
+        const V std_ = vsqrt(s1) + a.eps;
+        const V w1 = w[k] - vdiv(a.lr * g[k], std_);
+        *sp[k] = s1;
+        *wp[k] = w1;
+      }
+    }
+  }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void adam_kernel(AdamArgs a) {
+  typedef typename Vf<VEC>::type V;
+  __shared__ int64_t s_row[kRows];
+  __shared__ uint8_t s_hot[kRows];
+  __shared__ float s_c1[kRows];
+  __shared__ float s_c2[kRows];
+  const int rows_here = resolve_rows(a.r, s_row, s_hot);
+  // per-row step counter and bias corrections (thread r owns row r in both loops)
+  for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+    float* sp = (s_hot[r] ? a.hot_step : a.cold_step) + s_row[r];
+    const float step = *sp + 1.0f;
+    *sp = step;
+    s_c1[r] = 1.0f - powf(a.beta1, step);
+    s_c2[r] = 1.0f - powf(a.beta2, step);
+  }
+  __syncthreads();
+  if (rows_here == 0) return;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRows;
+  const int cpr = static_cast<int>(a.r.dim / VEC);
+  const int total = rows_here * cpr;
+  for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
+    V g[kUnroll], m[kUnroll], v[kUnroll], w[kUnroll];
+    V* mp[kUnroll];
+    V* vp[kUnroll];
+    V* wp[kUnroll];
+    float c1[kUnroll], c2[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int c = base + k * kThreads;
+      if (c < total) {
+        const int r = c / cpr;
+        const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
+        const int64_t off = s_row[r] * a.r.dim + col;
+        const bool hot = s_hot[r];
+        mp[k] = reinterpret_cast<V*>((hot ? a.hot_m : a.cold_m) + off);
+        vp[k] = reinterpret_cast<V*>((hot ? a.hot_v : a.cold_v) + off);
+        wp[k] = reinterpret_cast<V*>((hot ? a.hot_w : a.cold_w) + off);
+        g[k] = *reinterpret_cast<const V*>(a.r.grad + (row0 + r) * a.r.dim + col);
+        m[k] = *mp[k];
+        v[k] = *vp[k];
+        w[k] = *wp[k];
+        c1[k] = s_c1[r];
+        c2[k] = s_c2[r];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int c = base + k * kThreads;
+      if (c < total) {
+        const V m1 = a.beta1 * m[k] + a.one_minus_beta1 * g[k];
+        const V v1 = a.beta2 * v[k] + a.one_minus_beta2 * (g[k] * g[k]);
+        const V mc = vdiv(m1, V(c1[k]));
+        const V vc = vdiv(v1, V(c2[k]));
+        const V upd = vdiv(a.lr * mc, vsqrt(vc) + a.eps);
+        *mp[k] = m1;
+        *vp[k] = v1;
+        *wp[k] = w[k] - upd;
+      }
+    }
+  }
+}
+
+bool aligned16(std::initializer_list<const void*> ps) {
+  for (const void* p : ps)
+    if (p && (align_of_ptr(p) % 16) != 0) return false;
+  return true;
+}
+
+int check_rows(const int64_t* uids, const float* grad, int64_t max_rows, int64_t dim,
+               const int64_t* sorted_hot, int64_t num_hot) {
+  HADES_REQUIRE(max_rows >= 0 && dim >= 1, "max_rows must be >= 0 and dim >= 1");
+  HADES_REQUIRE(num_hot >= 0, "num_hot must be >= 0");
+  HADES_REQUIRE(max_rows == 0 || (uids && grad), "null pointer argument");
+  HADES_REQUIRE(num_hot == 0 || sorted_hot, "sorted_hot is null but num_hot > 0");
+  HADES_REQUIRE(dim * kRows < (int64_t(1) << 30), "dim too large");
+  HADES_REQUIRE(ceil_div(max_rows > 0 ? max_rows : 1, kRows) < (int64_t(1) << 31), "too many rows");
+  return HADES_OK;
+}
+
+}  // namespace
+}  // namespace hades
+
+using namespace hades;
+
+extern "C" {
+
+int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
+                         int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,
+                         float* hot_w, float* hot_s, float* cold_w, float* cold_s, float lr,
+                         float eps, void* stream) {
+  int rc = check_rows(uids, grad, max_rows, dim, sorted_hot, num_hot);
+  if (rc != HADES_OK) return rc;
+  if (max_rows == 0) return HADES_OK;
+  HADES_REQUIRE(num_hot == 0 || (hot_w && hot_s), "hot tables are null but num_hot > 0");
+  AdagradArgs a{{uids, grad, num_unique, max_rows, dim, sorted_hot, num_hot},
+                hot_w, hot_s, cold_w, cold_s, lr, eps};
+  const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dim % 4 == 0 && aligned16({grad, hot_w, hot_s, cold_w, cold_s}))
+    hipLaunchKernelGGL((adagrad_kernel<4>), grid, block, 0, st, a);
+  else
+    hipLaunchKernelGGL((adagrad_kernel<1>), grid, block, 0, st, a);
+  HADES_LAUNCH_CHECK();
+  return HADES_OK;
+}
+
+int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
+                      int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,
+                      float* hot_w, float* hot_step, float* hot_m, float* hot_v, float* cold_w,
+                      float* cold_step, float* cold_m, float* cold_v, float lr, float beta1,
+                      float beta2, float eps, void* stream) {
+  int rc = check_rows(uids, grad, max_rows, dim, sorted_hot, num_hot);
+  if (rc != HADES_OK) return rc;
+  if (max_rows == 0) return HADES_OK;
+  HADES_REQUIRE(num_hot == 0 || (hot_w && hot_step && hot_m && hot_v),
+                "hot tables are null but num_hot > 0");
+  // 1 - beta is formed in double like the reference's Python float arithmetic, then rounded
+  const float omb1 = static_cast<float>(1.0 - static_cast<double>(beta1));
+  const float omb2 = static_cast<float>(1.0 - static_cast<double>(beta2));
+  AdamArgs a{{uids, grad, num_unique, max_rows, dim, sorted_hot, num_hot},
+             hot_w, hot_step, hot_m, hot_v, cold_w, cold_step, cold_m, cold_v,
+             lr, beta1, beta2, omb1, omb2, eps};
+  const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dim % 4 == 0 && aligned16({grad, hot_w, hot_m, hot_v, cold_w, cold_m, cold_v}))
+    hipLaunchKernelGGL((adam_kernel<4>), grid, block, 0, st, a);
+  else
+    hipLaunchKernelGGL((adam_kernel<1>), grid, block, 0, st, a);
+  HADES_LAUNCH_CHECK();
+  return HADES_OK;
+}
+
+}  // extern "C"

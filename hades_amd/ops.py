@@ -1,0 +1,315 @@
+"""Fused operators of the embedding-cache hot path over torch-ROCm tensors.
+
+Thin, allocation-only wrappers around the C-ABI library: lookup against the sorted hot-ID set,
+hot/cold split with stable compaction, cached_fetch / cached_set, combine and the sparse row
+optimizers.  Every function launches on torch's current stream and returns without a host
+synchronisation unless its name or docstring says otherwise; data-dependent sizes stay on the
+device as one-element tensors (`num_unique`, `counts`) and outputs are padded to capacity.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from .EmbCacheLib import _check, _dev, _dev_or_pinned, _ptr, _stream
+
+COMBINE_FAST = _lib.COMBINE_FAST
+COMBINE_EXACT = _lib.COMBINE_EXACT
+
+_NULL = ctypes.c_void_p(0)
+
+
+def _i64(t, name):
+    _check(t.dtype == torch.int64, "%s must be int64" % name)
+    _dev(t, name)
+
+
+def _opt(t):
+    return _NULL if t is None else _ptr(t)
+
+
+def _dcode(t):
+    _check(t.dtype in (torch.float32, torch.float64), "Type can only be float or double")
+    return _lib.F32 if t.dtype == torch.float32 else _lib.F64
+
+
+class Workspace:
+    """A reusable, 256-byte aligned device scratch buffer that grows on demand."""
+
+    def __init__(self, device="cuda"):
+        self.device = torch.device(device)
+        self.buf = None
+
+    def get(self, nbytes):
+        if self.buf is None or self.buf.numel() < nbytes:
+            # zero-filled: the sort keeps a sticky status word at the start of its workspace
+            self.buf = torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=self.device)
+        return self.buf
+
+
+_default_ws = {}
+
+
+def _ws(device, kind):
+    key = (str(device), kind)
+    if key not in _default_ws:
+        _default_ws[key] = Workspace(device)
+    return _default_ws[key]
+
+
+# ---- lookup -------------------------------------------------------------------
+def lookup(ids, sorted_hot, out=None):
+    """loc[i] = slot of ids[i] in the ascending duplicate-free `sorted_hot`, or -1."""
+    _i64(ids, "ids"); _i64(sorted_hot, "sorted_hot")
+    loc = out if out is not None else torch.empty_like(ids)
+    _lib.call("hades_lookup_sorted", _ptr(ids), ids.numel(), _ptr(sorted_hot), sorted_hot.numel(),
+              _ptr(loc), _stream())
+    return loc
+
+
+# ---- split + compaction -------------------------------------------------------
+def split_padded(loc, workspace=None):
+    """Hot/cold split of a looked-up batch, no host synchronisation.
+
+    Returns (hot_mask bool[n], hot_pos int64[n], cold_pos int64[n], counts int64[2]); the first
+    counts[0] entries of hot_pos and counts[1] of cold_pos are the ascending positions of each
+    class, the rest is unspecified.
+    """
+    _i64(loc, "loc")
+    n = loc.numel()
+    hot_mask = torch.empty(n, dtype=torch.bool, device=loc.device)
+    hot_pos = torch.empty(n, dtype=torch.int64, device=loc.device)
+    cold_pos = torch.empty(n, dtype=torch.int64, device=loc.device)
+    counts = torch.empty(2, dtype=torch.int64, device=loc.device)
+    nbytes = _lib.query("hades_split_compact_workspace_bytes", n)
+    ws = (workspace or _ws(loc.device, "split")).get(nbytes)
+    _lib.call("hades_split_compact", _ptr(loc), n, _ptr(hot_mask), _ptr(hot_pos), _ptr(cold_pos),
+              _ptr(counts), _ptr(ws), ws.numel(), _stream())
+    return hot_mask, hot_pos, cold_pos, counts
+
+
+def split(loc, workspace=None):
+    """As split_padded, trimmed to size (one host synchronisation to read the two counts)."""
+    hot_mask, hot_pos, cold_pos, counts = split_padded(loc, workspace)
+    nh, nc = counts.tolist()
+    return hot_mask, hot_pos[:nh], cold_pos[:nc]
+
+
+def split3_padded(ids, class_table, workspace=None):
+    """Three-way split by the int8 class table (0 local, 1 remote-hot, 2 remote-cold) with the
+    compacted position lists; no host synchronisation.  Returns (masks[3], pos[3], counts[3])."""
+    from .EmbCacheLib import _SPLIT_ITYPE
+    _dev(ids, "ids"); _dev_or_pinned(class_table, "class_table")
+    _check(class_table.dtype == torch.int8, "class_table must be int8")
+    _check(ids.dtype in _SPLIT_ITYPE, "ids must be an integer tensor")
+    n = ids.numel()
+    masks = torch.empty((3, n), dtype=torch.bool, device=ids.device)
+    pos = torch.empty((3, n), dtype=torch.int64, device=ids.device)
+    counts = torch.empty(3, dtype=torch.int64, device=ids.device)
+    nbytes = _lib.query("hades_split_compact_workspace_bytes", n)
+    ws = (workspace or _ws(ids.device, "split")).get(nbytes)
+    _lib.call("hades_split3_compact", _ptr(ids), _SPLIT_ITYPE[ids.dtype], _ptr(class_table), n,
+              _ptr(masks[0]), _ptr(masks[1]), _ptr(masks[2]), _ptr(pos[0]), _ptr(pos[1]),
+              _ptr(pos[2]), _ptr(counts), _ptr(ws), ws.numel(), _stream())
+    return masks, pos, counts
+
+
+# ---- cached_fetch / cached_set ------------------------------------------------
+def _table_dim(*tables):
+    ref = next(t for t in tables if t is not None)
+    _check(ref.dim() in (1, 2), "tables must be 1-D or 2-D")
+    for t in tables:
+        if t is not None:
+            _check(t.dim() == ref.dim() and t.dtype == ref.dtype, "table shape/dtype mismatch")
+            _check(ref.dim() == 1 or t.size(1) == ref.size(1), "row widths differ")
+    return 1 if ref.dim() == 1 else ref.size(1)
+
+
+def cached_fetch(cold, hot, ids, sorted_hot, out=None, return_loc=False):
+    """out[i] = hot[slot] if ids[i] is in sorted_hot (slot = its rank there) else cold[ids[i]].
+
+    `cold` may be a device tensor or a pinned host tensor (read zero-copy).  The lookup runs
+    inside the gather kernel."""
+    _i64(ids, "ids"); _i64(sorted_hot, "sorted_hot")
+    _dev_or_pinned(cold, "cold"); _dev(hot, "hot")
+    dim = _table_dim(cold, hot)
+    n = ids.numel()
+    shape = (n,) if hot.dim() == 1 else (n, dim)
+    if out is None:
+        out = torch.empty(shape, dtype=hot.dtype, device=ids.device)
+    else:
+        _dev(out, "out")
+        _check(tuple(out.shape) == shape and out.dtype == hot.dtype, "out has the wrong shape/dtype")
+    loc = torch.empty_like(ids) if return_loc else None
+    _lib.call("hades_cached_fetch", _ptr(cold), _ptr(hot), _ptr(ids), n, _ptr(sorted_hot),
+              sorted_hot.numel(), _ptr(out), _opt(loc), dim, _dcode(hot), _stream())
+    return (out, loc) if return_loc else out
+
+
+def cached_fetch_loc(cold, hot, ids, loc, out=None):
+    """cached_fetch when the slots are already known (loc from `lookup`)."""
+    _i64(ids, "ids"); _i64(loc, "loc")
+    _dev_or_pinned(cold, "cold"); _dev(hot, "hot")
+    _check(loc.numel() == ids.numel(), "loc and ids differ in length")
+    dim = _table_dim(cold, hot)
+    n = ids.numel()
+    shape = (n,) if hot.dim() == 1 else (n, dim)
+    if out is None:
+        out = torch.empty(shape, dtype=hot.dtype, device=ids.device)
+    _lib.call("hades_cached_fetch_loc", _ptr(cold), _ptr(hot), _ptr(ids), _ptr(loc), n, _ptr(out),
+              dim, _dcode(hot), _stream())
+    return out
+
+
+def cached_set(src, cold, hot, ids, sorted_hot):
+    """(hot[slot] if ids[i] in sorted_hot else cold[ids[i]]) = src[i]; ids must be duplicate-free
+    for a defined result."""
+    _i64(ids, "ids"); _i64(sorted_hot, "sorted_hot")
+    _dev(src, "src"); _dev_or_pinned(cold, "cold"); _dev(hot, "hot")
+    dim = _table_dim(cold, hot, src)
+    _check(src.size(0) >= ids.numel(), "src has fewer rows than ids has entries")
+    _lib.call("hades_cached_set", _ptr(src), _ptr(cold), _ptr(hot), _ptr(ids), ids.numel(),
+              _ptr(sorted_hot), sorted_hot.numel(), dim, _dcode(hot), _stream())
+
+
+# ---- combine ------------------------------------------------------------------
+def combine_padded(idx, grad, id_bound=0, mode=COMBINE_FAST, return_inverse=False, workspace=None,
+                   out=None):
+    """Sort + dedup + segment-sum, no host synchronisation.
+
+    Returns (uids int64[n], sums float32[n, D], cnts int64[n], num_unique int64[1]) - and
+    inverse int32[n] when asked - of which the first num_unique[0] rows are live.
+    id_bound > 0 promises 0 <= idx < id_bound and shortens the sort.
+    """
+    _i64(idx, "idx"); _dev(grad, "grad")
+    _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
+    n, dim = idx.numel(), grad.size(1)
+    _check(grad.size(0) == n, "grad must have one row per id")
+    dev = idx.device
+    if out is None:
+        uids = torch.empty(n, dtype=torch.int64, device=dev)
+        sums = torch.empty((n, dim), dtype=torch.float32, device=dev)
+        cnts = torch.empty(n, dtype=torch.int64, device=dev)
+        num_unique = torch.empty(1, dtype=torch.int64, device=dev)
+    else:
+        uids, sums, cnts, num_unique = out
+    inverse = torch.empty(n, dtype=torch.int32, device=dev) if return_inverse else None
+    nbytes = _lib.query("hades_combine_workspace_bytes", n, dim)
+    ws = (workspace or _ws(dev, "combine")).get(nbytes)
+    _lib.call("hades_combine", _ptr(idx), _ptr(grad), n, dim, int(id_bound), int(mode), _ptr(uids),
+              _ptr(sums), _ptr(cnts), _ptr(num_unique), _opt(inverse), _ptr(ws), ws.numel(),
+              _stream())
+    if return_inverse:
+        return uids, sums, cnts, num_unique, inverse
+    return uids, sums, cnts, num_unique
+
+
+def combine(idx, grad, id_bound=0, mode=COMBINE_FAST, workspace=None):
+    """As combine_padded, trimmed to the number of distinct ids (one host synchronisation)."""
+    uids, sums, cnts, num_unique = combine_padded(idx, grad, id_bound, mode, workspace=workspace)
+    u = int(num_unique.item())
+    return uids[:u], sums[:u], cnts[:u]
+
+
+def rows_div_count_(sums, cnts, num_unique=None, one_plus=False):
+    """In place: sums[u] /= (cnts[u] + one_plus) for the live rows."""
+    _dev(sums, "sums"); _i64(cnts, "cnts")
+    _lib.call("hades_rows_div_count", _ptr(sums), _ptr(cnts), _opt(num_unique), sums.size(0),
+              sums.size(1), 1 if one_plus else 0, _stream())
+    return sums
+
+
+# ---- row optimizers -----------------------------------------------------------
+def adagrad_update_(uids, grad, hot_w, hot_s, cold_w, cold_s, sorted_hot, lr, eps,
+                    num_unique=None):
+    """Sparse Adagrad over the rows named by the duplicate-free `uids`, in place:
+    s += g*g;  w -= lr * g / (sqrt(s) + eps), each row in the hot tables if its id is in
+    sorted_hot, else in the cold tables (device or pinned host)."""
+    _i64(uids, "uids"); _dev(grad, "grad")
+    _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
+    dim = grad.size(1)
+    nh = 0 if sorted_hot is None else sorted_hot.numel()
+    for name, t in (("hot_w", hot_w), ("hot_s", hot_s)):
+        if t is not None:
+            _dev(t, name)
+            _check(t.dtype == torch.float32 and t.size(1) == dim, "%s: wrong dtype/width" % name)
+    for name, t in (("cold_w", cold_w), ("cold_s", cold_s)):
+        if t is not None:
+            _dev_or_pinned(t, name)
+            _check(t.dtype == torch.float32 and t.size(1) == dim, "%s: wrong dtype/width" % name)
+    _check(grad.size(0) >= uids.numel(), "grad has fewer rows than uids has entries")
+    _lib.call("hades_adagrad_update", _ptr(uids), _ptr(grad), _opt(num_unique), uids.numel(), dim,
+              _opt(sorted_hot), nh, _opt(hot_w), _opt(hot_s), _opt(cold_w), _opt(cold_s),
+              float(lr), float(eps), _stream())
+
+
+def adam_update_(uids, grad, hot, cold, sorted_hot, lr, beta1, beta2, eps, num_unique=None):
+    """SparseAdam row update in place.  `hot` and `cold` are (w, step, mem, power) tuples."""
+    _i64(uids, "uids"); _dev(grad, "grad")
+    dim = grad.size(1)
+    nh = 0 if sorted_hot is None else sorted_hot.numel()
+    hot = hot if hot is not None else (None, None, None, None)
+    _lib.call("hades_adam_update", _ptr(uids), _ptr(grad), _opt(num_unique), uids.numel(), dim,
+              _opt(sorted_hot), nh, _opt(hot[0]), _opt(hot[1]), _opt(hot[2]), _opt(hot[3]),
+              _opt(cold[0]), _opt(cold[1]), _opt(cold[2]), _opt(cold[3]),
+              float(lr), float(beta1), float(beta2), float(eps), _stream())
+
+
+# ---- cold-gradient accumulator ------------------------------------------------
+class ColdGradAccumulator:
+    """Open-addressing hash table in HBM: int64 id -> float32[dim] running sum and a count.
+
+    accumulate() adds a duplicate-free batch (combine it first); flush() returns every live entry
+    in ascending id order and empties the table.  The arithmetic is that of the reference's cache
+    server (python/EmbCache/server.py:546-562, 346-497) with a flush decided by the caller.
+    """
+
+    def __init__(self, num_slots, dim, id_bound=0, device="cuda"):
+        _check(num_slots > 0 and (num_slots & (num_slots - 1)) == 0, "num_slots must be a power of two")
+        self.num_slots, self.dim, self.id_bound = int(num_slots), int(dim), int(id_bound)
+        self.device = torch.device(device)
+        self.keys = torch.empty(num_slots, dtype=torch.int64, device=self.device)
+        self.accum = torch.empty((num_slots, dim), dtype=torch.float32, device=self.device)
+        self.cnt = torch.empty(num_slots, dtype=torch.int64, device=self.device)
+        self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self._ws = Workspace(self.device)
+        self.clear()
+
+    def clear(self):
+        _lib.call("hades_hash_clear", _ptr(self.keys), _ptr(self.accum), _ptr(self.cnt),
+                  self.num_slots, self.dim, _stream())
+
+    def accumulate(self, ids, grad, cnt=None, num_rows=None):
+        _i64(ids, "ids"); _dev(grad, "grad")
+        _check(grad.dtype == torch.float32 and grad.dim() == 2 and grad.size(1) == self.dim,
+               "grad must be float32 [rows, dim]")
+        _lib.call("hades_hash_accumulate", _ptr(self.keys), _ptr(self.accum), _ptr(self.cnt),
+                  self.num_slots, _ptr(ids), _ptr(grad), _opt(cnt), _opt(num_rows), ids.numel(),
+                  self.dim, _ptr(self.status), _stream())
+
+    def flush_padded(self, cap):
+        """Returns (ids int64[cap], sums float32[cap, dim], cnts int64[cap], num_out int64[1])."""
+        dev = self.device
+        out_ids = torch.empty(cap, dtype=torch.int64, device=dev)
+        out_sums = torch.empty((cap, self.dim), dtype=torch.float32, device=dev)
+        out_cnts = torch.empty(cap, dtype=torch.int64, device=dev)
+        num_out = torch.empty(1, dtype=torch.int64, device=dev)
+        nbytes = _lib.query("hades_hash_flush_workspace_bytes", self.num_slots, cap)
+        ws = self._ws.get(nbytes)
+        _lib.call("hades_hash_flush", _ptr(self.keys), _ptr(self.accum), _ptr(self.cnt),
+                  self.num_slots, self.dim, self.id_bound, _ptr(out_ids), _ptr(out_sums),
+                  _ptr(out_cnts), _ptr(num_out), cap, _ptr(self.status), _ptr(ws), ws.numel(),
+                  _stream())
+        return out_ids, out_sums, out_cnts, num_out
+
+    def flush(self, cap=None):
+        """Trimmed flush (one host synchronisation).  Raises if the table overflowed."""
+        cap = cap or self.num_slots
+        ids, sums, cnts, num_out = self.flush_padded(cap)
+        n = int(num_out.item())
+        st = int(self.status.item())
+        if st:
+            self.status.zero_()
+            raise RuntimeError("cold-gradient accumulator overflow (status %d): table full or "
+                               "flush capacity too small" % st)
+        return ids[:n], sums[:n], cnts[:n]

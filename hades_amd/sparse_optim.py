@@ -1,0 +1,110 @@
+"""Gradient combine and sparse row optimizers, host side.
+
+Mirrors the reference's python/EmbCache/sparse_optim.py for one GPU: `only_unique_grads` and
+`unique_grads` keep the reference's names, arguments and return values (:132-157); SparseAdagrad
+(the optimizer of the benchmark configurations) and SparseAdam (the one the reference ships,
+:531-685) run the whole update - lookup, state gather, row math, scatter-back - in one kernel over
+an EmbCache-style (hot, cold) table pair.  The cross-trainer all-to-all of the reference
+(:19-129, 267-341) is not part of this build.
+"""
+import torch
+
+from . import ops
+
+
+def only_unique_grads(idx, grad, id_bound=0, mode=ops.COMBINE_FAST):
+    """(unique ids ascending, per-id summed float32 grads, per-id counts) - python/EmbCache/sparse_optim.py:132-139."""
+    return ops.combine(idx, grad, id_bound=id_bound, mode=mode)
+
+
+def unique_grads(idx, grad, cnt=None, id_bound=0, mode=ops.COMBINE_FAST):
+    """(unique ids, per-id mean grads) - python/EmbCache/sparse_optim.py:142-157.
+
+    With `cnt` given, the divisor of row u is 1 + sum of the cnt entries of its occurrences: the
+    reference starts that count from ones (:145-148) and this keeps it."""
+    if cnt is None:
+        uids, sums, cnts, nu = ops.combine_padded(idx, grad, id_bound, mode)
+        ops.rows_div_count_(sums, cnts, nu)
+        u = int(nu.item())
+        return uids[:u], sums[:u]
+    uids, sums, _, nu, inverse = ops.combine_padded(idx, grad, id_bound, mode, return_inverse=True)
+    u = int(nu.item())
+    grad_cnt = torch.ones(u, dtype=cnt.dtype, device=cnt.device)
+    grad_cnt.index_add_(0, inverse.long(), cnt)
+    sums = sums[:u] / grad_cnt.unsqueeze(1)
+    return uids[:u], sums
+
+
+class _SparseRowOptimizer:
+    """State shared by the two optimizers: weights and state as (hot, cold) pairs keyed by the
+    ascending hot-ID set.  `weight_cold` is [N, D] on the device or pinned on the host."""
+
+    def __init__(self, weight_cold, hot_ids, lr, device="cuda"):
+        self.device = torch.device(device)
+        self.lr = lr
+        self.cold_w = weight_cold
+        self.num_rows, self.dim = weight_cold.shape
+        hot_ids = torch.as_tensor(hot_ids, dtype=torch.int64)
+        self.hot_ids = hot_ids.to(self.device)
+        self.hot_w = self._gather_hot(weight_cold)
+        self._ws = ops.Workspace(self.device)
+
+    def _gather_hot(self, cold):
+        if cold.is_cuda:
+            return cold[self.hot_ids].contiguous()
+        return cold[self.hot_ids.cpu()].to(self.device)
+
+    def _new_state_like(self, cold, shape=None):
+        shape = shape or tuple(cold.shape)
+        if cold.is_cuda:
+            return torch.zeros(shape, dtype=torch.float32, device=cold.device)
+        t = torch.empty(shape, dtype=torch.float32, pin_memory=True)
+        t.zero_()
+        return t
+
+    def fetch(self, ids, out=None):
+        """Forward fetch of embedding rows (cached_fetch)."""
+        return ops.cached_fetch(self.cold_w, self.hot_w, ids, self.hot_ids, out=out)
+
+    def step(self, idx, grad, mode=ops.COMBINE_FAST):
+        """combine the per-occurrence gradients, then update every distinct row once.
+        No host synchronisation."""
+        uids, sums, cnts, nu = ops.combine_padded(idx, grad, id_bound=self.num_rows, mode=mode,
+                                                  workspace=self._ws)
+        self.update(uids, sums, nu)
+        return uids, sums, cnts, nu
+
+
+class SparseAdagrad(_SparseRowOptimizer):
+    """s += g*g;  w -= lr * g / (sqrt(s) + eps) on the rows a step touches
+    (torch.optim.Adagrad with lr_decay = weight_decay = initial_accumulator_value = 0)."""
+
+    def __init__(self, weight_cold, hot_ids, lr=0.01, eps=1e-10, device="cuda"):
+        super().__init__(weight_cold, hot_ids, lr, device)
+        self.eps = eps
+        self.cold_s = self._new_state_like(weight_cold)
+        self.hot_s = torch.zeros_like(self.hot_w)
+
+    def update(self, uids, grad, num_unique=None):
+        ops.adagrad_update_(uids, grad, self.hot_w, self.hot_s, self.cold_w, self.cold_s,
+                            self.hot_ids, self.lr, self.eps, num_unique)
+
+
+class SparseAdam(_SparseRowOptimizer):
+    """The reference's SparseAdam.update (python/EmbCache/sparse_optim.py:590-685) as one kernel."""
+
+    def __init__(self, weight_cold, hot_ids, lr=0.01, betas=(0.9, 0.999), eps=1e-8, device="cuda"):
+        super().__init__(weight_cold, hot_ids, lr, device)
+        self.betas, self.eps = betas, eps
+        n, h = self.num_rows, self.hot_ids.numel()
+        self.cold_step = self._new_state_like(weight_cold, (n,))
+        self.cold_m = self._new_state_like(weight_cold)
+        self.cold_v = self._new_state_like(weight_cold)
+        self.hot_step = torch.zeros(h, dtype=torch.float32, device=self.device)
+        self.hot_m = torch.zeros_like(self.hot_w)
+        self.hot_v = torch.zeros_like(self.hot_w)
+
+    def update(self, uids, grad, num_unique=None):
+        ops.adam_update_(uids, grad, (self.hot_w, self.hot_step, self.hot_m, self.hot_v),
+                         (self.cold_w, self.cold_step, self.cold_m, self.cold_v), self.hot_ids,
+                         self.lr, self.betas[0], self.betas[1], self.eps, num_unique)

@@ -1,0 +1,256 @@
+/*
+ * hades_hip.h - C ABI of libhades_hip.so, the MI355X (gfx950) implementation of
+ * the HADES per-GPU embedding-cache hot path.
+ *
+ * Every entry point takes plain pointers, sizes and a HIP stream handle; no
+ * torch types cross this boundary.  The caller owns all memory.  Entry points
+ * return 0 on success and a non-zero code on failure; the message for the last
+ * failure on the calling thread is returned by hades_last_error().  Nothing in
+ * this library calls exit() or abort() (the reference's CUDA_CALL does:
+ * src/utils.h:12-24).
+ *
+ * Pointers named "cold"/"cpu" may address pinned host memory (allocated with
+ * hades_host_alloc / hipHostMalloc / torch pin_memory=True): kernels read and
+ * write it zero-copy over the host link.  All other pointers are device memory.
+ * Launches are asynchronous on `stream` (a hipStream_t passed as void*; NULL is
+ * the default stream).  Tensors are dense row-major.
+ *
+ * The first group mirrors, one for one, the functions the reference binds in
+ * src/pybind.cc:46-70 (declared in src/cuda/ops.h:9-41).  The second group are
+ * the fused operators of the same path (sorted-set lookup, split + compaction,
+ * combine, sparse Adagrad, cold-gradient accumulator).
+ */
+#ifndef HADES_HIP_H_
+#define HADES_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of row payloads (reference: FLOAT_TYPE_SWITCH, src/utils.h:26-37) */
+#define HADES_F32 0
+#define HADES_F64 1
+/* index type (reference: INTEGER_TYPE_SWITCH, src/utils.h:39-50) */
+#define HADES_I32 0
+#define HADES_I64 1
+/* extra id types accepted by hades_split only (reference: AT_DISPATCH_ALL_TYPES,
+ * src/cuda/split.cu:53-56; the floating-point cases of that dispatch are rejected) */
+#define HADES_I16 2
+#define HADES_I8 3
+#define HADES_U8 4
+
+/* status codes */
+#define HADES_OK 0
+#define HADES_ERR_ARG 1      /* bad argument (shape, dtype code, alignment, size) */
+#define HADES_ERR_HIP 2      /* a HIP runtime call or kernel launch failed */
+#define HADES_ERR_WORKSPACE 3 /* workspace too small */
+
+/* combine modes */
+#define HADES_COMBINE_FAST 0  /* fixed-shape tree sum: reproducible run to run, <=1e-5 rel. of exact */
+#define HADES_COMBINE_EXACT 1 /* strictly sequential sum in occurrence order: bit-equal to CPU index_add_ */
+
+const char* hades_last_error(void);
+int hades_version(void);
+
+/* ------------------------------------------------------------------------- */
+/* Group 1: one entry point per function bound in src/pybind.cc:46-70          */
+/* ------------------------------------------------------------------------- */
+
+/* cudaPinPtr / cudaPin: RegisterPtr, PinTensor (src/cuda/pin_memory.cu:9-22).
+ * Page-locks and maps an existing host allocation.  Returns HADES_ERR_HIP (and
+ * clears the HIP error state) where the platform refuses hipHostRegister. */
+int hades_pin(void* host_ptr, size_t bytes);
+/* cudaUnpinPtr / cudaUnpin: UnregisterPtr, UnpinTensor (src/cuda/pin_memory.cu:15-26) */
+int hades_unpin(void* host_ptr);
+/* Pinned, device-mapped host allocation for the cold table where registering
+ * existing memory is not possible.  The returned pointer is valid on host and device. */
+int hades_host_alloc(void** out_ptr, size_t bytes);
+int hades_host_free(void* ptr);
+
+/* cudaFetch: CUDAFetch (src/cuda/uva_fetch.cu:28-45)
+ *   dst[dst_index[i], :] = src[src_index[i], :]            for i in [0, n) */
+int hades_fetch(const void* src, const void* src_index, void* dst, const void* dst_index,
+                int64_t n, int64_t dim, int dtype, int itype, void* stream);
+
+/* cudaFetch2: CUDAFetch2 (src/cuda/uva_fetch.cu:72-105); dim == 1 is the 1-D form (:64-70)
+ *   dst[i, :] = src[src_index[i], :] */
+int hades_fetch2(const void* src, const void* src_index, void* dst,
+                 int64_t n, int64_t dim, int dtype, int itype, void* stream);
+
+/* cudaFetchWithCache2: CUDAFetchWithCache2 (src/cuda/uva_fetch.cu:108-192)
+ *   g = index_map[src_index[i]];  dst[i, :] = g != -1 ? gpu_src[g, :] : cpu_src[src_index[i], :] */
+int hades_fetch_with_cache2(const void* cpu_src, const void* gpu_src, const void* src_index,
+                            const void* index_map, void* dst,
+                            int64_t n, int64_t dim, int dtype, int itype, void* stream);
+
+/* cudaSet: CUDASet (src/cuda/uva_set.cu:11-68)
+ *   dst[dst_index[i], :] = src[i, :]      (duplicate indices: one writer wins, unspecified which) */
+int hades_set(const void* src, void* dst, const void* dst_index,
+              int64_t n, int64_t dim, int dtype, int itype, void* stream);
+
+/* cudaSetWithCache: CUDASetWithCache (src/cuda/uva_set.cu:71-153)
+ *   g = index_map[dst_index[i]];  (g != -1 ? gpu_dst[g, :] : cpu_dst[dst_index[i], :]) = src[i, :] */
+int hades_set_with_cache(const void* src, void* cpu_dst, void* gpu_dst, const void* dst_index,
+                         const void* index_map,
+                         int64_t n, int64_t dim, int dtype, int itype, void* stream);
+
+/* cudaCombine: CUDACombine (src/cuda/uva_fetch.cu:195-227) - a row scatter despite
+ * its name, identical to hades_set */
+int hades_combine_scatter(const void* src, void* dst, const void* dst_index,
+                          int64_t n, int64_t dim, int dtype, int itype, void* stream);
+
+/* cudaReminder: Reminder / ReminderKernel (src/cuda/binary_search.cu:36-43,76-87)
+ *   out[i] = in[i] % local_num_gpus   (C remainder: sign follows the dividend) */
+int hades_reminder(const void* in, int64_t local_num_gpus, void* out,
+                   int64_t n, int itype, void* stream);
+
+/* cudaBinarySearch: CUDABinarySearch / BinarySearchKernel (src/cuda/binary_search.cu:11-21,45-59)
+ *   out[i] = (upper_bound(range_partition, in[i]) - 1) * local_num_gpus + in[i] % local_num_gpus */
+int hades_binary_search(const void* in, const void* range_partition, int64_t num_part,
+                        int64_t local_num_gpus, void* out,
+                        int64_t n, int itype, void* stream);
+
+/* cudaBinarySearch2: CUDABinarySearch2 / BinarySearchKernel2 (src/cuda/binary_search.cu:24-33,61-74)
+ *   out[i] = upper_bound(range, in[i]) = number of entries of the ascending `range` that are <= in[i] */
+int hades_binary_search2(const void* in, const void* range, int64_t num_part, void* out,
+                         int64_t n, int itype, void* stream);
+
+/* cudaSplit: splitCUDA / _split (src/cuda/split.cu:13-56)
+ *   v = class_table[ids[i]];  local[i] = v==0; remote_hot[i] = v==1; remote_cold[i] = v==2
+ * The three masks are bool (1 byte) arrays of n entries, fully written (no prior zero-fill
+ * needed).  class_table (int8) may be device or pinned host memory (test/test_pin.py:24-29). */
+int hades_split(const void* ids, int id_type, const int8_t* class_table, int64_t n,
+                uint8_t* local_mask, uint8_t* remote_hot_mask, uint8_t* remote_cold_mask,
+                void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Group 2: fused operators of the same path                                  */
+/* ------------------------------------------------------------------------- */
+
+/* EmbCache lookup: membership + slot of each query in the ascending, duplicate-free hot-ID
+ * set.  Closed form over BinarySearchKernel2 (src/cuda/binary_search.cu:24-33):
+ *   pos = upper_bound(sorted_hot, q[i]);  loc[i] = (pos > 0 && sorted_hot[pos-1] == q[i]) ? pos-1 : -1
+ * Replaces the dense index_map probe (python/EmbCache/cache.py:163-171) and the CPU
+ * IndexCache round trip (python/EmbCache/dist_emb.py:184-185).  q, sorted_hot, loc: int64. */
+int hades_lookup_sorted(const int64_t* q, int64_t n, const int64_t* sorted_hot, int64_t num_hot,
+                        int64_t* loc, void* stream);
+
+/* Hot/cold split of a looked-up batch with stable compaction (replaces cudaSplit + torch.nonzero,
+ * python/EmbCache/dist_emb.py:174-191):  hot <=> loc[i] >= 0.
+ *   hot_mask[i]  = loc[i] >= 0                              (bool[n])
+ *   hot_pos      = ascending positions i with loc[i] >= 0   (int64, capacity n)
+ *   cold_pos     = ascending positions i with loc[i] <  0   (int64, capacity n)
+ *   counts[0..1] = {number hot, number cold}                (int64[2], device)
+ * workspace: device scratch of hades_split_compact_workspace_bytes(n) bytes. */
+size_t hades_split_compact_workspace_bytes(int64_t n);
+int hades_split_compact(const int64_t* loc, int64_t n, uint8_t* hot_mask, int64_t* hot_pos,
+                        int64_t* cold_pos, int64_t* counts, void* workspace, size_t workspace_bytes,
+                        void* stream);
+
+/* Three-way form of the same thing from the reference's class table (src/cuda/split.cu:11):
+ * masks as hades_split, plus pos[k] = ascending positions of class k (each int64 capacity n) and
+ * counts[0..2].  Any of the mask pointers may be NULL. */
+int hades_split3_compact(const void* ids, int id_type, const int8_t* class_table, int64_t n,
+                         uint8_t* mask0, uint8_t* mask1, uint8_t* mask2,
+                         int64_t* pos0, int64_t* pos1, int64_t* pos2, int64_t* counts,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* cached_fetch keyed by the sorted hot set: lookup fused into the gather
+ * (CUDAFetchWithCacheKernel2 semantics, src/cuda/uva_fetch.cu:108-130, with the
+ * index_map probe replaced by the binary search above).
+ *   loc = lookup(q[i]);  dst[i, :] = loc >= 0 ? hot_src[loc, :] : cold_src[q[i], :]
+ * loc_out (int64[n]) may be NULL.  cold_src may be device or pinned host memory. */
+int hades_cached_fetch(const void* cold_src, const void* hot_src, const int64_t* q, int64_t n,
+                       const int64_t* sorted_hot, int64_t num_hot, void* dst, int64_t* loc_out,
+                       int64_t dim, int dtype, void* stream);
+
+/* Same gather when the slots are already known (loc from hades_lookup_sorted). */
+int hades_cached_fetch_loc(const void* cold_src, const void* hot_src, const int64_t* q,
+                           const int64_t* loc, int64_t n, void* dst,
+                           int64_t dim, int dtype, void* stream);
+
+/* cached_set keyed by the sorted hot set (CUDASetWithCacheKernel semantics,
+ * src/cuda/uva_set.cu:71-93):
+ *   loc = lookup(q[i]);  (loc >= 0 ? hot_dst[loc, :] : cold_dst[q[i], :]) = src[i, :] */
+int hades_cached_set(const void* src, void* cold_dst, void* hot_dst, const int64_t* q, int64_t n,
+                     const int64_t* sorted_hot, int64_t num_hot,
+                     int64_t dim, int dtype, void* stream);
+
+/* combine: sort + dedup + segment-sum of duplicate-ID gradient rows; the arithmetic of
+ * only_unique_grads (python/EmbCache/sparse_optim.py:132-139), which is also the
+ * local-aggregation reduction (:310) over concatenated trainer batches.
+ *   uids  = ascending distinct values of idx                (int64, capacity n)
+ *   cnts  = occurrences of each                             (int64, capacity n)
+ *   sums  = per-id sum of grad rows, fp32                   (float, capacity n x dim)
+ *   num_unique[0] = U                                       (int64[1], device)
+ * Entries at and beyond U are left unspecified.  id_bound > 0 promises 0 <= idx[i] < id_bound
+ * (fewer sort passes); id_bound == 0 sorts all 64 bits as signed integers.
+ * mode: HADES_COMBINE_FAST or HADES_COMBINE_EXACT.  n must be < 2^30.
+ * Optional outputs (may be NULL): perm = occurrence positions in sorted order (int32[n]);
+ * inverse[i] = index of idx[i] in uids (int32[n]). */
+size_t hades_combine_workspace_bytes(int64_t n, int64_t dim);
+int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim, int64_t id_bound,
+                  int mode, int64_t* uids, float* sums, int64_t* cnts, int64_t* num_unique,
+                  int32_t* inverse, void* workspace, size_t workspace_bytes, void* stream);
+
+/* unique_grads (python/EmbCache/sparse_optim.py:142-157): in-place division of the first
+ * num_unique[0] rows of sums by cnts (plus `one_plus` added to the divisor: the reference starts
+ * the count from ones when a cnt vector is supplied, :145-148). */
+int hades_rows_div_count(float* sums, const int64_t* cnts, const int64_t* num_unique,
+                         int64_t max_rows, int64_t dim, int one_plus, void* stream);
+
+/* Sparse Adagrad row update with the lookup, the state/weight gather and the scatter-back fused
+ * (the reference ships SparseAdam only, python/EmbCache/sparse_optim.py:590-685; this is the same
+ * gather -> row math -> scatter skeleton, state via cache.py:66-131, for Adagrad):
+ *   for u < num_unique[0]:  id = uids[u]; g = grad[u, :]; loc = lookup(id)
+ *     (w, s) = loc >= 0 ? (hot_w[loc], hot_s[loc]) : (cold_w[id], cold_s[id])
+ *     s += g*g;  w -= lr * g / (sqrt(s) + eps)          (each operation rounded to fp32, no FMA)
+ * uids must be duplicate-free.  num_unique may be NULL (then all max_rows rows are live).
+ * sorted_hot may be NULL with num_hot == 0 (everything in the cold tables). */
+int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
+                         int64_t max_rows, int64_t dim,
+                         const int64_t* sorted_hot, int64_t num_hot,
+                         float* hot_w, float* hot_s, float* cold_w, float* cold_s,
+                         float lr, float eps, void* stream);
+
+/* SparseAdam row update, same fusion (python/EmbCache/sparse_optim.py:632-657,681):
+ *   step += 1; m = b1*m + (1-b1)*g; v = b2*v + (1-b2)*g*g
+ *   w -= lr * (m / (1 - b1^step)) / (sqrt(v / (1 - b2^step)) + eps)
+ * step: float[N] / float[H]; m, v, w: float[., dim]. */
+int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
+                      int64_t max_rows, int64_t dim,
+                      const int64_t* sorted_hot, int64_t num_hot,
+                      float* hot_w, float* hot_step, float* hot_m, float* hot_v,
+                      float* cold_w, float* cold_step, float* cold_m, float* cold_v,
+                      float lr, float beta1, float beta2, float eps, void* stream);
+
+/* Cold-gradient accumulator (delayed synchronisation): an open-addressing hash table in HBM,
+ * int64 key -> fp32[dim] running sum and an int64 count.  Restates on the GPU the arithmetic of
+ * EmbCacheServer._accumulate_gradients_cold_remote (python/EmbCache/server.py:546-562): per unique
+ * incoming id  buf[slot] += g; cnt[slot] += c; key[slot] = id.
+ * num_slots must be a power of two.  keys: int64[num_slots] (empty = -1), accum: float[num_slots,dim],
+ * cnt: int64[num_slots].  ids within one call must be duplicate-free (combine first).
+ * status[0] (int32, device) is set non-zero if the table is full. */
+int hades_hash_clear(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots, int64_t dim,
+                     void* stream);
+int hades_hash_accumulate(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots,
+                          const int64_t* ids, const float* grad, const int64_t* in_cnt,
+                          const int64_t* num_rows, int64_t max_rows, int64_t dim,
+                          int32_t* status, void* stream);
+/* Flush: emit every live slot as (id, sum row, count) in ascending id order, then clear the table
+ * (evident intent of python/EmbCache/server.py:413-419; see the note on :414 in the oracle).
+ *   out_ids int64[cap], out_sums float[cap, dim], out_cnts int64[cap], num_out int64[1] (device)
+ * cap bounds the number of live slots emitted (status[0] set non-zero if exceeded). */
+size_t hades_hash_flush_workspace_bytes(int64_t num_slots, int64_t cap);
+int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots, int64_t dim,
+                     int64_t id_bound, int64_t* out_ids, float* out_sums, int64_t* out_cnts,
+                     int64_t* num_out, int64_t cap, int32_t* status,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HADES_HIP_H_ */

@@ -1,0 +1,375 @@
+"""CPU restatement of the HADES embedding-cache hot path.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker, never the product: only tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py may import it.  Nothing under hades_amd/ imports it and nothing here
+touches a GPU.
+
+Every function restates one reference function and cites it.  Native (CUDA) functions of the
+reference are restated with numpy; the Python functions of the reference (only_unique_grads,
+unique_grads, SparseAdam.update) are restated with the same torch CPU calls the reference makes,
+next to an independent numpy restatement used to cross-check them.
+
+How each function is pinned (tests/test_oracle.py):
+  upper_bound / owner_rank / reminder : Python bisect and C remainder on random and edge inputs;
+                                        the split-size recipe of test/test_binarysearch2.py:13-27
+  lookup_sorted                       : brute-force membership on small inputs, edge cases
+  split_masks / split_compact         : the CPU split of test/test_split.py:30-37, mask invariants
+  fetch* / set*                       : the recipes of test/test_cached_fetch.py:22,43,
+                                        test/test_cached_set.py:22,26, test/test_fetch.py:16,
+                                        test/test_combine.py:16 (plain torch indexing, bit-exact),
+                                        independence from which rows are cached
+  combine                             : torch.unique + index_add_ (the reference's own calls) vs
+                                        the numpy stable-sort restatement vs float64 sums; closed
+                                        forms (all ids distinct, all ids equal), sum(cnt) == n
+  adagrad                             : torch.optim.Adagrad on the gathered rows; g == 0 leaves w
+                                        unchanged; first-step closed form
+  adam                                : torch.optim.Adam (same mathematics, different rounding) at
+                                        1e-6 relative; the reference has no test of its own
+  hash accumulator                    : a Python dict model; flush(accumulate(batches)) equals
+                                        combine(concat(batches))
+  hot placement                       : the reference's own argsort recipe, cache.py:165-171
+The C restatement of the native functions (hades_oracle.c) is checked against this module.
+"""
+import numpy as np
+import torch
+
+
+# ---------------------------------------------------------------------------
+# routing arithmetic: src/cuda/binary_search.cu
+# ---------------------------------------------------------------------------
+def upper_bound(sorted_range, values):
+    """cub::UpperBound as used by BinarySearchKernel2 (src/cuda/binary_search.cu:24-33):
+    number of entries of the ascending range that are <= value.  Output dtype = input dtype (:64)."""
+    sorted_range = np.asarray(sorted_range)
+    values = np.asarray(values)
+    return np.searchsorted(sorted_range, values, side="right").astype(values.dtype)
+
+
+def c_remainder(values, m):
+    """C `%` (sign follows the dividend), what ReminderKernel computes (src/cuda/binary_search.cu:36-43)."""
+    values = np.asarray(values)
+    return np.fmod(values, values.dtype.type(m)).astype(values.dtype)
+
+
+def owner_rank(values, range_partition, local_num_gpus):
+    """BinarySearchKernel (src/cuda/binary_search.cu:11-21):
+    (UpperBound(range_partition, v) - 1) * local_num_gpus + v % local_num_gpus."""
+    values = np.asarray(values)
+    rank = np.searchsorted(np.asarray(range_partition), values, side="right").astype(np.int64)
+    out = (rank - 1) * int(local_num_gpus) + c_remainder(values, local_num_gpus).astype(np.int64)
+    return out.astype(values.dtype)
+
+
+def split_sizes(sorted_owner, num_owners):
+    """The split-size recipe of swap_gradients (python/EmbCache/sparse_optim.py:50-54) and
+    test/test_binarysearch2.py:23-27: cudaBinarySearch2(arange(P), sorted owners), then adjacent
+    differences."""
+    ub = upper_bound(sorted_owner, np.arange(num_owners, dtype=np.asarray(sorted_owner).dtype))
+    ub = ub.astype(np.int64)
+    ub[1:] = ub[1:] - ub[:-1]
+    return ub
+
+
+# ---------------------------------------------------------------------------
+# lookup against the sorted hot set (closed form over BinarySearchKernel2)
+# ---------------------------------------------------------------------------
+def lookup_sorted(q, sorted_hot):
+    """loc = slot of q in the ascending duplicate-free hot set, or -1.  Built on the reference's
+    UpperBound (src/cuda/binary_search.cu:24-33); replaces index_map[q] of
+    python/EmbCache/cache.py:163-171 (there: -1 for uncached, arange slot otherwise)."""
+    q = np.asarray(q, dtype=np.int64)
+    sorted_hot = np.asarray(sorted_hot, dtype=np.int64)
+    pos = np.searchsorted(sorted_hot, q, side="right")
+    loc = np.full(q.shape, -1, dtype=np.int64)
+    if sorted_hot.size:
+        prev = sorted_hot[np.maximum(pos - 1, 0)]
+        hit = (pos > 0) & (prev == q)
+        loc[hit] = pos[hit] - 1
+    return loc
+
+
+def dense_index_map(num_rows, cached_ids, dtype=np.int64):
+    """idx_map of python/EmbCache/cache.py:163,170: -1 everywhere, slot number at cached ids."""
+    m = np.full(num_rows, -1, dtype=dtype)
+    m[np.asarray(cached_ids)] = np.arange(len(cached_ids), dtype=dtype)
+    return m
+
+
+def select_hot_ids(hotness, num_hot, candidate_ids=None):
+    """Placement of python/EmbCache/cache.py:165-168: argsort(hotness, descending)[:cached_num].
+    Returned ascending.  (Ties are broken however torch.argsort breaks them, as in the reference.)"""
+    hotness = torch.as_tensor(hotness)
+    if candidate_ids is None:
+        candidate_ids = torch.arange(hotness.numel(), dtype=torch.int64)
+    order = torch.argsort(hotness[candidate_ids], descending=True)
+    return np.sort(candidate_ids[order][:num_hot].numpy().astype(np.int64))
+
+
+# ---------------------------------------------------------------------------
+# split: src/cuda/split.cu
+# ---------------------------------------------------------------------------
+def split_masks(ids, class_table):
+    """_split (src/cuda/split.cu:13-51): three bool masks, mask_k[i] = class_table[ids[i]] == k
+    (0 local, 1 remote-hot, 2 remote-cold, :11); other table values set no mask."""
+    v = np.asarray(class_table)[np.asarray(ids).astype(np.int64)]
+    return v == 0, v == 1, v == 2
+
+
+def split_compact(loc):
+    """hot <=> loc >= 0; compaction as the reference does it with torch.nonzero
+    (python/EmbCache/dist_emb.py:179-180): ascending positions of each class."""
+    loc = np.asarray(loc)
+    hot = loc >= 0
+    return hot, np.nonzero(hot)[0].astype(np.int64), np.nonzero(~hot)[0].astype(np.int64)
+
+
+def split3_compact(ids, class_table):
+    masks = split_masks(ids, class_table)
+    return masks, tuple(np.nonzero(m)[0].astype(np.int64) for m in masks)
+
+
+# ---------------------------------------------------------------------------
+# row gather / scatter: src/cuda/uva_fetch.cu, src/cuda/uva_set.cu
+# ---------------------------------------------------------------------------
+def fetch(src, src_index, dst, dst_index):
+    """UVAFetchKernel (src/cuda/uva_fetch.cu:11-26): dst[dst_index[i]] = src[src_index[i]], in place."""
+    dst[np.asarray(dst_index).astype(np.int64)] = src[np.asarray(src_index).astype(np.int64)]
+    return dst
+
+
+def fetch2(src, src_index):
+    """UVAFetchKernel2 / UVAFetch1DKernel2 (src/cuda/uva_fetch.cu:48-70): dst[i] = src[src_index[i]]."""
+    return np.asarray(src)[np.asarray(src_index).astype(np.int64)].copy()
+
+
+def fetch_with_cache2(cpu_src, gpu_src, src_index, index_map):
+    """CUDAFetchWithCacheKernel2 (src/cuda/uva_fetch.cu:108-130):
+    g = index_map[idx]; dst[i] = gpu_src[g] if g != -1 else cpu_src[idx]."""
+    idx = np.asarray(src_index).astype(np.int64)
+    g = np.asarray(index_map)[idx].astype(np.int64)
+    out = np.asarray(cpu_src)[idx].copy()
+    hit = g != -1
+    out[hit] = np.asarray(gpu_src)[g[hit]]
+    return out
+
+
+def set_rows(src, dst, dst_index):
+    """UVASetKernel / UVACombineKernel (src/cuda/uva_set.cu:11-24, src/cuda/uva_fetch.cu:195-210):
+    dst[dst_index[i]] = src[i], in place (indices unique in every caller)."""
+    di = np.asarray(dst_index).astype(np.int64)
+    dst[di] = np.asarray(src)[: di.size]
+    return dst
+
+
+def set_with_cache(src, cpu_dst, gpu_dst, dst_index, index_map):
+    """CUDASetWithCacheKernel (src/cuda/uva_set.cu:71-93): the row goes to gpu_dst[g] when
+    g = index_map[idx] != -1, else to cpu_dst[idx].  In place on both."""
+    idx = np.asarray(dst_index).astype(np.int64)
+    g = np.asarray(index_map)[idx].astype(np.int64)
+    hit = g != -1
+    src = np.asarray(src)[: idx.size]
+    gpu_dst[g[hit]] = src[hit]
+    cpu_dst[idx[~hit]] = src[~hit]
+    return cpu_dst, gpu_dst
+
+
+def cached_fetch(cold, hot, q, sorted_hot):
+    """cached_fetch keyed by the sorted hot set = fetch_with_cache2 with index_map replaced by the
+    binary search (same select: src/cuda/uva_fetch.cu:118-128)."""
+    q = np.asarray(q, dtype=np.int64)
+    loc = lookup_sorted(q, sorted_hot)
+    out = np.asarray(cold)[q].copy()
+    hit = loc >= 0
+    out[hit] = np.asarray(hot)[loc[hit]]
+    return out
+
+
+def cached_set(src, cold, hot, q, sorted_hot):
+    q = np.asarray(q, dtype=np.int64)
+    loc = lookup_sorted(q, sorted_hot)
+    hit = loc >= 0
+    src = np.asarray(src)[: q.size]
+    hot[loc[hit]] = src[hit]
+    cold[q[~hit]] = src[~hit]
+    return cold, hot
+
+
+# ---------------------------------------------------------------------------
+# combine: python/EmbCache/sparse_optim.py:132-157
+# ---------------------------------------------------------------------------
+def only_unique_grads(idx, grad):
+    """The reference's code verbatim in behaviour (python/EmbCache/sparse_optim.py:132-139):
+    torch.unique(return_inverse, return_counts) then zeros(float32).index_add_.  torch CPU tensors
+    in, torch CPU tensors out."""
+    idx = torch.as_tensor(idx)
+    grad = torch.as_tensor(grad)
+    grad_indices, inverse, grad_cnt = torch.unique(idx, return_inverse=True, return_counts=True)
+    grad_values = torch.zeros((grad_indices.shape[0], grad.shape[1]))
+    grad_values.index_add_(0, inverse, grad)
+    return grad_indices, grad_values, grad_cnt
+
+
+def unique_grads(idx, grad, cnt=None):
+    """python/EmbCache/sparse_optim.py:142-157, including the count that starts from ones when a
+    cnt vector is given (:145-148)."""
+    idx = torch.as_tensor(idx)
+    grad = torch.as_tensor(grad)
+    if cnt is not None:
+        cnt = torch.as_tensor(cnt)
+        grad_indices, inverse = torch.unique(idx, return_inverse=True)
+        grad_cnt = torch.ones((grad_indices.shape[0],), dtype=cnt.dtype)
+        grad_cnt.index_add_(0, inverse, cnt)
+    else:
+        grad_indices, inverse, grad_cnt = torch.unique(idx, return_inverse=True, return_counts=True)
+    grad_values = torch.zeros((grad_indices.shape[0], grad.shape[1]))
+    grad_values.index_add_(0, inverse, grad)
+    grad_values = grad_values / grad_cnt.unsqueeze(1)
+    return grad_indices, grad_values
+
+
+def combine_sequential(idx, grad):
+    """Independent numpy restatement of only_unique_grads: stable sort by id, then a strictly
+    sequential float32 sum ((0 + g1) + g2) + ... of each id's rows in occurrence order - the order
+    CPU index_add_ adds them in.  Used to cross-check the torch form and as the bit-exact target of
+    the deterministic-order mode."""
+    idx = np.asarray(idx, dtype=np.int64)
+    grad = np.asarray(grad, dtype=np.float32)
+    order = np.argsort(idx, kind="stable")
+    sidx = idx[order]
+    if sidx.size == 0:
+        return (np.zeros(0, np.int64), np.zeros((0, grad.shape[1]), np.float32), np.zeros(0, np.int64))
+    starts = np.nonzero(np.concatenate(([True], sidx[1:] != sidx[:-1])))[0]
+    ends = np.concatenate((starts[1:], [sidx.size]))
+    uids = sidx[starts]
+    cnts = (ends - starts).astype(np.int64)
+    sums = np.zeros((uids.size, grad.shape[1]), dtype=np.float32)
+    # add the k-th occurrence of every id that has one, k = 0, 1, 2, ...: each row of `sums`
+    # still receives its rows one at a time in occurrence order
+    live = np.arange(uids.size)
+    k = 0
+    while live.size:
+        sums[live] = sums[live] + grad[order[starts[live] + k]]
+        k += 1
+        live = live[cnts[live] > k]
+    return uids, sums, cnts
+
+
+def combine_float64(idx, grad):
+    """Reference sums in float64 (for the tolerance mode)."""
+    idx = np.asarray(idx, dtype=np.int64)
+    uids, inverse, cnts = np.unique(idx, return_inverse=True, return_counts=True)
+    sums = np.zeros((uids.size, np.asarray(grad).shape[1]), dtype=np.float64)
+    np.add.at(sums, inverse, np.asarray(grad, dtype=np.float64))
+    return uids, sums, cnts.astype(np.int64)
+
+
+# ---------------------------------------------------------------------------
+# row optimizers
+# ---------------------------------------------------------------------------
+def adagrad_rows(w, s, g, lr, eps):
+    """Sparse Adagrad on gathered rows, float32, one rounding per operation, in torch's order
+    (torch.optim.Adagrad: state_sum.addcmul_(g, g); std = state_sum.sqrt().add_(eps);
+    param.addcdiv_(g, std, value=-lr)).  The reference has no Adagrad (its optimizer is SparseAdam,
+    python/EmbCache/sparse_optim.py:531); this is the optimizer the benchmark configurations name.
+    Returns (w_new, s_new)."""
+    w = np.asarray(w, dtype=np.float32)
+    s = np.asarray(s, dtype=np.float32)
+    g = np.asarray(g, dtype=np.float32)
+    lr = np.float32(lr)
+    eps = np.float32(eps)
+    s1 = (s + g * g).astype(np.float32)
+    std = (np.sqrt(s1) + eps).astype(np.float32)
+    w1 = (w - (lr * g) / std).astype(np.float32)
+    return w1, s1
+
+
+def sparse_adagrad_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, uids, g, lr, eps):
+    """Gather (cached_fetch), adagrad_rows, scatter back (cached_set); in place."""
+    w = cached_fetch(cold_w, hot_w, uids, sorted_hot)
+    s = cached_fetch(cold_s, hot_s, uids, sorted_hot)
+    w1, s1 = adagrad_rows(w, s, g, lr, eps)
+    cached_set(w1, cold_w, hot_w, uids, sorted_hot)
+    cached_set(s1, cold_s, hot_s, uids, sorted_hot)
+
+
+def adam_rows(w, step, m, v, g, lr, beta1, beta2, eps):
+    """SparseAdam.update arithmetic (python/EmbCache/sparse_optim.py:632-657,681) on gathered rows,
+    with torch CPU float32 ops in the reference's order.  Returns (w, step, m, v) new."""
+    w, step, m, v, g = (torch.as_tensor(np.asarray(x, dtype=np.float32)) for x in (w, step, m, v, g))
+    state_step = step + 1                                                  # :634
+    grad_power = g * g                                                     # :640
+    update_mem = beta1 * m + (1.0 - beta1) * g                             # :641
+    update_power = beta2 * v + (1.0 - beta2) * grad_power                  # :642
+    update_mem_corr = update_mem / (1.0 - torch.pow(torch.tensor(beta1), state_step)).unsqueeze(1)    # :652
+    update_power_corr = update_power / (1.0 - torch.pow(torch.tensor(beta2), state_step)).unsqueeze(1)  # :654
+    std_values = lr * update_mem_corr / (torch.sqrt(update_power_corr) + eps)                           # :656
+    w_new = w - std_values                                                 # :681
+    return w_new.numpy(), state_step.numpy(), update_mem.numpy(), update_power.numpy()
+
+
+# ---------------------------------------------------------------------------
+# cold-gradient accumulator: python/EmbCache/server.py:546-562 (accumulate), :346-419 (flush)
+# ---------------------------------------------------------------------------
+class ColdGradAccumulatorModel:
+    """Dict model: per unique incoming id  buf[id] += g; cnt[id] += c  (server.py:556-559); flush
+    emits every entry with cnt > 0 in ascending id order and resets it (:413-419; the gradient row
+    is zeroed too - the reference's `buf[idx][:] = 0` at :414 writes to a temporary copy and is a
+    no-op there, the evident intent is what is modelled)."""
+
+    def __init__(self, dim):
+        self.dim = dim
+        self.rows = {}
+        self.cnt = {}
+
+    def accumulate(self, ids, grad, cnt=None):
+        ids = np.asarray(ids, dtype=np.int64)
+        grad = np.asarray(grad, dtype=np.float32)
+        for i, k in enumerate(ids.tolist()):
+            c = 1 if cnt is None else int(cnt[i])
+            if k in self.rows:
+                self.rows[k] = (self.rows[k] + grad[i]).astype(np.float32)
+                self.cnt[k] += c
+            else:
+                self.rows[k] = (np.zeros(self.dim, np.float32) + grad[i]).astype(np.float32)
+                self.cnt[k] = c
+
+    def flush(self):
+        keys = sorted(self.rows)
+        ids = np.array(keys, dtype=np.int64)
+        sums = np.stack([self.rows[k] for k in keys]) if keys else np.zeros((0, self.dim), np.float32)
+        cnts = np.array([self.cnt[k] for k in keys], dtype=np.int64)
+        self.rows, self.cnt = {}, {}
+        return ids, sums, cnts
+
+
+# ---------------------------------------------------------------------------
+# the whole step, for smoke tests and the CPU baseline (torch CPU, as the reference's CPU path)
+# ---------------------------------------------------------------------------
+def torch_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps):
+    """lookup -> cached_fetch -> combine -> sparse Adagrad with torch CPU ops on torch CPU tensors,
+    in place on the four tables.  Returns (fetched rows, uids, sums, cnts).  This is the shape the
+    reference's CPU-side code has: searchsorted for the lookup, indexed reads, torch.unique +
+    index_add_ for the combine (python/EmbCache/sparse_optim.py:132-139), element-wise update."""
+    def lookup(ids):
+        pos = torch.searchsorted(sorted_hot, ids, right=True)
+        prev = sorted_hot[(pos - 1).clamp_(min=0)]
+        return torch.where((pos > 0) & (prev == ids), pos - 1, torch.full_like(pos, -1))
+
+    loc = lookup(q)
+    hit = loc >= 0
+    rows = torch.empty((q.numel(), cold_w.shape[1]), dtype=cold_w.dtype)
+    rows[hit] = hot_w[loc[hit]]
+    rows[~hit] = cold_w[q[~hit]]
+
+    uids, sums, cnts = only_unique_grads(q, grad)
+
+    uloc = lookup(uids)
+    uh = uloc >= 0
+    for (w_tab, s_tab, sel, index) in ((hot_w, hot_s, uh, uloc[uh]), (cold_w, cold_s, ~uh, uids[~uh])):
+        g = sums[sel]
+        s = s_tab[index].addcmul_(g, g, value=1.0)
+        std = s.sqrt().add_(eps)
+        w = w_tab[index].addcdiv_(g, std, value=-lr)
+        s_tab[index] = s
+        w_tab[index] = w
+    return rows, uids, sums, cnts

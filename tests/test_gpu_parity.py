@@ -1,0 +1,488 @@
+"""GPU parity: every operator of the C-ABI library against the CPU oracle on the same seeded
+inputs.  Integer, index and payload results must be bit-exact; float32 sums and updates are
+bit-exact in the deterministic modes and within the stated tolerance otherwise."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hades_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib(cuda_device):
+    import hades_amd.EmbCacheLib as E
+    from hades_amd import ops
+    return E, ops
+
+
+def dev(a, device="cuda"):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def zipfish(rng, n, n_ids):
+    return np.minimum((rng.pareto(0.9, n)).astype(np.int64), n_ids - 1)
+
+
+NP_F = {torch.float32: np.float32, torch.float64: np.float64}
+NP_I = {torch.int32: np.int32, torch.int64: np.int64}
+
+
+# ---- cudaFetch* / cudaSet* / cudaCombine: the reference's test recipes --------------------
+@pytest.mark.parametrize("dim", [1, 3, 7, 64, 100, 128, 260])
+@pytest.mark.parametrize("fdt,idt", [(torch.float32, torch.int64), (torch.float64, torch.int32)])
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_fetch_and_set_with_cache(lib, dim, fdt, idt, host_cold):
+    E, _ = lib
+    rng = np.random.default_rng(100 + dim)
+    n_rows, n_cached, n_q = 5000, 2000, 1537
+    shape = (n_rows,) if dim == 1 else (n_rows, dim)
+    src = rng.standard_normal(shape).astype(NP_F[fdt])
+    cached_idx = rng.permutation(n_rows)[:n_cached]
+    idx_map = O.dense_index_map(n_rows, cached_idx, NP_I[idt])
+    gpu_src_np = src[cached_idx].copy()
+    q = rng.permutation(n_rows)[:n_q].astype(NP_I[idt])
+
+    if host_cold:
+        cpu_src = torch.empty(shape, dtype=fdt, pin_memory=True)
+        cpu_src.copy_(torch.from_numpy(src))
+        E.cudaPin(cpu_src)          # already page-locked: a no-op, as for the reference after pinning
+    else:
+        cpu_src = dev(src)
+    gpu_src, d_map, d_q = dev(gpu_src_np), dev(idx_map), dev(q)
+    dst = torch.zeros((n_q,) + shape[1:], dtype=fdt, device="cuda")
+
+    # test/test_cached_fetch.py:52-60 / :66-74 (and _1D)
+    E.cudaFetchWithCache2(cpu_src, gpu_src, d_q, d_map, dst)
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.cpu().numpy(), O.fetch_with_cache2(src, gpu_src_np, q, idx_map))
+    assert np.array_equal(dst.cpu().numpy(), src[q])
+    dst.zero_()
+    E.cudaFetch2(cpu_src, d_q, dst)
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.cpu().numpy(), O.fetch2(src, q))
+
+    # test/test_cached_set.py:50-58 / :64-72
+    rows = rng.standard_normal((n_q,) + shape[1:]).astype(NP_F[fdt])
+    want_cpu, want_gpu = src.copy(), gpu_src_np.copy()
+    O.set_with_cache(rows, want_cpu, want_gpu, q, idx_map)
+    E.cudaSetWithCache(dev(rows), cpu_src, gpu_src, d_q, d_map)
+    torch.cuda.synchronize()
+    assert np.array_equal(cpu_src.cpu().numpy(), want_cpu)
+    assert np.array_equal(gpu_src.cpu().numpy(), want_gpu)
+    want = want_cpu.copy()
+    O.set_rows(rows, want, q)
+    E.cudaSet(dev(rows), cpu_src, d_q)
+    torch.cuda.synchronize()
+    assert np.array_equal(cpu_src.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("dim", [4, 128, 33])
+def test_fetch_dst_indexed_and_combine_scatter(lib, dim):
+    E, _ = lib
+    rng = np.random.default_rng(200 + dim)
+    src = rng.standard_normal((4000, dim)).astype(np.float32)
+    dst = rng.standard_normal((900, dim)).astype(np.float32)
+    si = rng.permutation(4000)[:700].astype(np.int64)
+    di = rng.permutation(900)[:700].astype(np.int64)
+    d_dst = dev(dst)
+    E.cudaFetch(dev(src), dev(si), d_dst, dev(di))                 # test/test_fetch.py:31
+    torch.cuda.synchronize()
+    assert np.array_equal(d_dst.cpu().numpy(), O.fetch(src, si, dst.copy(), di))
+    big = np.zeros((4000, dim), np.float32)
+    d_big = dev(big)
+    rows = rng.standard_normal((700, dim)).astype(np.float32)
+    E.cudaCombine(dev(rows), d_big, dev(si))                        # test/test_combine.py:33
+    torch.cuda.synchronize()
+    assert np.array_equal(d_big.cpu().numpy(), O.set_rows(rows, big.copy(), si))
+
+
+def test_mover_unaligned_views_and_empty(lib):
+    E, _ = lib
+    rng = np.random.default_rng(3)
+    base = torch.from_numpy(rng.standard_normal(4 * 1000 + 1).astype(np.float32)).cuda()
+    src = base[1:].view(1000, 4)            # 4-byte aligned only: takes the narrow copy path
+    assert src.data_ptr() % 16 != 0
+    q = rng.integers(0, 1000, 333).astype(np.int64)
+    dst = torch.empty((333, 4), device="cuda")
+    E.cudaFetch2(src, dev(q), dst)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.cpu(), src.cpu()[torch.from_numpy(q)])
+    empty = torch.empty(0, dtype=torch.int64, device="cuda")
+    E.cudaFetch2(src, empty, torch.empty((0, 4), device="cuda"))
+    E.cudaSet(torch.empty((0, 4), device="cuda"), src, empty)
+    torch.cuda.synchronize()
+
+
+def test_shim_rejects_bad_arguments(lib):
+    E, _ = lib
+    a = torch.zeros((10, 4), device="cuda")
+    i = torch.zeros(3, dtype=torch.int64, device="cuda")
+    with pytest.raises(RuntimeError):
+        E.cudaFetch(a, i, torch.zeros((10, 5), device="cuda"), i)       # CHECK(src.size(1) == dst.size(1))
+    with pytest.raises(RuntimeError):
+        E.cudaFetch(a, i, a, torch.zeros(4, dtype=torch.int64, device="cuda"))
+    with pytest.raises(RuntimeError):
+        E.cudaFetch2(a.half(), i, a.half())                              # float or double only
+    with pytest.raises(RuntimeError):
+        E.cudaFetch2(a, i.to(torch.int16), a)                            # int32 or int64 only
+    with pytest.raises(RuntimeError):
+        E.cudaFetch2(torch.zeros((10, 4)), i, a)                         # pageable host memory
+    with pytest.raises(RuntimeError):
+        E.cudaFetch2(a.t(), i, a)                                        # not contiguous
+
+
+# ---- routing ----------------------------------------------------------------------------
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+def test_routing_ops(lib, idt):
+    E, _ = lib
+    rng = np.random.default_rng(4)
+    v = rng.integers(0, 3_000_000, 10_001).astype(NP_I[idt])
+    rp = np.array([0, 1_500_000, 3_000_000], NP_I[idt])
+    assert np.array_equal(E.cudaReminder(dev(v), 4).cpu().numpy(), O.c_remainder(v, 4))
+    owner = E.cudaBinarySearch(dev(v), dev(rp), 4)
+    assert owner.dtype == idt
+    assert np.array_equal(owner.cpu().numpy(), O.owner_rank(v, rp, 4))
+    # split sizes (test/test_binarysearch2.py:19-27, python/EmbCache/sparse_optim.py:43-54)
+    value, _ = torch.sort(owner)
+    ranges = torch.arange(8, device="cuda", dtype=idt)
+    splits = E.cudaBinarySearch2(ranges, value)
+    assert np.array_equal(splits.cpu().numpy(), O.upper_bound(np.sort(O.owner_rank(v, rp, 4)), np.arange(8, dtype=NP_I[idt])))
+    splits[1:] = splits[1:] - splits[:-1].clone()
+    assert np.array_equal(splits.cpu().numpy().astype(np.int64), O.split_sizes(np.sort(O.owner_rank(v, rp, 4)), 8))
+    # negative values: C remainder
+    neg = np.array([-7, 7, -1, 0], NP_I[idt])
+    assert np.array_equal(E.cudaReminder(dev(neg), 4).cpu().numpy(), O.c_remainder(neg, 4))
+    # empty range / empty input
+    assert E.cudaBinarySearch2(dev(v), torch.empty(0, dtype=idt, device="cuda")).sum().item() == 0
+    assert E.cudaReminder(torch.empty(0, dtype=idt, device="cuda"), 4).numel() == 0
+
+
+# ---- lookup / split -----------------------------------------------------------------------
+@pytest.mark.parametrize("n,h", [(0, 10), (1, 1), (1000, 0), (4097, 511), (200_000, 48_000)])
+def test_lookup_sorted(lib, n, h):
+    _, ops = lib
+    rng = np.random.default_rng(5 + n)
+    n_rows = max(4 * h, 100)
+    hot = np.sort(rng.choice(n_rows, h, replace=False)).astype(np.int64)
+    q = rng.integers(-3, n_rows + 3, n).astype(np.int64)
+    if n > 4 and h > 0:
+        q[:4] = [hot[0], hot[-1], hot[0] - 1, hot[-1] + 1]
+    loc = ops.lookup(dev(q), dev(hot))
+    assert np.array_equal(loc.cpu().numpy(), O.lookup_sorted(q, hot))
+
+
+@pytest.mark.parametrize("n", [0, 1, 7, 2048, 2049, 100_003])
+def test_split_compact(lib, n):
+    _, ops = lib
+    rng = np.random.default_rng(6 + n)
+    loc = np.where(rng.random(n) < 0.9, rng.integers(0, 1000, n), -1).astype(np.int64)
+    hot_mask, hot_pos, cold_pos = ops.split(dev(loc))
+    w_mask, w_hot, w_cold = O.split_compact(loc)
+    assert hot_mask.dtype == torch.bool
+    assert np.array_equal(hot_mask.cpu().numpy(), w_mask)
+    assert np.array_equal(hot_pos.cpu().numpy(), w_hot)
+    assert np.array_equal(cold_pos.cpu().numpy(), w_cold)
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32, torch.int16])
+@pytest.mark.parametrize("pinned_table", [False, True])
+def test_cuda_split_and_split3(lib, idt, pinned_table):
+    E, ops = lib
+    rng = np.random.default_rng(7)
+    n_nodes = 30_000
+    table = rng.integers(0, 4, n_nodes).astype(np.int8)       # value 3 belongs to no class
+    ids = rng.integers(0, n_nodes, 50_001).astype(np.int64)
+    t_ids = torch.from_numpy(ids).to(idt).cuda()
+    if pinned_table:                                          # test/test_pin.py:24-29
+        t_table = torch.empty(n_nodes, dtype=torch.int8, pin_memory=True)
+        t_table.copy_(torch.from_numpy(table))
+    else:
+        t_table = dev(table)
+    want = O.split_masks(ids, table)
+    got = E.cudaSplit(t_ids, t_table)
+    assert len(got) == 3 and all(g.dtype == torch.bool for g in got)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+    masks, pos, counts = ops.split3_padded(t_ids, t_table)
+    counts = counts.tolist()
+    w_masks, w_pos = O.split3_compact(ids, table)
+    for k in range(3):
+        assert np.array_equal(masks[k].cpu().numpy(), w_masks[k])
+        assert counts[k] == w_pos[k].size
+        assert np.array_equal(pos[k][:counts[k]].cpu().numpy(), w_pos[k])
+
+
+# ---- cached_fetch / cached_set by the sorted hot set -----------------------------------------
+@pytest.mark.parametrize("dim", [1, 64, 128, 100])
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_cached_fetch_and_set_sorted(lib, dim, host_cold):
+    _, ops = lib
+    rng = np.random.default_rng(8 + dim)
+    n_rows, h, n = 20_000, 3000, 7001
+    shape = (n_rows,) if dim == 1 else (n_rows, dim)
+    cold = rng.standard_normal(shape).astype(np.float32)
+    hot_ids = np.sort(rng.choice(n_rows, h, replace=False)).astype(np.int64)
+    hot = (cold[hot_ids] + 1.0).astype(np.float32)      # distinguishable from the cold copy
+    q = zipfish(rng, n, n_rows)
+    if host_cold:
+        t_cold = torch.empty(shape, dtype=torch.float32, pin_memory=True)
+        t_cold.copy_(torch.from_numpy(cold))
+    else:
+        t_cold = dev(cold)
+    t_hot, t_q, t_ids = dev(hot), dev(q), dev(hot_ids)
+    out, loc = ops.cached_fetch(t_cold, t_hot, t_q, t_ids, return_loc=True)
+    assert np.array_equal(out.cpu().numpy(), O.cached_fetch(cold, hot, q, hot_ids))
+    assert np.array_equal(loc.cpu().numpy(), O.lookup_sorted(q, hot_ids))
+    out2 = ops.cached_fetch_loc(t_cold, t_hot, t_q, loc)
+    assert torch.equal(out, out2)
+    # set on duplicate-free ids
+    u = np.unique(q)
+    rows = rng.standard_normal((u.size,) + shape[1:]).astype(np.float32)
+    w_cold, w_hot = cold.copy(), hot.copy()
+    O.cached_set(rows, w_cold, w_hot, u, hot_ids)
+    ops.cached_set(dev(rows), t_cold, t_hot, dev(u), t_ids)
+    torch.cuda.synchronize()
+    assert np.array_equal(t_cold.cpu().numpy(), w_cold)
+    assert np.array_equal(t_hot.cpu().numpy(), w_hot)
+
+
+# ---- combine ------------------------------------------------------------------------------
+def combine_tol_ok(got, want64, scale):
+    """tolerance mode: |got - exact| <= 1e-5 * max|exact| elementwise (exact = float64 sums)."""
+    return np.abs(got.astype(np.float64) - want64).max() <= 1e-5 * scale
+
+
+CASES = [  # (n, dim, id space, kind)
+    (0, 8, 100, "zipf"), (1, 8, 100, "zipf"), (2, 4, 2, "zipf"), (31, 1, 10, "zipf"),
+    (32, 7, 10, "zipf"), (33, 128, 50, "zipf"), (1000, 64, 1, "same"), (4096, 128, 10**9, "distinct"),
+    (5000, 100, 300, "zipf"), (20_000, 128, 2_400_000, "zipf"), (70_001, 260, 5000, "zipf"),
+    (65_536, 64, 1_000_000, "zipf"),
+]
+
+
+@pytest.mark.parametrize("n,dim,space,kind", CASES)
+@pytest.mark.parametrize("bounded", [True, False])
+def test_combine(lib, n, dim, space, kind, bounded):
+    _, ops = lib
+    rng = np.random.default_rng(9 + n + dim)
+    if kind == "same":
+        idx = np.full(n, 0, np.int64)
+    elif kind == "distinct":
+        idx = rng.choice(space, n, replace=False).astype(np.int64)
+    else:
+        idx = zipfish(rng, n, space)
+    if not bounded and n > 3:
+        idx = idx.copy()
+        idx[:3] = [-5, 2**40 + 7, -(2**50)]        # negative and wide ids: full 64-bit signed sort
+    grad = (rng.standard_normal((n, dim)) * 1e-3).astype(np.float32)
+    bound = space if bounded else 0
+    wu, ws, wc = O.combine_sequential(idx, grad)
+    if 0 < n <= 20_000:
+        tu, ts, tc = O.only_unique_grads(torch.from_numpy(idx), torch.from_numpy(grad))
+        assert np.array_equal(ts.numpy(), ws)       # the reference's own torch calls agree
+    _, w64, _ = O.combine_float64(idx, grad)
+
+    t_idx, t_grad = dev(idx), dev(grad)
+    # deterministic-order mode: bit-equal to CPU index_add_
+    uids, sums, cnts, nu, inv = ops.combine_padded(t_idx, t_grad, bound, ops.COMBINE_EXACT,
+                                                   return_inverse=True)
+    U = int(nu.item())
+    assert U == wu.size
+    assert np.array_equal(uids[:U].cpu().numpy(), wu)
+    assert np.array_equal(cnts[:U].cpu().numpy(), wc)
+    assert np.array_equal(sums[:U].cpu().numpy(), ws)
+    if n:
+        assert np.array_equal(wu[inv.cpu().numpy()], idx)
+    # fast mode: ids/counts exact, sums within 1e-5 of the float64 sums, and reproducible
+    uids, sums, cnts = ops.combine(t_idx, t_grad, bound, ops.COMBINE_FAST)
+    assert np.array_equal(uids.cpu().numpy(), wu) and np.array_equal(cnts.cpu().numpy(), wc)
+    if n:
+        got = sums.cpu().numpy()
+        assert combine_tol_ok(got, w64, np.abs(w64).max())
+        _, sums2, _ = ops.combine(t_idx, t_grad, bound, ops.COMBINE_FAST)
+        assert torch.equal(sums, sums2)
+        # runs that fit inside one chunk are summed left to right: bit-equal to the exact mode
+        short = wc <= 1
+        assert np.array_equal(got[short], ws[short])
+
+
+def test_unique_grads_dropin(lib):
+    from hades_amd import sparse_optim as S
+    rng = np.random.default_rng(10)
+    idx = zipfish(rng, 3000, 200)
+    grad = rng.standard_normal((3000, 16)).astype(np.float32)
+    cnt = rng.integers(1, 5, 3000).astype(np.int64)
+    u, m = S.unique_grads(dev(idx), dev(grad), mode=S.ops.COMBINE_EXACT)
+    wu, wm = O.unique_grads(idx, grad)
+    assert np.array_equal(u.cpu().numpy(), wu.numpy())
+    assert np.allclose(m.cpu().numpy(), wm.numpy(), rtol=1e-6, atol=0)
+    u, m = S.unique_grads(dev(idx), dev(grad), dev(cnt), mode=S.ops.COMBINE_EXACT)
+    wu, wm = O.unique_grads(idx, grad, cnt)
+    assert np.array_equal(u.cpu().numpy(), wu.numpy())
+    assert np.allclose(m.cpu().numpy(), wm.numpy(), rtol=1e-6, atol=0)
+    u, s, c = S.only_unique_grads(dev(idx), dev(grad), mode=S.ops.COMBINE_EXACT)
+    wu, ws, wc = O.only_unique_grads(idx, grad)
+    assert torch.equal(s.cpu(), ws) and torch.equal(c.cpu(), wc) and torch.equal(u.cpu(), wu)
+
+
+# ---- row optimizers -------------------------------------------------------------------------
+@pytest.mark.parametrize("dim", [64, 128, 7])
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_adagrad_update(lib, dim, host_cold):
+    _, ops = lib
+    rng = np.random.default_rng(11 + dim)
+    n_rows, h = 30_000, 4000
+    cw = (rng.standard_normal((n_rows, dim)) * 0.01).astype(np.float32)
+    cs = np.zeros((n_rows, dim), np.float32)
+    hot_ids = np.sort(rng.choice(n_rows, h, replace=False)).astype(np.int64)
+    hw, hs = cw[hot_ids].copy(), cs[hot_ids].copy()
+
+    def place(a):
+        if host_cold:
+            t = torch.empty(a.shape, dtype=torch.float32, pin_memory=True)
+            t.copy_(torch.from_numpy(a))
+            return t
+        return dev(a)
+    t_cw, t_cs, t_hw, t_hs, t_ids = place(cw), place(cs), dev(hw), dev(hs), dev(hot_ids)
+    for step in range(3):
+        u = np.unique(zipfish(rng, 9000, n_rows))
+        g = (rng.standard_normal((u.size, dim)) * 1e-3).astype(np.float32)
+        O.sparse_adagrad_step(cw, cs, hw, hs, hot_ids, u, g, 0.01, 1e-10)
+        # pad the device batch and pass the live count from device memory
+        pad = 100
+        t_u = dev(np.concatenate([u, np.zeros(pad, np.int64)]))
+        t_g = dev(np.concatenate([g, np.ones((pad, dim), np.float32)]))
+        nu = torch.tensor([u.size], dtype=torch.int64, device="cuda")
+        ops.adagrad_update_(t_u, t_g, t_hw, t_hs, t_cw, t_cs, t_ids, 0.01, 1e-10, num_unique=nu)
+        torch.cuda.synchronize()
+        for got, want in ((t_cw, cw), (t_cs, cs), (t_hw, hw), (t_hs, hs)):
+            assert np.array_equal(got.cpu().numpy(), want)      # one rounding per operation: bit-exact
+
+
+def test_adagrad_vs_torch_optim(lib):
+    """The same update against torch.optim.Adagrad on a dense parameter: <= 1e-5 relative."""
+    _, ops = lib
+    rng = np.random.default_rng(12)
+    n_rows, dim = 2000, 32
+    w0 = (rng.standard_normal((n_rows, dim)) * 0.01).astype(np.float32)
+    p = torch.nn.Parameter(torch.from_numpy(w0.copy()))
+    opt = torch.optim.Adagrad([p], lr=0.01, eps=1e-10)
+    t_w, t_s = dev(w0), torch.zeros((n_rows, dim), device="cuda")
+    for _ in range(3):
+        u = np.unique(rng.integers(0, n_rows, 700))
+        g = (rng.standard_normal((u.size, dim)) * 1e-3).astype(np.float32)
+        dense = np.zeros_like(w0)
+        dense[u] = g
+        p.grad = torch.from_numpy(dense)
+        opt.step()
+        ops.adagrad_update_(dev(u), dev(g), None, None, t_w, t_s, None, 0.01, 1e-10)
+    assert np.allclose(t_w.cpu().numpy(), p.detach().numpy(), rtol=1e-5, atol=1e-9)
+
+
+def test_adam_update(lib):
+    _, ops = lib
+    rng = np.random.default_rng(13)
+    n_rows, h, dim = 8000, 1000, 64
+    w = (rng.standard_normal((n_rows, dim)) * 0.01).astype(np.float32)
+    st = np.zeros(n_rows, np.float32); m = np.zeros_like(w); v = np.zeros_like(w)
+    hot_ids = np.sort(rng.choice(n_rows, h, replace=False)).astype(np.int64)
+    t_cold = tuple(dev(x) for x in (w, st, m, v))
+    t_hot = tuple(dev(x[hot_ids]) for x in (w, st, m, v))
+    t_ids = dev(hot_ids)
+    for _ in range(3):
+        u = np.unique(zipfish(rng, 3000, n_rows))
+        g = (rng.standard_normal((u.size, dim)) * 1e-2).astype(np.float32)
+        w[u], st[u], m[u], v[u] = O.adam_rows(w[u], st[u], m[u], v[u], g, 0.01, 0.9, 0.999, 1e-8)
+        ops.adam_update_(dev(u), dev(g), t_hot, t_cold, t_ids, 0.01, 0.9, 0.999, 1e-8)
+    torch.cuda.synchronize()
+    for k, want in enumerate((w, st, m, v)):
+        got = t_cold[k].cpu().numpy()
+        got[hot_ids] = t_hot[k].cpu().numpy()
+        if k == 0:
+            # powf differs by an ulp between host and device and 1 - 0.999^t amplifies it:
+            # compare to 1e-4 of one update (lr = 0.01)
+            assert np.abs(got - want).max() <= 1e-4 * 0.01
+        elif k == 1:
+            assert np.array_equal(got, want)
+        else:
+            assert np.allclose(got, want, rtol=1e-6, atol=1e-12)
+
+
+# ---- cold-gradient accumulator ------------------------------------------------------------------
+@pytest.mark.parametrize("dim", [128, 5])
+def test_hash_accumulator(lib, dim):
+    _, ops = lib
+    rng = np.random.default_rng(14 + dim)
+    acc = ops.ColdGradAccumulator(num_slots=4096, dim=dim, id_bound=10**6)
+    model = O.ColdGradAccumulatorModel(dim)
+    for rounds in range(2):
+        for step in range(4):
+            ids = np.minimum(rng.pareto(0.5, 900).astype(np.int64), 10**6 - 1)
+            g = (rng.standard_normal((900, dim)) * 1e-3).astype(np.float32)
+            u, s, c = O.combine_sequential(ids, g)
+            model.accumulate(u, s, c)
+            uids, sums, cnts, nu = ops.combine_padded(dev(ids), dev(g), 10**6, ops.COMBINE_EXACT)
+            acc.accumulate(uids, sums, cnts, num_rows=nu)
+        wi, ws, wc = model.flush()
+        gi, gs, gc = acc.flush(cap=4096)
+        assert np.array_equal(gi.cpu().numpy(), wi)
+        assert np.array_equal(gc.cpu().numpy(), wc)
+        assert np.array_equal(gs.cpu().numpy(), ws)   # one add per slot per step, in step order
+    gi, _, _ = acc.flush(cap=4096)
+    assert gi.numel() == 0
+    assert bool((acc.keys == -1).all()) and float(acc.accum.abs().sum()) == 0.0
+
+
+def test_hash_accumulator_overflow_is_reported(lib):
+    _, ops = lib
+    acc = ops.ColdGradAccumulator(num_slots=64, dim=4)
+    ids = torch.arange(100, dtype=torch.int64, device="cuda")
+    acc.accumulate(ids, torch.ones((100, 4), device="cuda"))
+    with pytest.raises(RuntimeError):
+        acc.flush()
+
+
+# ---- the whole step at benchmark size: properties that do not need the oracle --------------------
+def test_full_size_step_properties(lib):
+    _, ops = lib
+    from hades_amd import synth
+    from hades_amd.sparse_optim import SparseAdagrad
+    cfg = synth.CONFIGS["cfg2"]
+    N, D, H, n = cfg["num_rows"], cfg["dim"], cfg["num_hot"], cfg["batch"]
+    table = torch.empty((N, D), device="cuda")
+    synth.fill_normal_(table, 0.01, 1)
+    hot_ids = synth.hot_ids(N, H, "cuda")
+    opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10)
+    sampler = synth.ZipfSampler(N, cfg["zipf_s"], "cuda")
+    q = synth.make_ids(sampler, N, n, 7)
+    grad = synth.make_grads(n, D, 8, "cuda")
+    # fetch agrees with plain indexing of the merged table (hot copy == cold copy before any update)
+    rows = opt.fetch(q)
+    assert torch.equal(rows, table[q])
+    loc = ops.lookup(q, hot_ids)
+    hit = loc >= 0
+    assert torch.equal(hot_ids[loc[hit]], q[hit])
+    assert not torch.isin(q[~hit], hot_ids).any()
+    hot_mask, hot_pos, cold_pos = ops.split(loc)
+    assert torch.equal(hot_mask, hit)
+    assert torch.equal(hot_pos, torch.nonzero(hit).flatten())
+    assert torch.equal(cold_pos, torch.nonzero(~hit).flatten())
+    # combine: torch's own unique/index_add_ on the device as an independent check
+    uids, sums, cnts, nu = opt.step(q, grad)
+    U = int(nu.item())
+    tu, tinv, tc = torch.unique(q, return_inverse=True, return_counts=True)
+    assert U == tu.numel() and torch.equal(uids[:U], tu) and torch.equal(cnts[:U], tc)
+    ref = torch.zeros((U, D), dtype=torch.float64, device="cuda").index_add_(0, tinv, grad.double())
+    assert (sums[:U].double() - ref).abs().max().item() <= 1e-5 * ref.abs().max().item()
+    assert int(cnts[:U].sum()) == n
+    # update touched exactly the rows of uids, hot rows in the hot copy only
+    uloc = ops.lookup(uids[:U], hot_ids)
+    cold_u = uids[:U][uloc < 0]
+    changed = (opt.cold_s.abs().sum(1) > 0).nonzero().flatten()
+    assert torch.equal(changed, cold_u)
+    hot_changed = (opt.hot_s.abs().sum(1) > 0).nonzero().flatten()
+    assert torch.equal(hot_changed, torch.sort(uloc[uloc >= 0]).values)
+    g = sums[:U][uloc < 0]
+    assert torch.equal(opt.cold_s[cold_u], g * g)      # first step from a zero accumulator

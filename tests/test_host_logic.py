@@ -1,0 +1,93 @@
+"""Host-side logic that needs no GPU: the drop-in module's surface and argument checks, hot-set
+placement, the synthetic workload generators."""
+import inspect
+
+import numpy as np
+import pytest
+import torch
+
+import hades_amd
+from hades_amd import cache, synth
+from oracle import hades_oracle as O
+
+
+def test_dropin_surface_matches_reference_binding():
+    # names and argument order of src/pybind.cc:46-70
+    E = hades_amd.install_as_embcachelib()
+    import EmbCacheLib
+    assert EmbCacheLib is E
+    want = {
+        "cudaSplit": ["ids", "mask"],
+        "cudaPin": ["tensor"], "cudaUnpin": ["tensor"],
+        "cudaFetch": ["src", "src_index", "dst", "dst_index"],
+        "cudaFetch2": ["src", "src_index", "dst"],
+        "cudaFetchWithCache2": ["cpu_src", "gpu_src", "src_index", "index_map", "dst"],
+        "cudaSet": ["src", "dst", "dst_index"],
+        "cudaSetWithCache": ["src", "cpu_dst", "gpu_dst", "dst_index", "index_map"],
+        "cudaCombine": ["src", "dst", "dst_index"],
+        "cudaPinPtr": ["ptr", "size"], "cudaUnpinPtr": ["ptr"],
+    }
+    for name, params in want.items():
+        assert list(inspect.signature(getattr(E, name)).parameters) == params, name
+    for name in ("cudaReminder", "cudaBinarySearch", "cudaBinarySearch2"):   # first argument is `in`
+        assert callable(getattr(E, name))
+
+
+def test_dropin_rejects_host_tensors_without_gpu():
+    import hades_amd.EmbCacheLib as E
+    a = torch.zeros((4, 4))
+    i = torch.zeros(2, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="pageable host memory|device tensor"):
+        E.cudaFetch2(a, i, a)
+    with pytest.raises(RuntimeError):
+        E.cudaSplit(i, torch.zeros(4, dtype=torch.int8))
+
+
+def test_select_hot_ids_matches_oracle_and_reference_recipe():
+    g = torch.Generator().manual_seed(0)
+    hotness = torch.rand(5000, generator=g)
+    for k in (0, 1, 777, 5000):
+        got = cache.select_hot_ids(hotness, k)
+        assert np.array_equal(got.numpy(), O.select_hot_ids(hotness, k))
+        assert got.numel() == k
+        if 0 < k < 5000:
+            assert hotness[got].min() >= np.sort(hotness.numpy())[-k]
+    thr = cache.hot_ids_by_threshold(hotness, 0.9)
+    assert np.array_equal(thr.numpy(), np.nonzero(hotness.numpy() >= 0.9)[0])
+
+
+def test_rank_to_id_is_a_bijection_and_hot_ids_sorted():
+    for n_rows in (10, 1000, 99_991, 2_400_000):
+        ranks = torch.arange(1, n_rows + 1, dtype=torch.int64)
+        ids = synth.rank_to_id(ranks, n_rows)
+        assert ids.min() == 0 and ids.max() == n_rows - 1
+        assert torch.unique(ids).numel() == n_rows
+    hot = synth.hot_ids(99_991, 1000)
+    assert bool((hot[1:] > hot[:-1]).all())
+    assert set(hot.tolist()) == set(synth.rank_to_id(torch.arange(1, 1001), 99_991).tolist())
+
+
+def test_zipf_sampler_statistics():
+    # cfg1: 1M ranks, s = 1.1, hot = top 10 %: expected hot-hit fraction 0.919
+    cfg = synth.CONFIGS["cfg1"]
+    s = synth.ZipfSampler(cfg["num_rows"], cfg["zipf_s"])
+    g = torch.Generator().manual_seed(1)
+    ranks = s.sample_ranks(200_000, g)
+    assert ranks.min() >= 1 and ranks.max() <= cfg["num_rows"]
+    hit = float((ranks <= cfg["num_hot"]).float().mean())
+    assert abs(hit - 0.919) < 0.005
+    k = torch.arange(1, cfg["num_rows"] + 1, dtype=torch.float64)
+    p1 = float(1.0 / k.pow(-1.1).sum())
+    assert abs(float((ranks == 1).float().mean()) - p1) < 0.003
+    ids = synth.make_ids(s, cfg["num_rows"], 65_536, 5)
+    assert torch.equal(ids, synth.make_ids(s, cfg["num_rows"], 65_536, 5))      # seeded
+    u = torch.unique(ids).numel()
+    assert abs(u - 17_235) < 600                                                 # E[unique] of cfg1
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess, sys, os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr

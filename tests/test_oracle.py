@@ -1,0 +1,416 @@
+"""Pins the CPU oracle (oracle/hades_oracle.py, oracle/hades_oracle.c) against library routines,
+brute force, closed forms and the recipes held by the reference's own test scripts.  No GPU."""
+import bisect
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hades_oracle as O
+
+RNG = np.random.default_rng(20251125)
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+# ---- routing ---------------------------------------------------------------------
+def test_upper_bound_matches_bisect_and_edges():
+    rng = np.random.default_rng(1)
+    r = np.sort(rng.integers(-50, 50, size=40)).astype(np.int64)  # duplicates allowed in a range
+    v = rng.integers(-60, 60, size=300).astype(np.int64)
+    want = np.array([bisect.bisect_right(r.tolist(), x) for x in v.tolist()], dtype=np.int64)
+    assert np.array_equal(O.upper_bound(r, v), want)
+    assert O.upper_bound(np.zeros(0, np.int64), v).sum() == 0          # empty range
+    assert O.upper_bound(r, np.array([r[0] - 1]))[0] == 0              # below the minimum
+    assert O.upper_bound(r, np.array([r[-1]]))[0] == r.size            # equal to the maximum
+    assert O.upper_bound(r.astype(np.int32), v.astype(np.int32)).dtype == np.int32
+
+
+def test_reminder_is_c_remainder():
+    v = np.array([7, -7, 0, 12345678901, -1], dtype=np.int64)
+    want = np.array([int(np.fmod(x, 4)) for x in v], dtype=np.int64)
+    assert np.array_equal(O.c_remainder(v, 4), want)
+    assert list(O.c_remainder(v, 4)) == [3, -3, 0, 12345678901 % 4, -1]
+
+
+def test_owner_rank_and_split_sizes_recipe():
+    # the recipe printed by test/test_binarysearch2.py:6-27, with an assertion added:
+    # ids in [0, 3M), 2 partitions x 4 local GPUs, then split sizes by sorted owner
+    num_part, local = 2, 4
+    rng = np.random.default_rng(2)
+    index = rng.integers(0, 3_000_000, size=1000).astype(np.int64)
+    range_partition = np.array([i * 3_000_000 // num_part for i in range(num_part + 1)], np.int64)
+    owner = O.owner_rank(index, range_partition, local)
+    want = np.array([(bisect.bisect_right(range_partition.tolist(), x) - 1) * local + x % local
+                     for x in index.tolist()], dtype=np.int64)
+    assert np.array_equal(owner, want)
+    assert owner.min() >= 0 and owner.max() < num_part * local
+    sizes = O.split_sizes(np.sort(owner), num_part * local)
+    assert np.array_equal(sizes, np.bincount(owner, minlength=num_part * local))
+    assert sizes.sum() == index.size
+
+
+# ---- lookup -----------------------------------------------------------------------
+def test_lookup_sorted_brute_force_and_edges():
+    rng = np.random.default_rng(3)
+    hot = np.sort(rng.choice(500, size=60, replace=False)).astype(np.int64)
+    q = rng.integers(-5, 510, size=400).astype(np.int64)
+    eq = q[:, None] == hot[None, :]
+    want = np.where(eq.any(1), eq.argmax(1), -1)
+    assert np.array_equal(O.lookup_sorted(q, hot), want)
+    assert np.array_equal(O.lookup_sorted(q, np.zeros(0, np.int64)), np.full(q.size, -1))
+    assert np.array_equal(O.lookup_sorted(np.array([hot[0], hot[-1], hot[0] - 1, hot[-1] + 1]), hot),
+                          [0, hot.size - 1, -1, -1])
+    # agrees with the dense index_map of the reference (cache.py:163,170)
+    m = O.dense_index_map(600, hot)
+    qq = q[(q >= 0) & (q < 600)]
+    assert np.array_equal(O.lookup_sorted(qq, hot), m[qq])
+
+
+def test_select_hot_ids_is_topk_by_hotness():
+    hotness = torch.tensor([0.1, 5.0, 3.0, 9.0, 0.0, 4.0])
+    assert list(O.select_hot_ids(hotness, 3)) == [1, 3, 5]
+    assert list(O.select_hot_ids(hotness, 0)) == []
+    cand = torch.tensor([0, 2, 4, 5])
+    assert list(O.select_hot_ids(hotness, 2, cand)) == [2, 5]
+
+
+# ---- split ------------------------------------------------------------------------
+def test_split_matches_reference_cpu_recipe():
+    # test/test_split.py:9-37: hot/remote masks -> int8 class table -> boolean-mask split on CPU
+    torch.manual_seed(42)
+    n_nodes = 20_000
+    remote = torch.zeros(n_nodes).bool()
+    remote[torch.randint(0, n_nodes, (n_nodes // 2,))] = True
+    hot = torch.zeros(n_nodes).bool()
+    hot[torch.randint(0, n_nodes, (n_nodes // 2,))] = True
+    total = torch.zeros(n_nodes).char()
+    total[hot & remote] = 1
+    total[(~hot) & remote] = 2
+    index = torch.randint(0, n_nodes, (5000,))
+    local_m, rhot_m, rcold_m = O.split_masks(index.numpy(), total.numpy())
+    assert np.array_equal(rhot_m, (hot & remote)[index].numpy())
+    assert np.array_equal(rcold_m, ((~hot) & remote)[index].numpy())
+    assert np.array_equal(local_m, (~remote)[index].numpy())
+    assert np.array_equal(local_m ^ rhot_m ^ rcold_m, np.ones(5000, bool))   # disjoint cover
+    assert not (local_m & rhot_m).any() and not (rhot_m & rcold_m).any()
+    # a class value outside {0,1,2} sets no mask (split.cu:37-43 has no else branch)
+    t2 = total.numpy().copy()
+    t2[index[0]] = 5
+    a, b, c = O.split_masks(index.numpy(), t2)
+    assert not (a[0] or b[0] or c[0])
+
+
+def test_split_compact_is_nonzero():
+    loc = np.array([3, -1, -1, 0, 7, -1], dtype=np.int64)
+    hot, hp, cp = O.split_compact(loc)
+    assert list(hot) == [True, False, False, True, True, False]
+    assert list(hp) == [0, 3, 4] and list(cp) == [1, 2, 5]
+    assert hp.size + cp.size == loc.size
+
+
+# ---- gather / scatter: the reference's test recipes ------------------------------------
+def _cache_case(rng, n_rows=4000, n_cached=2000, n_q=500, dim=8, dtype=np.float32):
+    # test/test_cached_fetch.py:8-17 scaled down
+    src = rng.standard_normal((n_rows, dim)).astype(dtype)
+    cached_idx = rng.permutation(n_cached).astype(np.int64)
+    idx_map = np.full(n_rows, -1, np.int64)
+    idx_map[cached_idx] = np.arange(n_cached)
+    gpu_src = src[cached_idx].copy()
+    q = rng.permutation(n_rows)[:n_q].astype(np.int64)
+    return src, gpu_src, idx_map, q
+
+
+def test_fetch_recipes_bit_exact():
+    rng = np.random.default_rng(4)
+    src, gpu_src, idx_map, q = _cache_case(rng)
+    a = src[q]                                                    # test_cached_fetch.py:22
+    assert np.array_equal(O.fetch_with_cache2(src, gpu_src, q, idx_map), a)   # :43, :60
+    assert np.array_equal(O.fetch2(src, q), a)                    # :74
+    # cached rows really come from the cache copy: poison the host copy of cached rows
+    poisoned = src.copy()
+    poisoned[idx_map != -1] = np.nan
+    assert np.array_equal(O.fetch_with_cache2(poisoned, gpu_src, q, idx_map), a)
+    # test/test_fetch.py:16: dst[dst_index] = src[src_index]
+    dst = rng.standard_normal((400, 8)).astype(np.float32)
+    want = dst.copy()
+    di = rng.permutation(400)[:100]
+    si = rng.permutation(4000)[:100]
+    want[di] = src[si]
+    assert np.array_equal(O.fetch(src, si, dst, di), want)
+    # 1-D (test_cached_fetch_1D.py)
+    s1 = src[:, 0].copy()
+    assert np.array_equal(O.fetch_with_cache2(s1, gpu_src[:, 0].copy(), q, idx_map), s1[q])
+
+
+def test_set_recipes_bit_exact():
+    rng = np.random.default_rng(5)
+    dst, gpu_dst, idx_map, q = _cache_case(rng)
+    src = rng.standard_normal((q.size, 8)).astype(np.float32)
+    want = dst.copy()
+    want[q] = src                                                  # test_cached_set.py:22
+    d1 = dst.copy()
+    O.set_rows(src, d1, q)                                         # cudaSet / cudaCombine
+    assert np.array_equal(d1[q], want[q]) and np.array_equal(d1, want)
+    d2, g2 = dst.copy(), gpu_dst.copy()
+    O.set_with_cache(src, d2, g2, q, idx_map)                      # :54-58
+    # read back through the cache: equals the plain scatter on the touched rows
+    assert np.array_equal(O.fetch_with_cache2(d2, g2, q, idx_map), want[q])
+    # and only the live copy was written
+    hit = idx_map[q] != -1
+    assert np.array_equal(d2[q[hit]], dst[q[hit]])
+
+
+def test_cached_fetch_sorted_equals_map_form():
+    rng = np.random.default_rng(6)
+    n_rows, dim = 3000, 4
+    cold = rng.standard_normal((n_rows, dim)).astype(np.float32)
+    hot_ids = np.sort(rng.choice(n_rows, 700, replace=False)).astype(np.int64)
+    hot = cold[hot_ids] + 1.0       # distinguishable
+    q = rng.integers(0, n_rows, 900).astype(np.int64)
+    m = O.dense_index_map(n_rows, hot_ids)
+    assert np.array_equal(O.cached_fetch(cold, hot, q, hot_ids), O.fetch_with_cache2(cold, hot, q, m))
+
+
+# ---- combine ---------------------------------------------------------------------------
+def _zipfish(rng, n, n_ids):
+    return np.minimum((rng.pareto(0.9, n)).astype(np.int64), n_ids - 1)
+
+
+def test_combine_torch_equals_sequential_numpy_bit_exact():
+    # index_add_ on CPU adds rows in occurrence order: a stable sort plus a left-to-right float32
+    # sum reproduces it bit for bit (also with several intra-op threads)
+    rng = np.random.default_rng(7)
+    idx = _zipfish(rng, 20000, 300)
+    grad = (rng.standard_normal((20000, 16)) * 1e-3).astype(np.float32)
+    for threads in (1, 4):
+        torch.set_num_threads(threads)
+        tu, ts, tc = O.only_unique_grads(torch.from_numpy(idx), torch.from_numpy(grad))
+        nu, ns, nc = O.combine_sequential(idx, grad)
+        assert np.array_equal(tu.numpy(), nu) and np.array_equal(tc.numpy(), nc)
+        assert np.array_equal(ts.numpy(), ns)
+    assert ts.dtype == torch.float32
+    # against float64 sums
+    du, ds, dc = O.combine_float64(idx, grad)
+    assert np.array_equal(du, nu) and np.array_equal(dc, nc)
+    assert np.abs(ns - ds).max() <= 1e-5 * np.abs(ds).max()
+
+
+def test_combine_closed_forms_and_invariants():
+    rng = np.random.default_rng(8)
+    n, d = 257, 8
+    grad = rng.standard_normal((n, d)).astype(np.float32)
+    # all distinct: output = input permuted by argsort, counts all one
+    idx = rng.permutation(10 * n)[:n].astype(np.int64)
+    u, s, c = O.combine_sequential(idx, grad)
+    order = np.argsort(idx)
+    assert np.array_equal(u, idx[order]) and np.array_equal(s, grad[order]) and (c == 1).all()
+    # all equal: one row = sequential column sum, count n
+    u, s, c = O.combine_sequential(np.full(n, 42, np.int64), grad)
+    acc = np.zeros(d, np.float32)
+    for r in grad:
+        acc = acc + r
+    assert list(u) == [42] and list(c) == [n] and np.array_equal(s[0], acc)
+    # invariants on a skewed batch
+    idx = _zipfish(rng, 5000, 100)
+    g = rng.standard_normal((5000, d)).astype(np.float32)
+    u, s, c = O.combine_sequential(idx, g)
+    assert c.sum() == 5000 and (np.diff(u) > 0).all()
+    assert np.allclose(s.sum(0), g.sum(0), rtol=1e-4, atol=1e-3)
+    # empty
+    u, s, c = O.combine_sequential(np.zeros(0, np.int64), np.zeros((0, d), np.float32))
+    assert u.size == 0 and s.shape == (0, d) and c.size == 0
+    # -0.0 handling: 0.0f + (-0.0f) = +0.0f
+    u, s, c = O.combine_sequential(np.array([1]), np.array([[-0.0]], np.float32))
+    assert not np.signbit(s[0, 0])
+
+
+def test_local_aggregation_is_combine_of_concatenation():
+    # combine(concat(batches)) == combine(concat(combine(batch_t))) on ids; counts add up
+    rng = np.random.default_rng(9)
+    batches = [(_zipfish(rng, 3000, 500), rng.standard_normal((3000, 4)).astype(np.float32))
+               for _ in range(4)]
+    idx = np.concatenate([b[0] for b in batches])
+    g = np.concatenate([b[1] for b in batches])
+    u, s, c = O.combine_sequential(idx, g)
+    parts = [O.combine_sequential(*b) for b in batches]
+    u2, s2, _ = O.combine_sequential(np.concatenate([p[0] for p in parts]),
+                                     np.concatenate([p[1] for p in parts]))
+    assert np.array_equal(u, u2)
+    assert np.allclose(s, s2, rtol=1e-5, atol=1e-6)
+    cc = np.zeros(u.size, np.int64)
+    for p in parts:
+        cc[np.searchsorted(u, p[0])] += p[2]
+    assert np.array_equal(cc, c)
+
+
+def test_unique_grads_mean_and_count_quirk():
+    idx = torch.tensor([5, 3, 5, 5, 3])
+    grad = torch.tensor([[1.0], [2.0], [3.0], [5.0], [4.0]])
+    u, m = O.unique_grads(idx, grad)
+    assert u.tolist() == [3, 5] and m.flatten().tolist() == [3.0, 3.0]
+    # with cnt: divisor = 1 + sum(cnt) (sparse_optim.py:145-148)
+    u, m = O.unique_grads(idx, grad, cnt=torch.tensor([1, 1, 1, 1, 1]))
+    assert m.flatten().tolist() == [6.0 / 3, 9.0 / 4]
+
+
+# ---- optimizers --------------------------------------------------------------------------
+def test_adagrad_matches_torch_optim():
+    rng = np.random.default_rng(10)
+    w0 = (rng.standard_normal((300, 16)) * 0.01).astype(np.float32)
+    p = torch.nn.Parameter(torch.from_numpy(w0.copy()))
+    opt = torch.optim.Adagrad([p], lr=0.01, eps=1e-10)
+    w, s = w0.copy(), np.zeros_like(w0)
+    for step in range(3):
+        g = (rng.standard_normal(w0.shape) * 1e-3).astype(np.float32)
+        p.grad = torch.from_numpy(g.copy())
+        opt.step()
+        w, s = O.adagrad_rows(w, s, g, 0.01, 1e-10)
+        # tolerance of the update parity: 1e-5 relative (bit-exact unless the torch build fuses)
+        assert np.allclose(w, p.detach().numpy(), rtol=1e-5, atol=1e-8)
+        assert np.allclose(s, opt.state[p]["sum"].numpy(), rtol=1e-6, atol=0)
+
+
+def test_adagrad_special_cases():
+    w = np.array([[0.5, -0.25]], np.float32)
+    s = np.array([[0.0, 4.0]], np.float32)
+    w1, s1 = O.adagrad_rows(w, s, np.zeros_like(w), 0.01, 1e-10)        # g = 0: w unchanged
+    assert np.array_equal(w1, w) and np.array_equal(s1, s)
+    g = np.array([[2.0, -3.0]], np.float32)                               # s = 0: step = lr*sign(g)
+    w1, s1 = O.adagrad_rows(np.zeros_like(g), np.zeros_like(g), g, 0.01, 1e-10)
+    assert np.allclose(w1, -0.01 * np.sign(g), rtol=1e-6) and np.array_equal(s1, g * g)
+    # a wrong sign or a dropped sqrt would fail this one: s=9 -> std=3 (+eps), w -= lr*g/3
+    w1, _ = O.adagrad_rows(np.ones((1, 1), np.float32), np.full((1, 1), 5.0, np.float32),
+                           np.full((1, 1), 2.0, np.float32), 0.3, 0.0)
+    assert np.allclose(w1, 1.0 - 0.3 * 2.0 / 3.0, rtol=1e-6)
+
+
+def test_adam_matches_torch_optim_adam():
+    rng = np.random.default_rng(11)
+    w0 = (rng.standard_normal((50, 8)) * 0.01).astype(np.float32)
+    p = torch.nn.Parameter(torch.from_numpy(w0.copy()))
+    opt = torch.optim.Adam([p], lr=0.01, betas=(0.9, 0.999), eps=1e-8)
+    w = w0.copy()
+    step = np.zeros(50, np.float32)
+    m = np.zeros_like(w0)
+    v = np.zeros_like(w0)
+    for _ in range(4):
+        g = (rng.standard_normal(w0.shape) * 1e-2).astype(np.float32)
+        p.grad = torch.from_numpy(g.copy())
+        opt.step()
+        w, step, m, v = O.adam_rows(w, step, m, v, g, 0.01, 0.9, 0.999, 1e-8)
+        # the reference forms 1 - beta^step in float32 (sparse_optim.py:652-655): 1 - 0.999 carries a
+        # relative error near 6e-5 that torch.optim.Adam (Python doubles) does not have, so the two
+        # agree to about 1e-4 of one update (lr), not to 1e-5 of w
+        assert np.abs(w - p.detach().numpy()).max() <= 2e-4 * 0.01
+    assert (step == 4).all()
+
+
+# ---- accumulator ----------------------------------------------------------------------------
+def test_accumulator_flush_equals_combine_of_all_batches():
+    rng = np.random.default_rng(12)
+    acc = O.ColdGradAccumulatorModel(4)
+    all_ids, all_g = [], []
+    for _ in range(5):
+        ids = _zipfish(rng, 400, 200)
+        g = rng.standard_normal((400, 4)).astype(np.float32)
+        u, s, c = O.combine_sequential(ids, g)
+        acc.accumulate(u, s, c)
+        all_ids.append(ids)
+        all_g.append(g)
+    ids, sums, cnts = acc.flush()
+    u, s, c = O.combine_float64(np.concatenate(all_ids), np.concatenate(all_g))
+    assert np.array_equal(ids, u) and np.array_equal(cnts, c)
+    assert np.allclose(sums, s, rtol=1e-5, atol=1e-6)
+    assert acc.flush()[0].size == 0          # emptied
+
+
+# ---- C restatement vs numpy restatement -----------------------------------------------------
+def test_c_oracle_agrees_with_numpy_oracle(oracle_c):
+    C = oracle_c
+    rng = np.random.default_rng(13)
+    i64 = np.int64
+    rng_part = np.array([0, 1000, 2500, 4000], i64)
+    v = rng.integers(0, 4000, 777).astype(i64)
+    out = np.empty_like(v)
+    C.o_binary_search2(_p(v), _p(rng_part), ctypes.c_int64(4), _p(out), ctypes.c_int64(v.size))
+    assert np.array_equal(out, O.upper_bound(rng_part, v))
+    C.o_binary_search(_p(v), _p(rng_part), ctypes.c_int64(4), ctypes.c_int64(4), _p(out),
+                      ctypes.c_int64(v.size))
+    assert np.array_equal(out, O.owner_rank(v, rng_part, 4))
+    vv = rng.integers(-100, 100, 50).astype(i64)
+    o2 = np.empty_like(vv)
+    C.o_reminder(_p(vv), ctypes.c_int64(7), _p(o2), ctypes.c_int64(vv.size))
+    assert np.array_equal(o2, O.c_remainder(vv, 7))
+
+    hot = np.sort(rng.choice(4000, 500, replace=False)).astype(i64)
+    loc = np.empty_like(v)
+    C.o_lookup_sorted(_p(v), ctypes.c_int64(v.size), _p(hot), ctypes.c_int64(hot.size), _p(loc))
+    assert np.array_equal(loc, O.lookup_sorted(v, hot))
+
+    table = rng.integers(0, 4, 4000).astype(np.int8)
+    m = [np.empty(v.size, np.uint8) for _ in range(3)]
+    C.o_split(_p(v), _p(table), ctypes.c_int64(v.size), _p(m[0]), _p(m[1]), _p(m[2]))
+    for got, want in zip(m, O.split_masks(v, table)):
+        assert np.array_equal(got.astype(bool), want)
+
+    src, gpu_src, idx_map, q = _cache_case(rng)
+    dst = np.empty((q.size, 8), np.float32)
+    C.o_fetch_with_cache2(_p(src), _p(gpu_src), _p(q), _p(idx_map), _p(dst), ctypes.c_int64(q.size),
+                          ctypes.c_int64(32))
+    assert np.array_equal(dst, O.fetch_with_cache2(src, gpu_src, q, idx_map))
+    C.o_fetch2(_p(src), _p(q), _p(dst), ctypes.c_int64(q.size), ctypes.c_int64(32))
+    assert np.array_equal(dst, src[q])
+    rows = rng.standard_normal((q.size, 8)).astype(np.float32)
+    c_cpu, c_gpu = src.copy(), gpu_src.copy()
+    C.o_set_with_cache(_p(rows), _p(c_cpu), _p(c_gpu), _p(q), _p(idx_map), ctypes.c_int64(q.size),
+                       ctypes.c_int64(32))
+    n_cpu, n_gpu = src.copy(), gpu_src.copy()
+    O.set_with_cache(rows, n_cpu, n_gpu, q, idx_map)
+    assert np.array_equal(c_cpu, n_cpu) and np.array_equal(c_gpu, n_gpu)
+
+    idx = _zipfish(rng, 5000, 400)
+    g = (rng.standard_normal((5000, 8)) * 1e-3).astype(np.float32)
+    uids = np.empty(5000, i64); sums = np.empty((5000, 8), np.float32); cnts = np.empty(5000, i64)
+    C.o_combine.restype = ctypes.c_int64
+    U = C.o_combine(_p(idx), _p(g), ctypes.c_int64(5000), ctypes.c_int64(8), _p(uids), _p(sums), _p(cnts))
+    nu, ns, nc = O.combine_sequential(idx, g)
+    assert U == nu.size and np.array_equal(uids[:U], nu) and np.array_equal(cnts[:U], nc)
+    assert np.array_equal(sums[:U], ns)
+
+    n_rows = 4000
+    cw = (rng.standard_normal((n_rows, 8)) * 0.01).astype(np.float32)
+    cs = np.abs(rng.standard_normal((n_rows, 8))).astype(np.float32)
+    hw, hs = cw[hot].copy(), cs[hot].copy()
+    cw2, cs2, hw2, hs2 = cw.copy(), cs.copy(), hw.copy(), hs.copy()
+    u = np.unique(v)
+    gg = (rng.standard_normal((u.size, 8)) * 1e-3).astype(np.float32)
+    C.o_adagrad(_p(u), _p(gg), ctypes.c_int64(u.size), ctypes.c_int64(8), _p(hot),
+                ctypes.c_int64(hot.size), _p(hw), _p(hs), _p(cw), _p(cs), ctypes.c_float(0.01),
+                ctypes.c_float(1e-10))
+    O.sparse_adagrad_step(cw2, cs2, hw2, hs2, hot, u, gg, 0.01, 1e-10)
+    for a, b in ((cw, cw2), (cs, cs2), (hw, hw2), (hs, hs2)):
+        assert np.array_equal(a, b)
+
+
+def test_torch_step_agrees_with_numpy_pieces():
+    rng = np.random.default_rng(14)
+    n_rows, dim = 5000, 8
+    cw = (rng.standard_normal((n_rows, dim)) * 0.01).astype(np.float32)
+    cs = np.zeros((n_rows, dim), np.float32)
+    hot = np.sort(rng.choice(n_rows, 600, replace=False)).astype(np.int64)
+    hw, hs = cw[hot].copy(), cs[hot].copy()
+    q = _zipfish(rng, 3000, n_rows)
+    g = (rng.standard_normal((3000, dim)) * 1e-3).astype(np.float32)
+    t = [torch.from_numpy(x.copy()) for x in (cw, cs, hw, hs)]
+    rows, uids, sums, cnts = O.torch_step(t[0], t[1], t[2], t[3], torch.from_numpy(hot),
+                                          torch.from_numpy(q), torch.from_numpy(g), 0.01, 1e-10)
+    assert np.array_equal(rows.numpy(), O.cached_fetch(cw, hw, q, hot))
+    u, s, c = O.combine_sequential(q, g)
+    assert np.array_equal(uids.numpy(), u) and np.array_equal(sums.numpy(), s)
+    O.sparse_adagrad_step(cw, cs, hw, hs, hot, u, s, 0.01, 1e-10)
+    for a, b in zip(t, (cw, cs, hw, hs)):
+        assert np.allclose(a.numpy(), b, rtol=1e-5, atol=1e-9)
