@@ -44,7 +44,7 @@ _SIGNATURES = {
     "hades_rows_div_count": [_P, _P, _P, _L, _L, c_int, _P],
     "hades_adagrad_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, c_float, c_float, _P],
     "hades_adam_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P,
-                          c_float, c_float, c_float, c_float, _P],
+                          c_float, ctypes.c_double, ctypes.c_double, c_float, _P],
     "hades_hash_clear": [_P, _P, _P, _L, _L, _P],
     "hades_hash_accumulate": [_P, _P, _P, _L, _P, _P, _P, _P, _L, _L, _P, _P],
     "hades_hash_flush": [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P, _P, c_size_t, _P],

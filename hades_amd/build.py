@@ -26,7 +26,7 @@ HIPCC_FLAGS = [
 ]
 # Row-update arithmetic is compared bit-for-bit with a CPU restatement that rounds after every
 # operation: forbid fused multiply-add contraction in device code.
-NO_CONTRACT = ["-ffp-contract=off"]
+NO_CONTRACT = ["-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"]
 
 
 def hipcc_path():

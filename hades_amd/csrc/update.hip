@@ -30,13 +30,15 @@ struct Vf<1> {
   typedef float type;
 };
 
-__device__ __forceinline__ float vsqrt(float x) { return __fsqrt_rn(x); }
+// sqrtf and the division operator are correctly rounded (the library is compiled with
+// -fhip-fp32-correctly-rounded-divide-sqrt); the __fsqrt_rn intrinsic is the fast native one.
+__device__ __forceinline__ float vsqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ f32x4 vsqrt(f32x4 x) {
-  return f32x4{__fsqrt_rn(x.x), __fsqrt_rn(x.y), __fsqrt_rn(x.z), __fsqrt_rn(x.w)};
+  return f32x4{sqrtf(x.x), sqrtf(x.y), sqrtf(x.z), sqrtf(x.w)};
 }
-__device__ __forceinline__ float vdiv(float a, float b) { return __fdiv_rn(a, b); }
+__device__ __forceinline__ float vdiv(float a, float b) { return a / b; }
 __device__ __forceinline__ f32x4 vdiv(f32x4 a, f32x4 b) {
-  return f32x4{__fdiv_rn(a.x, b.x), __fdiv_rn(a.y, b.y), __fdiv_rn(a.z, b.z), __fdiv_rn(a.w, b.w)};
+  return f32x4{a.x / b.x, a.y / b.y, a.z / b.z, a.w / b.w};
 }
 
 struct RowArgs {
@@ -231,19 +233,21 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
 int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                       int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,
                       float* hot_w, float* hot_step, float* hot_m, float* hot_v, float* cold_w,
-                      float* cold_step, float* cold_m, float* cold_v, float lr, float beta1,
-                      float beta2, float eps, void* stream) {
+                      float* cold_step, float* cold_m, float* cold_v, float lr, double beta1,
+                      double beta2, float eps, void* stream) {
   int rc = check_rows(uids, grad, max_rows, dim, sorted_hot, num_hot);
   if (rc != HADES_OK) return rc;
   if (max_rows == 0) return HADES_OK;
   HADES_REQUIRE(num_hot == 0 || (hot_w && hot_step && hot_m && hot_v),
                 "hot tables are null but num_hot > 0");
-  // 1 - beta is formed in double like the reference's Python float arithmetic, then rounded
-  const float omb1 = static_cast<float>(1.0 - static_cast<double>(beta1));
-  const float omb2 = static_cast<float>(1.0 - static_cast<double>(beta2));
+  // the betas arrive as doubles because the reference forms 1 - beta in Python double arithmetic
+  // before the product with a float32 tensor rounds it (python/EmbCache/sparse_optim.py:641-642):
+  // 1 - float(0.999) would be off by 1.3e-5 relative
+  const float omb1 = static_cast<float>(1.0 - beta1);
+  const float omb2 = static_cast<float>(1.0 - beta2);
   AdamArgs a{{uids, grad, num_unique, max_rows, dim, sorted_hot, num_hot},
              hot_w, hot_step, hot_m, hot_v, cold_w, cold_step, cold_m, cold_v,
-             lr, beta1, beta2, omb1, omb2, eps};
+             lr, static_cast<float>(beta1), static_cast<float>(beta2), omb1, omb2, eps};
   const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dim % 4 == 0 && aligned16({grad, hot_w, hot_m, hot_v, cold_w, cold_m, cold_v}))

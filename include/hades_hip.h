@@ -225,7 +225,7 @@ int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num
                       const int64_t* sorted_hot, int64_t num_hot,
                       float* hot_w, float* hot_step, float* hot_m, float* hot_v,
                       float* cold_w, float* cold_step, float* cold_m, float* cold_v,
-                      float lr, float beta1, float beta2, float eps, void* stream);
+                      float lr, double beta1, double beta2, float eps, void* stream);
 
 /* Cold-gradient accumulator (delayed synchronisation): an open-addressing hash table in HBM,
  * int64 key -> fp32[dim] running sum and an int64 count.  Restates on the GPU the arithmetic of
