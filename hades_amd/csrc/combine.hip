@@ -3,18 +3,25 @@
 // reduction at :310 over concatenated trainer batches).
 //
 // Pipeline, all on one stream, no host synchronisation (the number of distinct ids stays on the
-// device):
-//   1. stable LSD radix sort of (key = id, value = occurrence position), only over the key bits
-//      that id_bound leaves significant.  Stability keeps the positions of equal ids ascending,
-//      which is what makes a sequential in-segment sum reproduce CPU index_add_.
+// device) and no spin-waits between blocks:
+//   1. stable LSD radix sort of (key = id, value = occurrence position), 8 bits per pass, only
+//      over the key bits that id_bound leaves significant.  Stability keeps the positions of
+//      equal ids ascending, which is what makes a sequential in-segment sum reproduce CPU
+//      index_add_.  Per pass ONE kernel: every block derives its own global digit offsets from the
+//      per-tile digit counts [tile][digit] (column sums over all tiles and over the tiles before
+//      it), ranks its keys stably through LDS, scatters, and counts the NEXT pass's per-tile
+//      digits with aggregated global atomics at the scattered position.  Only the first pass
+//      needs a counting kernel of its own.
 //   2. run boundaries -> uids, seg_start, seg_of (index of the run every sorted position is in).
 //   3. segmented sum of the gradient rows:
 //        EXACT: one lane group per distinct id walks its rows left to right.
-//        FAST : the sorted sequence is cut into fixed chunks of R positions, one lane group per
-//               chunk; runs inside a chunk are summed left to right and stored directly, runs
-//               that cross chunk borders leave partial rows that a second kernel adds in chunk
+//        FAST : the sorted sequence is cut into fixed chunks of 32 positions per lane group; a
+//               block stages the sort permutation of its groups in LDS, every group sums its
+//               runs left to right with 16 row loads in flight, runs that cross group borders
+//               are merged in group order inside the block, and runs that cross block borders
+//               leave at most two partial rows per block that a second kernel adds in block
 //               order.  Work per group is uniform whatever the id skew; the shape of the sum
-//               depends only on (n, R), so results are reproducible run to run.
+//               depends only on (n, dim), so results are reproducible run to run.
 #include "internal.h"
 
 namespace hades {
@@ -24,6 +31,7 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kRadixBits = 8;
 constexpr int kBins = 1 << kRadixBits;
+constexpr int kMaxPasses = 8;
 
 // ---- key transforms ---------------------------------------------------------
 template <typename KeyT>
@@ -53,16 +61,28 @@ __device__ __forceinline__ KeyT load_key(const void* __restrict__ in, int64_t i)
   return static_cast<const KeyT*>(in)[i];
 }
 
-// ---- radix pass, kernel 1: per-tile digit histogram -------------------------
-// hist layout: hist[digit * nblocks + block]
-template <typename KeyT, bool FIRST, int IPT>
-__global__ __launch_bounds__(kThreads) void radix_hist_kernel(const void* __restrict__ keys_in,
-                                                             int64_t n, int shift, uint32_t mask,
-                                                             uint32_t* __restrict__ hist,
-                                                             int64_t nblocks, int64_t id_bound,
-                                                             int32_t* __restrict__ status) {
+// lanes of the wave whose `v` equals mine, among the lanes in `among` (nbits significant bits)
+__device__ __forceinline__ uint64_t match_any(uint32_t v, int nbits, uint64_t among) {
+  uint64_t peers = among;
+  for (int b = 0; b < nbits; ++b) {
+    const uint64_t bal = __ballot((v >> b) & 1u);
+    peers &= ((v >> b) & 1u) ? bal : ~bal;
+  }
+  return peers;
+}
+
+// ---- first pass only: per-tile digit counts, and zero-fill of the later passes' counts ----
+// counts layout: cnt[tile * kBins + digit]
+template <typename KeyT, int IPT>
+__global__ __launch_bounds__(kThreads) void radix_count0_kernel(
+    const int64_t* __restrict__ ids, int64_t n, uint32_t mask, uint32_t* __restrict__ cnt0,
+    uint32_t* __restrict__ cnt_later, int64_t cnt_later_len, int64_t id_bound,
+    int32_t* __restrict__ status) {
   __shared__ uint32_t s_hist[kBins];
   for (int d = threadIdx.x; d < kBins; d += kThreads) s_hist[d] = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < cnt_later_len;
+       i += static_cast<int64_t>(gridDim.x) * kThreads)
+    cnt_later[i] = 0;
   __syncthreads();
   const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * (kThreads * IPT);
   bool bad = false;
@@ -70,63 +90,59 @@ __global__ __launch_bounds__(kThreads) void radix_hist_kernel(const void* __rest
   for (int r = 0; r < IPT; ++r) {
     const int64_t i = tile0 + r * kThreads + threadIdx.x;
     if (i < n) {
-      if (FIRST && id_bound > 0) {
-        const int64_t id = static_cast<const int64_t*>(keys_in)[i];
-        bad = bad || id < 0 || id >= id_bound;
-      }
-      const KeyT k = load_key<KeyT, FIRST>(keys_in, i);
-      atomicAdd(&s_hist[static_cast<uint32_t>(k >> shift) & mask], 1u);
+      const int64_t id = ids[i];
+      bad = bad || (id_bound > 0 && (id < 0 || id >= id_bound));
+      atomicAdd(&s_hist[static_cast<uint32_t>(key_from_id<KeyT>(id)) & mask], 1u);
     }
   }
-  if (FIRST && bad) atomicOr(status, 1);
+  if (bad) atomicOr(status, 1);
   __syncthreads();
-  for (int d = threadIdx.x; d < kBins; d += kThreads) hist[d * nblocks + blockIdx.x] = s_hist[d];
+  for (int d = threadIdx.x; d < kBins; d += kThreads)
+    cnt0[static_cast<int64_t>(blockIdx.x) * kBins + d] = s_hist[d];
 }
 
-// ---- single-block exclusive scan of a u32 array (in place) ------------------
-constexpr int kScanThreads = 1024;
-constexpr int kScanItems = 8;
-__global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* __restrict__ data,
-                                                               int64_t len,
-                                                               uint32_t* __restrict__ total_out) {
-  __shared__ uint32_t smem[kScanThreads / kWave + 1];
-  uint32_t carry = 0;
-  for (int64_t base = 0; base < len; base += kScanThreads * kScanItems) {
-    const int64_t i0 = base + static_cast<int64_t>(threadIdx.x) * kScanItems;
-    uint32_t v[kScanItems];
-    uint32_t sum = 0;
-#pragma unroll
-    for (int k = 0; k < kScanItems; ++k) {
-      v[k] = (i0 + k < len) ? data[i0 + k] : 0u;
-      sum += v[k];
-    }
-    uint32_t total;
-    uint32_t ex = carry + block_exclusive_sum<uint32_t, kScanThreads>(sum, smem, &total);
-#pragma unroll
-    for (int k = 0; k < kScanItems; ++k) {
-      if (i0 + k < len) data[i0 + k] = ex;
-      ex += v[k];
-    }
-    carry += total;
-  }
-  if (total_out && threadIdx.x == 0) *total_out = carry;
-}
-
-// ---- radix pass, kernel 3: stable scatter -----------------------------------
+// ---- one radix pass ---------------------------------------------------------------------
 // Tile order: wave w of the block owns tile positions [w*IPT*64, (w+1)*IPT*64), round r of that
 // wave the 64 positions from r*64 on.  Ranks are handed out in exactly that order.
 template <typename KeyT, bool FIRST, int IPT>
-__global__ __launch_bounds__(kThreads) void radix_scatter_kernel(
+__global__ __launch_bounds__(kThreads) void radix_pass_kernel(
     const void* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, int64_t n, int shift,
-    uint32_t mask, int bits, const uint32_t* __restrict__ hist_scanned, int64_t nblocks,
-    KeyT* __restrict__ keys_out, uint32_t* __restrict__ vals_out) {
+    uint32_t mask, int bits, const uint32_t* __restrict__ cnt_cur, int64_t ntiles,
+    KeyT* __restrict__ keys_out, uint32_t* __restrict__ vals_out, uint32_t* __restrict__ cnt_next,
+    int next_shift, uint32_t next_mask, int tile_shift, int cell_bits) {
   __shared__ uint32_t s_cnt[kWaves][kBins];
   __shared__ uint32_t s_glob[kBins];
+  __shared__ uint32_t s_scan[kWaves + 1];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   for (int d = threadIdx.x; d < kWaves * kBins; d += kThreads) (&s_cnt[0][0])[d] = 0;
-  for (int d = threadIdx.x; d < kBins; d += kThreads)
-    s_glob[d] = hist_scanned[d * nblocks + blockIdx.x];
+
+  // global offset of (digit, this tile): all keys with a smaller digit, plus the keys with this
+  // digit in the tiles before this one.  Thread d owns digit d (kThreads == kBins).
+  {
+    const int d = threadIdx.x;
+    uint32_t tot = 0, pre = 0;
+    const int64_t me = blockIdx.x;
+    int64_t t = 0;
+    for (; t + 8 <= ntiles; t += 8) {
+      uint32_t h[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) h[k] = cnt_cur[(t + k) * kBins + d];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        tot += h[k];
+        pre += (t + k < me) ? h[k] : 0u;
+      }
+    }
+    for (; t < ntiles; ++t) {
+      const uint32_t h = cnt_cur[t * kBins + d];
+      tot += h;
+      pre += (t < me) ? h : 0u;
+    }
+    uint32_t total;
+    const uint32_t base = block_exclusive_sum<uint32_t, kThreads>(tot, s_scan, &total);
+    s_glob[d] = base + pre;
+  }
   __syncthreads();
 
   const int64_t wave0 = static_cast<int64_t>(blockIdx.x) * (kThreads * IPT) + wave * (IPT * kWave);
@@ -141,19 +157,9 @@ __global__ __launch_bounds__(kThreads) void radix_scatter_kernel(
     key[r] = valid ? load_key<KeyT, FIRST>(keys_in, i) : KeyT(0);
     val[r] = valid ? (FIRST ? static_cast<uint32_t>(i) : vals_in[i]) : 0u;
     const uint32_t d = static_cast<uint32_t>(key[r] >> shift) & mask;
-    // lanes of this wave that hold the same digit
-    uint64_t peers = __ballot(valid);
-#pragma unroll
-    for (int b = 0; b < kRadixBits; ++b) {
-      if (b < bits) {
-        const uint64_t bal = __ballot((d >> b) & 1u);
-        peers &= ((d >> b) & 1u) ? bal : ~bal;
-      }
-    }
+    const uint64_t peers = match_any(d, bits, __ballot(valid));
     uint32_t old = 0;
-    if (valid) {
-      old = s_cnt[wave][d];
-    }
+    if (valid) old = s_cnt[wave][d];
     // every peer has read the counter before the leader bumps it: LDS operations of one wave
     // complete in program order
     __builtin_amdgcn_wave_barrier();
@@ -162,7 +168,8 @@ __global__ __launch_bounds__(kThreads) void radix_scatter_kernel(
   }
   __syncthreads();
   // exclusive prefix over the waves, per digit
-  for (int d = threadIdx.x; d < kBins; d += kThreads) {
+  {
+    const int d = threadIdx.x;
     uint32_t run = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
@@ -175,11 +182,21 @@ __global__ __launch_bounds__(kThreads) void radix_scatter_kernel(
 #pragma unroll
   for (int r = 0; r < IPT; ++r) {
     const int64_t i = wave0 + r * kWave + lane;
-    if (i < n) {
+    const bool valid = i < n;
+    uint32_t pos = 0;
+    if (valid) {
       const uint32_t d = static_cast<uint32_t>(key[r] >> shift) & mask;
-      const uint32_t pos = s_glob[d] + s_cnt[wave][d] + rank[r];
+      pos = s_glob[d] + s_cnt[wave][d] + rank[r];
       keys_out[pos] = key[r];
       vals_out[pos] = val[r];
+    }
+    if (cnt_next != nullptr) {
+      // count this key for the next pass, in the tile it has just been written to; lanes with
+      // the same (tile, digit) send one atomic between them
+      const uint32_t nd = static_cast<uint32_t>(key[r] >> next_shift) & next_mask;
+      const uint32_t cell = ((pos >> tile_shift) << kRadixBits) | nd;
+      const uint64_t peers = match_any(cell, cell_bits, __ballot(valid));
+      if (valid && (peers & lt_mask) == 0) atomicAdd(&cnt_next[cell], __popcll(peers));
     }
   }
 }
@@ -215,10 +232,17 @@ __global__ __launch_bounds__(kThreads) void run_count_kernel(const KeyT* __restr
 template <typename KeyT>
 __global__ __launch_bounds__(kThreads) void run_emit_kernel(
     const KeyT* __restrict__ keys, const uint32_t* __restrict__ perm, int64_t n,
-    const uint32_t* __restrict__ blk_off, int64_t* __restrict__ uids,
+    const uint32_t* __restrict__ blk_cnt, int64_t* __restrict__ uids,
     uint32_t* __restrict__ seg_start, uint32_t* __restrict__ seg_of,
     int64_t* __restrict__ num_unique, int32_t* __restrict__ inverse) {
   __shared__ uint32_t smem[kWaves + 1];
+  // runs that begin in the tiles before this one
+  uint32_t before = 0;
+  for (int64_t b = threadIdx.x; b < static_cast<int64_t>(blockIdx.x); b += kThreads)
+    before += blk_cnt[b];
+  uint32_t blk_base;
+  (void)block_exclusive_sum<uint32_t, kThreads>(before, smem, &blk_base);
+
   const int64_t j0 = static_cast<int64_t>(blockIdx.x) * kUTile + threadIdx.x * kUItems;
   uint32_t flag[kUItems];
   KeyT kk[kUItems];
@@ -238,7 +262,7 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
     }
   }
   uint32_t total;
-  uint32_t u = blk_off[blockIdx.x] + block_exclusive_sum<uint32_t, kThreads>(c, smem, &total);
+  uint32_t u = blk_base + block_exclusive_sum<uint32_t, kThreads>(c, smem, &total);
   // u = number of runs that begin before j0
   if (j0 < n) {
 #pragma unroll
@@ -282,7 +306,11 @@ struct RowVec<1> {
   static __device__ __forceinline__ type zero() { return 0.f; }
 };
 
-constexpr int kSegUnroll = 8;
+constexpr int kChunk = 32;       // sorted positions per lane group
+constexpr int kMinGroup = 4;     // lanes per group: power of two in [4, 64]
+constexpr int kMaxGroups = kThreads / kMinGroup;
+constexpr int kSegUnroll = 16;   // row loads in flight per lane
+constexpr uint32_t kNoRun = 0xffffffffu;
 
 struct SegArgs {
   const float* grad;
@@ -292,78 +320,150 @@ struct SegArgs {
   const int64_t* num_unique;
   float* sums;
   int64_t* cnts;
-  float* partial;  // [2 * nchunks][dim]
+  float* partial;  // [2 * nblocks][dim]: head and tail partial row of every block
   int64_t n;
   int64_t dim;
-  int chunk;       // R: sorted positions per lane group
-  int group;       // lanes per group (power of two <= 64)
+  int group;       // lanes per group
   int col_tiles;   // ceil(dim / (group * VEC))
 };
 
-// FAST, kernel 1: one lane group per chunk of R consecutive sorted positions.
+// FAST, kernel 1.  A block covers (kThreads / group) * kChunk consecutive sorted positions.
 template <int VEC>
 __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
   typedef typename RowVec<VEC>::type V;
-  const int64_t gtid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  const int64_t chunk_id = gtid / a.group;
-  const int gl = static_cast<int>(gtid & (a.group - 1));
-  const int64_t j0 = chunk_id * a.chunk;
-  if (j0 >= a.n) return;
-  const int64_t j1 = (j0 + a.chunk < a.n) ? j0 + a.chunk : a.n;
-  const uint32_t first_run = a.seg_of[j0];
+  __shared__ uint32_t s_perm[kMaxGroups * kChunk];
+  __shared__ uint32_t s_seg[kMaxGroups * kChunk + 2];   // s_seg[1 + t] = run of position B0 + t
+  __shared__ V s_part[kThreads * 2];                    // [group][first|last][lane]
+  __shared__ uint32_t s_first[kMaxGroups], s_last[kMaxGroups];
+  __shared__ uint8_t s_flags[kMaxGroups];               // 1 head open, 2 tail open, 4 active
+
+  const int G = a.group;
+  const int ngroups = kThreads / G;
+  const int bp = ngroups * kChunk;
+  const int64_t B0 = static_cast<int64_t>(blockIdx.x) * bp;
+  for (int t = threadIdx.x; t < bp + 2; t += kThreads) {
+    const int64_t j = B0 - 1 + t;
+    s_seg[t] = (j >= 0 && j < a.n) ? a.seg_of[j] : kNoRun;
+  }
+  for (int t = threadIdx.x; t < bp; t += kThreads) {
+    const int64_t j = B0 + t;
+    s_perm[t] = j < a.n ? a.perm[j] : 0u;
+  }
+  __syncthreads();
+
+  const int g = threadIdx.x / G;
+  const int gl = threadIdx.x & (G - 1);
+  const int t0 = g * kChunk;                       // block-relative first position of the group
+  const int64_t left = a.n - (B0 + t0);
+  const int len = left >= kChunk ? kChunk : (left > 0 ? static_cast<int>(left) : 0);
+  const bool active = len > 0;
+  const uint32_t first_run = s_seg[1 + t0];
+  const uint32_t last_run = active ? s_seg[t0 + len] : kNoRun;
+  const bool head_open = active && s_seg[t0] == first_run;
+  const bool tail_open = active && s_seg[1 + t0 + len] == last_run;
+  if (gl == 0) {
+    s_first[g] = first_run;
+    s_last[g] = last_run;
+    s_flags[g] = (head_open ? 1 : 0) | (tail_open ? 2 : 0) | (active ? 4 : 0);
+  }
 
   for (int ct = 0; ct < a.col_tiles; ++ct) {
-    const int64_t col = (static_cast<int64_t>(ct) * a.group + gl) * VEC;
+    const int64_t col = (static_cast<int64_t>(ct) * G + gl) * VEC;
     const bool col_ok = col < a.dim;
     V acc = RowVec<VEC>::zero();
     uint32_t cur = first_run;
-    for (int64_t jj = j0; jj < j1; jj += kSegUnroll) {
-      uint32_t seg[kSegUnroll];
+    for (int tt = 0; tt < len; tt += kSegUnroll) {
       V row[kSegUnroll];
 #pragma unroll
       for (int k = 0; k < kSegUnroll; ++k) {
-        const int64_t j = jj + k;
-        if (j < j1) {
-          seg[k] = a.seg_of[j];
-          const int64_t p = a.perm[j];
+        if (tt + k < len) {
+          const int64_t p = s_perm[t0 + tt + k];
           row[k] = col_ok ? *reinterpret_cast<const V*>(a.grad + p * a.dim + col)
                           : RowVec<VEC>::zero();
         }
       }
 #pragma unroll
       for (int k = 0; k < kSegUnroll; ++k) {
-        if (jj + k < j1) {
-          if (seg[k] != cur) {
-            // run `cur` ends inside this chunk; it is whole unless it began before the chunk
-            float* out = (cur != first_run || a.seg_start[cur] >= j0)
-                             ? a.sums + static_cast<int64_t>(cur) * a.dim
-                             : a.partial + (2 * chunk_id) * a.dim;
-            if (col_ok) *reinterpret_cast<V*>(out + col) = acc;
+        if (tt + k < len) {
+          const uint32_t seg = s_seg[1 + t0 + tt + k];
+          if (seg != cur) {
+            // run `cur` ends inside this group: whole unless it is the first run and began earlier
+            if (cur == first_run && head_open) {
+              s_part[(g * 2 + 0) * G + gl] = acc;
+            } else if (col_ok) {
+              *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(cur) * a.dim + col) = acc;
+            }
             acc = RowVec<VEC>::zero();
-            cur = seg[k];
+            cur = seg;
           }
           acc += row[k];
         }
       }
     }
-    // last run of the chunk: whole only if it ends exactly at the chunk end and began inside
-    const bool ends_here = a.seg_start[cur + 1] <= j1;
-    const bool began_here = a.seg_start[cur] >= j0;
-    float* out;
-    if (ends_here && began_here) {
-      out = a.sums + static_cast<int64_t>(cur) * a.dim;
-    } else if (cur == first_run) {
-      out = a.partial + (2 * chunk_id) * a.dim;  // head slot
-    } else {
-      out = a.partial + (2 * chunk_id + 1) * a.dim;  // tail slot
+    if (active) {
+      // the last run of the group
+      if (cur == first_run) {
+        if (!head_open && !tail_open) {
+          if (col_ok) *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(cur) * a.dim + col) = acc;
+        } else {
+          s_part[(g * 2 + 0) * G + gl] = acc;
+        }
+      } else if (!tail_open) {
+        if (col_ok) *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(cur) * a.dim + col) = acc;
+      } else {
+        s_part[(g * 2 + 1) * G + gl] = acc;
+      }
     }
-    if (col_ok) *reinterpret_cast<V*>(out + col) = acc;
+    __syncthreads();
+    // merge, in group order, the runs that cross group borders inside this block (group 0 only)
+    if (g == 0) {
+      V carry = RowVec<VEC>::zero();
+      uint32_t carry_run = kNoRun;
+      bool carry_on = false, carry_head = false, carry_outside = false;
+      for (int gg = 0; gg < ngroups; ++gg) {
+        const uint8_t f = s_flags[gg];
+        if (!(f & 4)) break;
+        const bool fo = f & 1, to = f & 2;
+        const bool single = s_first[gg] == s_last[gg];
+        if (fo || (single && to)) {                 // the first run of group gg is not whole
+          const V part = s_part[(gg * 2 + 0) * G + gl];
+          if (fo && gg > 0) {
+            carry += part;                          // continues the run carried in from gg-1
+          } else {
+            carry = part;
+            carry_run = s_first[gg];
+            carry_head = gg == 0;
+            carry_outside = fo;
+            carry_on = true;
+          }
+          if (!(single && to)) {                    // ... and it ends inside group gg
+            float* out = (carry_head && carry_outside)
+                             ? a.partial + (2 * static_cast<int64_t>(blockIdx.x)) * a.dim
+                             : a.sums + static_cast<int64_t>(carry_run) * a.dim;
+            if (col_ok) *reinterpret_cast<V*>(out + col) = carry;
+            carry_on = false;
+          }
+        }
+        if (!single && to) {                        // the last run of group gg goes on into gg+1
+          carry = s_part[(gg * 2 + 1) * G + gl];
+          carry_run = s_last[gg];
+          carry_head = false;
+          carry_outside = false;
+          carry_on = true;
+        }
+      }
+      if (carry_on) {                               // the run goes on into the next block
+        float* out = a.partial + (2 * static_cast<int64_t>(blockIdx.x) + (carry_head ? 0 : 1)) * a.dim;
+        if (col_ok) *reinterpret_cast<V*>(out + col) = carry;
+      }
+    }
+    __syncthreads();
   }
 }
 
-// FAST, kernel 2: block c finishes the run that begins in chunk c and crosses into chunk c+1,
-// adding its partial rows in chunk order (lane groups take partials round-robin, then group 0 adds
-// the per-group sums in group order).  Also writes the occurrence counts.
+// FAST, kernel 2: block c finishes the run that begins in block c's span and crosses into the
+// next one, adding the per-block partial rows in block order (lane groups take partials
+// round-robin, then group 0 adds the per-group sums in group order).  Also writes the counts.
 template <int VEC>
 __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
   typedef typename RowVec<VEC>::type V;
@@ -373,30 +473,32 @@ __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
   if (gtid < U)
     a.cnts[gtid] = static_cast<int64_t>(a.seg_start[gtid + 1]) - static_cast<int64_t>(a.seg_start[gtid]);
 
+  const int G = a.group;
+  const int ngroups = kThreads / G;
+  const int64_t span = static_cast<int64_t>(ngroups) * kChunk;
   const int64_t c = blockIdx.x;
-  const int64_t border = (c + 1) * a.chunk;
+  const int64_t border = (c + 1) * span;
   if (border >= a.n) return;
   const uint32_t u = a.seg_of[border - 1];
   if (a.seg_of[border] != u) return;           // no run crosses this border
   const int64_t start = a.seg_start[u];
-  if (start < c * a.chunk) return;              // the run began earlier: an earlier block owns it
+  if (start < c * span) return;                 // the run began earlier: an earlier block owns it
   const int64_t end = a.seg_start[u + 1];
-  const int64_t c_last = (end - 1) / a.chunk;
+  const int64_t c_last = (end - 1) / span;
   const int64_t nparts = c_last - c + 1;
-  const int ngroups = kThreads / a.group;
-  const int g = threadIdx.x / a.group;
-  const int gl = threadIdx.x & (a.group - 1);
-  // partial row of chunk c+t: chunk c keeps it in the tail slot unless the run opens the chunk
-  const int64_t first_slot = (start == c * a.chunk) ? 2 * c : 2 * c + 1;
+  const int g = threadIdx.x / G;
+  const int gl = threadIdx.x & (G - 1);
+  // block c keeps its share in the tail slot unless the run opens the block
+  const int64_t first_slot = (start == c * span) ? 2 * c : 2 * c + 1;
 
   for (int ct = 0; ct < a.col_tiles; ++ct) {
-    const int64_t col = (static_cast<int64_t>(ct) * a.group + gl) * VEC;
+    const int64_t col = (static_cast<int64_t>(ct) * G + gl) * VEC;
     const bool col_ok = col < a.dim;
     V acc = RowVec<VEC>::zero();
-    for (int64_t t0 = g; t0 < nparts; t0 += static_cast<int64_t>(ngroups) * kSegUnroll) {
-      V row[kSegUnroll];
+    for (int64_t t0 = g; t0 < nparts; t0 += static_cast<int64_t>(ngroups) * 8) {
+      V row[8];
 #pragma unroll
-      for (int k = 0; k < kSegUnroll; ++k) {
+      for (int k = 0; k < 8; ++k) {
         const int64_t t = t0 + static_cast<int64_t>(k) * ngroups;
         if (t < nparts) {
           const int64_t slot = t == 0 ? first_slot : 2 * (c + t);
@@ -405,7 +507,7 @@ __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
         }
       }
 #pragma unroll
-      for (int k = 0; k < kSegUnroll; ++k) {
+      for (int k = 0; k < 8; ++k) {
         const int64_t t = t0 + static_cast<int64_t>(k) * ngroups;
         if (t < nparts) acc += row[k];
       }
@@ -415,7 +517,7 @@ __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
     __syncthreads();
     if (g == 0) {
       V tot = s_part[gl];
-      for (int gg = 1; gg < ngroups; ++gg) tot += s_part[gg * a.group + gl];
+      for (int gg = 1; gg < ngroups; ++gg) tot += s_part[gg * G + gl];
       if (col_ok) *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(u) * a.dim + col) = tot;
     }
   }
@@ -437,17 +539,17 @@ __global__ __launch_bounds__(kThreads) void seg_exact_kernel(SegArgs a) {
     const int64_t col = (static_cast<int64_t>(ct) * a.group + gl) * VEC;
     if (col >= a.dim) continue;
     V acc = RowVec<VEC>::zero();
-    for (int64_t jj = j0; jj < j1; jj += kSegUnroll) {
-      V row[kSegUnroll];
+    for (int64_t jj = j0; jj < j1; jj += 8) {
+      V row[8];
 #pragma unroll
-      for (int k = 0; k < kSegUnroll; ++k) {
+      for (int k = 0; k < 8; ++k) {
         if (jj + k < j1) {
           const int64_t p = a.perm[jj + k];
           row[k] = *reinterpret_cast<const V*>(a.grad + p * a.dim + col);
         }
       }
 #pragma unroll
-      for (int k = 0; k < kSegUnroll; ++k) {
+      for (int k = 0; k < 8; ++k) {
         if (jj + k < j1) acc += row[k];
       }
     }
@@ -470,46 +572,43 @@ __global__ __launch_bounds__(kThreads) void rows_div_kernel(float* __restrict__ 
 }
 
 // ---- host-side plan ----------------------------------------------------------
-constexpr int kIPT = 4;                      // keys per thread in a radix tile
-constexpr int kRadixTile = kThreads * kIPT;
-
 struct Plan {
   bool key64;
   int key_bits;
   int passes;
-  int chunk;      // R
+  int ipt;        // keys per thread in a radix tile: 4, 8 or 16
   int vec;        // 4 or 1
   int group;
   int col_tiles;
-  int64_t nblocks_radix;
+  int64_t ntiles;        // radix tiles
   int64_t nblocks_runs;
-  int64_t nchunks;
+  int64_t nblocks_seg;   // blocks of the FAST segmented sum
 };
 
 Plan make_plan(int64_t n, int64_t dim, int64_t id_bound, bool grad_aligned) {
   Plan p;
-  if (id_bound > 0 && id_bound <= (int64_t(1) << 32)) {
-    p.key64 = false;
+  const int64_t nn = n > 0 ? n : 1;
+  if (id_bound > 0) {
     p.key_bits = ilog2_ceil(static_cast<uint64_t>(id_bound));
-  } else if (id_bound > 0) {
-    p.key64 = true;  // ids are non-negative: the flipped sign bit is constant, skip it
-    p.key_bits = ilog2_ceil(static_cast<uint64_t>(id_bound));
+    p.key64 = p.key_bits > 32;  // ids are non-negative: the flipped sign bit is constant, skip it
   } else {
     p.key64 = true;
     p.key_bits = 64;
   }
   if (p.key_bits < 1) p.key_bits = 1;
   p.passes = (p.key_bits + kRadixBits - 1) / kRadixBits;
+  // every pass reads all per-tile counts in every block: keep the number of tiles moderate
+  p.ipt = 4;
+  while (p.ipt < 16 && ceil_div(nn, kThreads * p.ipt) > 512) p.ipt *= 2;
+  p.ntiles = ceil_div(nn, kThreads * p.ipt);
   p.vec = (dim % 4 == 0 && grad_aligned) ? 4 : 1;
   const int64_t lanes = (dim + p.vec - 1) / p.vec;
-  int g = 1;
+  int g = kMinGroup;
   while (g < lanes && g < 64) g <<= 1;
   p.group = g;
   p.col_tiles = static_cast<int>((lanes + g - 1) / g);
-  p.chunk = 32;
-  p.nblocks_radix = ceil_div(n > 0 ? n : 1, kRadixTile);
-  p.nblocks_runs = ceil_div(n > 0 ? n : 1, kUTile);
-  p.nchunks = ceil_div(n > 0 ? n : 1, p.chunk);
+  p.nblocks_runs = ceil_div(nn, kUTile);
+  p.nblocks_seg = ceil_div(nn, static_cast<int64_t>(kThreads / g) * kChunk);
   return p;
 }
 
@@ -518,7 +617,8 @@ struct SortWs {
   int32_t* status;
   void* keys[2];
   uint32_t* vals[2];
-  uint32_t* hist;
+  uint32_t* cnt;        // [passes][ntiles][kBins]
+  int64_t cnt_len;
   size_t bytes;
 };
 
@@ -527,7 +627,11 @@ void carve_sort(Carver& c, int64_t n, SortWs* w) {
   w->status = c.take<int32_t>(64);
   for (int i = 0; i < 2; ++i) w->keys[i] = c.take<uint64_t>(nn);  // sized for 64-bit keys
   for (int i = 0; i < 2; ++i) w->vals[i] = c.take<uint32_t>(nn);
-  w->hist = c.take<uint32_t>(kBins * ceil_div(nn, kRadixTile));
+  // sized for the most passes and the most tiles any plan for this n can have
+  w->cnt_len = static_cast<int64_t>(kMaxPasses) * ceil_div(nn, kThreads * 4) * kBins;
+  if (ceil_div(nn, kThreads * 4) > 512)
+    w->cnt_len = static_cast<int64_t>(kMaxPasses) * make_plan(nn, 1, 0, true).ntiles * kBins;
+  w->cnt = c.take<uint32_t>(w->cnt_len);
   w->bytes = c.total();
 }
 
@@ -540,61 +644,78 @@ struct Ws {
   size_t bytes;
 };
 
-Ws carve(void* ws, int64_t n, int64_t dim, const Plan& p) {
+Ws carve(void* ws, int64_t n, int64_t dim) {
   Carver c(ws);
   Ws w;
   const int64_t nn = n > 0 ? n : 1;
   carve_sort(c, n, &w.sort);
-  w.run_cnt = c.take<uint32_t>(p.nblocks_runs + 1);
+  w.run_cnt = c.take<uint32_t>(ceil_div(nn, kUTile) + 1);
   w.seg_of = c.take<uint32_t>(nn);
   w.seg_start = c.take<uint32_t>(nn + 1);
-  w.partial = c.take<float>(2 * p.nchunks * dim);
+  // at most two partial rows per block of the FAST sum; the smallest block span is 128 positions
+  w.partial = c.take<float>(2 * ceil_div(nn, (kThreads / 64) * kChunk) * dim);
   w.bytes = c.total();
   return w;
 }
 
-template <typename KeyT>
-int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
-             hipStream_t st, const void** keys_out, const uint32_t** perm_out) {
-  const dim3 grid(static_cast<unsigned>(p.nblocks_radix)), block(kThreads);
+template <typename KeyT, int IPT>
+int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
+                 hipStream_t st, const void** keys_out, const uint32_t** perm_out) {
+  const dim3 grid(static_cast<unsigned>(p.ntiles)), block(kThreads);
+  const int base = p.key_bits / p.passes, extra = p.key_bits % p.passes;
+  int bits_of[kMaxPasses], shift_of[kMaxPasses + 1];
+  shift_of[0] = 0;
+  for (int pass = 0; pass < p.passes; ++pass) {
+    bits_of[pass] = base + (pass < extra ? 1 : 0);
+    shift_of[pass + 1] = shift_of[pass] + bits_of[pass];
+  }
+  const int tile_shift = ilog2_ceil(static_cast<uint64_t>(kThreads * IPT));
+  const int cell_bits = kRadixBits + ilog2_ceil(static_cast<uint64_t>(p.ntiles)) + 1;
+  const int64_t stride = p.ntiles * kBins;
+  hipLaunchKernelGGL((radix_count0_kernel<KeyT, IPT>), grid, block, 0, st, idx, n,
+                     (1u << bits_of[0]) - 1u, w.cnt, w.cnt + stride,
+                     static_cast<int64_t>(p.passes - 1) * stride, id_bound, w.status);
+  HADES_LAUNCH_CHECK();
   const void* kin = idx;
   const uint32_t* vin = nullptr;
   int cur = 0;
-  int shift = 0;
-  const int base = p.key_bits / p.passes, extra = p.key_bits % p.passes;
   for (int pass = 0; pass < p.passes; ++pass) {
-    const int bits = base + (pass < extra ? 1 : 0);
-    const uint32_t mask = (1u << bits) - 1u;
+    const uint32_t mask = (1u << bits_of[pass]) - 1u;
     KeyT* kout = static_cast<KeyT*>(w.keys[cur]);
     uint32_t* vout = w.vals[cur];
+    const bool last = pass + 1 == p.passes;
+    uint32_t* cnt_next = last ? nullptr : w.cnt + (pass + 1) * stride;
+    const int next_shift = last ? 0 : shift_of[pass + 1];
+    const uint32_t next_mask = last ? 0u : (1u << bits_of[pass + 1]) - 1u;
     if (pass == 0) {
-      hipLaunchKernelGGL((radix_hist_kernel<KeyT, true, kIPT>), grid, block, 0, st, kin, n, shift,
-                         mask, w.hist, p.nblocks_radix, id_bound, w.status);
+      hipLaunchKernelGGL((radix_pass_kernel<KeyT, true, IPT>), grid, block, 0, st, kin, vin, n,
+                         shift_of[pass], mask, bits_of[pass], w.cnt + pass * stride, p.ntiles, kout,
+                         vout, cnt_next, next_shift, next_mask, tile_shift, cell_bits);
     } else {
-      hipLaunchKernelGGL((radix_hist_kernel<KeyT, false, kIPT>), grid, block, 0, st, kin, n, shift,
-                         mask, w.hist, p.nblocks_radix, id_bound, w.status);
-    }
-    HADES_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_u32_kernel, dim3(1), dim3(kScanThreads), 0, st, w.hist,
-                       static_cast<int64_t>(kBins) * p.nblocks_radix,
-                       static_cast<uint32_t*>(nullptr));
-    HADES_LAUNCH_CHECK();
-    if (pass == 0) {
-      hipLaunchKernelGGL((radix_scatter_kernel<KeyT, true, kIPT>), grid, block, 0, st, kin, vin, n,
-                         shift, mask, bits, w.hist, p.nblocks_radix, kout, vout);
-    } else {
-      hipLaunchKernelGGL((radix_scatter_kernel<KeyT, false, kIPT>), grid, block, 0, st, kin, vin, n,
-                         shift, mask, bits, w.hist, p.nblocks_radix, kout, vout);
+      hipLaunchKernelGGL((radix_pass_kernel<KeyT, false, IPT>), grid, block, 0, st, kin, vin, n,
+                         shift_of[pass], mask, bits_of[pass], w.cnt + pass * stride, p.ntiles, kout,
+                         vout, cnt_next, next_shift, next_mask, tile_shift, cell_bits);
     }
     HADES_LAUNCH_CHECK();
     kin = kout;
     vin = vout;
     cur ^= 1;
-    shift += bits;
   }
   *keys_out = kin;
   *perm_out = vin;
   return HADES_OK;
+}
+
+template <typename KeyT>
+int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
+             hipStream_t st, const void** keys_out, const uint32_t** perm_out) {
+  HADES_REQUIRE(p.ntiles * kBins * static_cast<int64_t>(p.passes) <= w.cnt_len,
+                "internal: radix count buffer too small");
+  switch (p.ipt) {
+    case 4: return run_sort_ipt<KeyT, 4>(idx, n, id_bound, p, w, st, keys_out, perm_out);
+    case 8: return run_sort_ipt<KeyT, 8>(idx, n, id_bound, p, w, st, keys_out, perm_out);
+    default: return run_sort_ipt<KeyT, 16>(idx, n, id_bound, p, w, st, keys_out, perm_out);
+  }
 }
 
 template <typename KeyT>
@@ -603,9 +724,6 @@ int run_runs(const void* sorted_keys, const uint32_t* perm, int64_t n, const Pla
   const KeyT* keys = static_cast<const KeyT*>(sorted_keys);
   const dim3 rgrid(static_cast<unsigned>(p.nblocks_runs)), block(kThreads);
   hipLaunchKernelGGL((run_count_kernel<KeyT>), rgrid, block, 0, st, keys, n, w.run_cnt);
-  HADES_LAUNCH_CHECK();
-  hipLaunchKernelGGL(scan_u32_kernel, dim3(1), dim3(kScanThreads), 0, st, w.run_cnt,
-                     p.nblocks_runs, static_cast<uint32_t*>(nullptr));
   HADES_LAUNCH_CHECK();
   hipLaunchKernelGGL((run_emit_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt, uids,
                      w.seg_start, w.seg_of, num_unique, inverse);
@@ -645,8 +763,7 @@ extern "C" {
 
 size_t hades_combine_workspace_bytes(int64_t n, int64_t dim) {
   if (n < 0 || dim < 1) return 0;
-  const Plan p = make_plan(n, dim, 0, true);
-  return carve(nullptr, n, dim, p).bytes;
+  return carve(nullptr, n, dim).bytes;
 }
 
 int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim, int64_t id_bound,
@@ -667,7 +784,7 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
   HADES_REQUIRE(idx && grad && uids && sums && cnts, "null pointer argument");
   const bool aligned = (align_of_ptr(grad) % 16) == 0 && (align_of_ptr(sums) % 16) == 0;
   const Plan p = make_plan(n, dim, id_bound, aligned);
-  const Ws w = carve(workspace, n, dim, p);
+  const Ws w = carve(workspace, n, dim);
   if (workspace == nullptr || workspace_bytes < w.bytes)
     return set_error(HADES_ERR_WORKSPACE, "combine workspace too small: need %zu bytes, got %zu",
                      w.bytes, workspace_bytes);
@@ -693,7 +810,6 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
   a.partial = w.partial;
   a.n = n;
   a.dim = dim;
-  a.chunk = p.chunk;
   a.group = p.group;
   a.col_tiles = p.col_tiles;
   if (mode == HADES_COMBINE_EXACT) {
@@ -705,15 +821,16 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
       hipLaunchKernelGGL((seg_exact_kernel<1>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
     HADES_LAUNCH_CHECK();
   } else {
-    const int64_t blocks = ceil_div(p.nchunks * p.group, kThreads);
-    HADES_REQUIRE(blocks < (int64_t(1) << 31), "combine: too many rows");
+    HADES_REQUIRE(p.nblocks_seg < (int64_t(1) << 31), "combine: too many rows");
+    const dim3 grid(static_cast<unsigned>(p.nblocks_seg));
     if (p.vec == 4)
-      hipLaunchKernelGGL((seg_chunk_kernel<4>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
+      hipLaunchKernelGGL((seg_chunk_kernel<4>), grid, dim3(kThreads), 0, st, a);
     else
-      hipLaunchKernelGGL((seg_chunk_kernel<1>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
+      hipLaunchKernelGGL((seg_chunk_kernel<1>), grid, dim3(kThreads), 0, st, a);
     HADES_LAUNCH_CHECK();
-    // one block per chunk; also covers every u < U <= n with a thread for the counts
-    const int64_t fblocks = p.nchunks > ceil_div(n, kThreads) ? p.nchunks : ceil_div(n, kThreads);
+    // one block per span of the chunk kernel, and at least one thread per sorted position so that
+    // every u < U <= n gets its count written
+    const int64_t fblocks = p.nblocks_seg > ceil_div(n, kThreads) ? p.nblocks_seg : ceil_div(n, kThreads);
     if (p.vec == 4)
       hipLaunchKernelGGL((seg_fixup_kernel<4>), dim3((unsigned)fblocks), dim3(kThreads), 0, st, a);
     else
