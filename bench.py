@@ -95,7 +95,7 @@ def run_gpu(args):
     def step(i, events=None):
         q, g = wl.ids[i % nb], wl.grads[i % nb]
         if events: events[0].record()
-        ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_ids, out=wl.rows_out)
+        ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_set, out=wl.rows_out)
         if events: events[1].record()
         uids, sums, cnts, nu = ops.combine_padded(q, g, id_bound=wl.N, mode=mode, workspace=ws,
                                                   out=wl.comb_out)

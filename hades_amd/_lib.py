@@ -34,16 +34,17 @@ _SIGNATURES = {
     "hades_binary_search": [_P, _P, _L, _L, _P, _L, c_int, _P],
     "hades_binary_search2": [_P, _P, _L, _P, _L, c_int, _P],
     "hades_split": [_P, c_int, _P, _L, _P, _P, _P, _P],
-    "hades_lookup_sorted": [_P, _L, _P, _L, _P, _P],
+    "hades_lookup_sorted": [_P, _L, _P, _L, _P, _P, _P],
+    "hades_hot_index_build": [_P, _L, _P, c_size_t, _P],
     "hades_split_compact": [_P, _L, _P, _P, _P, _P, _P, c_size_t, _P],
     "hades_split3_compact": [_P, c_int, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t, _P],
-    "hades_cached_fetch": [_P, _P, _P, _L, _P, _L, _P, _P, _L, c_int, _P],
+    "hades_cached_fetch": [_P, _P, _P, _L, _P, _L, _P, _P, _P, _L, c_int, _P],
     "hades_cached_fetch_loc": [_P, _P, _P, _P, _L, _P, _L, c_int, _P],
-    "hades_cached_set": [_P, _P, _P, _P, _L, _P, _L, _L, c_int, _P],
+    "hades_cached_set": [_P, _P, _P, _P, _L, _P, _L, _P, _L, c_int, _P],
     "hades_combine": [_P, _P, _L, _L, _L, c_int, _P, _P, _P, _P, _P, _P, c_size_t, _P],
     "hades_rows_div_count": [_P, _P, _P, _L, _L, c_int, _P],
-    "hades_adagrad_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, c_float, c_float, _P],
-    "hades_adam_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P,
+    "hades_adagrad_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, _P, c_float, c_float, _P],
+    "hades_adam_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P,
                           c_float, ctypes.c_double, ctypes.c_double, c_float, _P],
     "hades_hash_clear": [_P, _P, _P, _L, _L, _P],
     "hades_hash_accumulate": [_P, _P, _P, _L, _P, _P, _P, _P, _L, _L, _P, _P],
@@ -51,6 +52,7 @@ _SIGNATURES = {
 }
 _SIZE_QUERIES = {
     "hades_split_compact_workspace_bytes": [_L],
+    "hades_hot_index_bytes": [_L],
     "hades_combine_workspace_bytes": [_L, _L],
     "hades_hash_flush_workspace_bytes": [_L, _L],
 }
@@ -67,6 +69,10 @@ def load():
         raise RuntimeError(
             "%s is missing: build it with `python -m hades_amd.build` (needs hipcc). "
             "There is no CPU fallback." % LIB_PATH)
+    # torch wheels bundle their own HIP runtime (same soname as the system one).  It has to be in
+    # the process before this library is opened, so that both bind to ONE runtime and torch's
+    # streams and allocations mean something to these kernels; the other order gives two runtimes.
+    import torch  # noqa: F401
     lib = ctypes.CDLL(LIB_PATH)
     lib.hades_last_error.restype = c_char_p
     lib.hades_last_error.argtypes = []

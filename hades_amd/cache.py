@@ -42,6 +42,7 @@ class EmbCache:
         if hot_ids.numel() > 1:
             assert bool((hot_ids[1:] > hot_ids[:-1]).all()), "hot_ids must be ascending and unique"
         self.hot_ids = hot_ids.to(self.device)
+        self.hot_set = ops.HotSet(self.hot_ids)
         self.hot = []
         cpu_ids = hot_ids.cpu()
         for t in self.cold:
@@ -64,7 +65,7 @@ class EmbCache:
 
     # -- the operators ---------------------------------------------------------
     def lookup(self, ids):
-        return ops.lookup(ids, self.hot_ids)
+        return ops.lookup(ids, self.hot_set)
 
     def split(self, ids):
         """(hot_mask, hot_pos, cold_pos) of a query batch; one host synchronisation."""
@@ -74,10 +75,10 @@ class EmbCache:
         if self._count_hit:
             self._hit_num += int((self.lookup(ids) >= 0).sum().item())
             self._lookup_num += ids.numel()
-        return ops.cached_fetch(self.cold[table], self.hot[table], ids, self.hot_ids, out=out)
+        return ops.cached_fetch(self.cold[table], self.hot[table], ids, self.hot_set, out=out)
 
     def cached_set(self, ids, rows, table=0):
-        ops.cached_set(rows, self.cold[table], self.hot[table], ids, self.hot_ids)
+        ops.cached_set(rows, self.cold[table], self.hot[table], ids, self.hot_set)
 
     def __getitem__(self, ids):
         return tuple(self.cached_fetch(ids, k) for k in range(len(self.cold)))

@@ -113,35 +113,50 @@ __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
   __shared__ uint32_t s_cnt[kWaves][kBins];
   __shared__ uint32_t s_glob[kBins];
   __shared__ uint32_t s_scan[kWaves + 1];
+  __shared__ uint32_t s_pre[kWaves][kBins];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  for (int d = threadIdx.x; d < kWaves * kBins; d += kThreads) (&s_cnt[0][0])[d] = 0;
 
   // global offset of (digit, this tile): all keys with a smaller digit, plus the keys with this
   // digit in the tiles before this one.  Thread d owns digit d (kThreads == kBins).
+  // The column sums are latency-bound: wave w takes the tiles t = w (mod kWaves), lane l the four
+  // digits 4l..4l+3 of a tile row as one 16-byte load, eight rows in flight.
   {
-    const int d = threadIdx.x;
-    uint32_t tot = 0, pre = 0;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     const int64_t me = blockIdx.x;
-    int64_t t = 0;
-    for (; t + 8 <= ntiles; t += 8) {
-      uint32_t h[8];
-#pragma unroll
-      for (int k = 0; k < 8; ++k) h[k] = cnt_cur[(t + k) * kBins + d];
+    u32x4 tot4 = {0, 0, 0, 0}, pre4 = {0, 0, 0, 0};
+    for (int64_t t = wave; t < ntiles; t += kWaves * 8) {
+      u32x4 h[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
-        tot += h[k];
-        pre += (t + k < me) ? h[k] : 0u;
+        const int64_t tt = t + static_cast<int64_t>(k) * kWaves;
+        h[k] = tt < ntiles ? reinterpret_cast<const u32x4*>(cnt_cur + tt * kBins)[lane]
+                           : u32x4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int64_t tt = t + static_cast<int64_t>(k) * kWaves;
+        tot4 += h[k];
+        if (tt < me) pre4 += h[k];
       }
     }
-    for (; t < ntiles; ++t) {
-      const uint32_t h = cnt_cur[t * kBins + d];
-      tot += h;
-      pre += (t < me) ? h : 0u;
+    // s_cnt doubles as scratch here: rows 0..3 hold the per-wave totals; the per-wave prefixes
+    // go to s_pre.  Both are folded over the waves by the thread that owns the digit.
+    reinterpret_cast<u32x4*>(&s_cnt[wave][0])[lane] = tot4;
+    reinterpret_cast<u32x4*>(&s_pre[wave][0])[lane] = pre4;
+    __syncthreads();
+    const int d = threadIdx.x;
+    uint32_t tot = 0, pre = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      tot += s_cnt[w][d];
+      pre += s_pre[w][d];
     }
     uint32_t total;
     const uint32_t base = block_exclusive_sum<uint32_t, kThreads>(tot, s_scan, &total);
     s_glob[d] = base + pre;
+    __syncthreads();
+    for (int i = threadIdx.x; i < kWaves * kBins; i += kThreads) (&s_cnt[0][0])[i] = 0;
   }
   __syncthreads();
 
@@ -672,7 +687,7 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
   const int tile_shift = ilog2_ceil(static_cast<uint64_t>(kThreads * IPT));
   const int cell_bits = kRadixBits + ilog2_ceil(static_cast<uint64_t>(p.ntiles)) + 1;
   const int64_t stride = p.ntiles * kBins;
-  hipLaunchKernelGGL((radix_count0_kernel<KeyT, IPT>), grid, block, 0, st, idx, n,
+  HADES_LAUNCH((radix_count0_kernel<KeyT, IPT>), grid, block, 0, st, idx, n,
                      (1u << bits_of[0]) - 1u, w.cnt, w.cnt + stride,
                      static_cast<int64_t>(p.passes - 1) * stride, id_bound, w.status);
   HADES_LAUNCH_CHECK();
@@ -688,11 +703,11 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
     const int next_shift = last ? 0 : shift_of[pass + 1];
     const uint32_t next_mask = last ? 0u : (1u << bits_of[pass + 1]) - 1u;
     if (pass == 0) {
-      hipLaunchKernelGGL((radix_pass_kernel<KeyT, true, IPT>), grid, block, 0, st, kin, vin, n,
+      HADES_LAUNCH((radix_pass_kernel<KeyT, true, IPT>), grid, block, 0, st, kin, vin, n,
                          shift_of[pass], mask, bits_of[pass], w.cnt + pass * stride, p.ntiles, kout,
                          vout, cnt_next, next_shift, next_mask, tile_shift, cell_bits);
     } else {
-      hipLaunchKernelGGL((radix_pass_kernel<KeyT, false, IPT>), grid, block, 0, st, kin, vin, n,
+      HADES_LAUNCH((radix_pass_kernel<KeyT, false, IPT>), grid, block, 0, st, kin, vin, n,
                          shift_of[pass], mask, bits_of[pass], w.cnt + pass * stride, p.ntiles, kout,
                          vout, cnt_next, next_shift, next_mask, tile_shift, cell_bits);
     }
@@ -723,9 +738,9 @@ int run_runs(const void* sorted_keys, const uint32_t* perm, int64_t n, const Pla
              int64_t* uids, int64_t* num_unique, int32_t* inverse, hipStream_t st) {
   const KeyT* keys = static_cast<const KeyT*>(sorted_keys);
   const dim3 rgrid(static_cast<unsigned>(p.nblocks_runs)), block(kThreads);
-  hipLaunchKernelGGL((run_count_kernel<KeyT>), rgrid, block, 0, st, keys, n, w.run_cnt);
+  HADES_LAUNCH((run_count_kernel<KeyT>), rgrid, block, 0, st, keys, n, w.run_cnt);
   HADES_LAUNCH_CHECK();
-  hipLaunchKernelGGL((run_emit_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt, uids,
+  HADES_LAUNCH((run_emit_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt, uids,
                      w.seg_start, w.seg_of, num_unique, inverse);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
@@ -777,7 +792,7 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
   HADES_REQUIRE(num_unique != nullptr, "num_unique must not be null");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (n == 0) {
-    hipLaunchKernelGGL(set_i64_kernel, dim3(1), dim3(64), 0, st, num_unique, int64_t(0));
+    HADES_LAUNCH(set_i64_kernel, dim3(1), dim3(64), 0, st, num_unique, int64_t(0));
     HADES_LAUNCH_CHECK();
     return HADES_OK;
   }
@@ -816,25 +831,25 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
     const int64_t blocks = ceil_div(n * p.group, kThreads);
     HADES_REQUIRE(blocks < (int64_t(1) << 31), "combine: too many rows");
     if (p.vec == 4)
-      hipLaunchKernelGGL((seg_exact_kernel<4>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
+      HADES_LAUNCH((seg_exact_kernel<4>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
     else
-      hipLaunchKernelGGL((seg_exact_kernel<1>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
+      HADES_LAUNCH((seg_exact_kernel<1>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
     HADES_LAUNCH_CHECK();
   } else {
     HADES_REQUIRE(p.nblocks_seg < (int64_t(1) << 31), "combine: too many rows");
     const dim3 grid(static_cast<unsigned>(p.nblocks_seg));
     if (p.vec == 4)
-      hipLaunchKernelGGL((seg_chunk_kernel<4>), grid, dim3(kThreads), 0, st, a);
+      HADES_LAUNCH((seg_chunk_kernel<4>), grid, dim3(kThreads), 0, st, a);
     else
-      hipLaunchKernelGGL((seg_chunk_kernel<1>), grid, dim3(kThreads), 0, st, a);
+      HADES_LAUNCH((seg_chunk_kernel<1>), grid, dim3(kThreads), 0, st, a);
     HADES_LAUNCH_CHECK();
     // one block per span of the chunk kernel, and at least one thread per sorted position so that
     // every u < U <= n gets its count written
     const int64_t fblocks = p.nblocks_seg > ceil_div(n, kThreads) ? p.nblocks_seg : ceil_div(n, kThreads);
     if (p.vec == 4)
-      hipLaunchKernelGGL((seg_fixup_kernel<4>), dim3((unsigned)fblocks), dim3(kThreads), 0, st, a);
+      HADES_LAUNCH((seg_fixup_kernel<4>), dim3((unsigned)fblocks), dim3(kThreads), 0, st, a);
     else
-      hipLaunchKernelGGL((seg_fixup_kernel<1>), dim3((unsigned)fblocks), dim3(kThreads), 0, st, a);
+      HADES_LAUNCH((seg_fixup_kernel<1>), dim3((unsigned)fblocks), dim3(kThreads), 0, st, a);
     HADES_LAUNCH_CHECK();
   }
   return HADES_OK;
@@ -847,7 +862,7 @@ int hades_rows_div_count(float* sums, const int64_t* cnts, const int64_t* num_un
   HADES_REQUIRE(sums && cnts, "null pointer argument");
   int64_t blocks = ceil_div(max_rows * dim, kThreads);
   if (blocks > 65536) blocks = 65536;
-  hipLaunchKernelGGL(rows_div_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
+  HADES_LAUNCH(rows_div_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
                      static_cast<hipStream_t>(stream), sums, cnts, num_unique, max_rows, dim,
                      one_plus);
   HADES_LAUNCH_CHECK();

@@ -30,7 +30,15 @@ int set_error(int code, const char* fmt, ...);
     if (!(cond)) return ::hades::set_error(HADES_ERR_ARG, __VA_ARGS__);              \
   } while (0)
 
-// Launch-error check after every <<<>>> (the reference never checks its launches).
+// Kernel launch with an error check (the reference never checks its launches).  The error state
+// is read once before the launch so that a stale error left by an earlier, unrelated HIP call of
+// the process is not blamed on this kernel.
+#define HADES_LAUNCH(...)                     \
+  do {                                        \
+    (void)hipGetLastError();                  \
+    hipLaunchKernelGGL(__VA_ARGS__);          \
+    HADES_HIP_TRY(hipGetLastError());         \
+  } while (0)
 #define HADES_LAUNCH_CHECK() HADES_HIP_TRY(hipGetLastError())
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -85,6 +93,33 @@ __device__ __forceinline__ int64_t lookup_slot_dev(const int64_t* __restrict__ a
   int64_t pos = upper_bound_dev<int64_t>(a, n, v);
   return (pos > 0 && a[pos - 1] == v) ? pos - 1 : int64_t(-1);
 }
+
+// The hot-ID set as the kernels see it: the ascending ids, and optionally a bucket index over
+// them.  Index layout (uint32 words): [0] shift, [1] log2(buckets), [2] valid, [3] unused, then
+// table[buckets + 1] with table[b] = first position whose id >= (b << shift).  A lookup is then
+// one table read (two adjacent words) plus a search over the handful of ids of one bucket,
+// instead of log2(n) dependent probes.
+constexpr int kHotIndexHeader = 4;
+struct HotSet {
+  const int64_t* sorted;
+  int64_t n;
+  const uint32_t* index;  // may be null
+
+  __device__ __forceinline__ int64_t slot(int64_t v) const {
+    if (index == nullptr || index[2] == 0u) return lookup_slot_dev(sorted, n, v);
+    if (v < 0) return -1;
+    const uint64_t b = static_cast<uint64_t>(v) >> index[0];
+    if (b >> index[1]) return -1;  // beyond the largest hot id
+    int64_t lo = index[kHotIndexHeader + b], hi = index[kHotIndexHeader + b + 1];
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      const int64_t x = sorted[mid];
+      if (x == v) return mid;
+      if (x < v) lo = mid + 1; else hi = mid;
+    }
+    return -1;
+  }
+};
 
 // wave64 inclusive prefix sum of a 32-bit value over the lanes of a wavefront
 __device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t v) {

@@ -221,7 +221,7 @@ int hades_hash_clear(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slot
   HADES_REQUIRE(dim >= 1 && keys && accum && cnt, "bad argument");
   int64_t blocks = ceil_div(num_slots * dim, kThreads * 8);
   if (blocks > 65536) blocks = 65536;
-  hipLaunchKernelGGL(hash_clear_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
+  HADES_LAUNCH(hash_clear_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
                      static_cast<hipStream_t>(stream), keys, accum, cnt, num_slots, dim);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
@@ -242,9 +242,9 @@ int hades_hash_accumulate(int64_t* keys, float* accum, int64_t* cnt, int64_t num
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec4 = dim % 4 == 0 && (align_of_ptr(accum) % 16) == 0 && (align_of_ptr(grad) % 16) == 0;
   if (vec4)
-    hipLaunchKernelGGL((hash_accumulate_kernel<4>), grid, block, 0, st, a);
+    HADES_LAUNCH((hash_accumulate_kernel<4>), grid, block, 0, st, a);
   else
-    hipLaunchKernelGGL((hash_accumulate_kernel<1>), grid, block, 0, st, a);
+    HADES_LAUNCH((hash_accumulate_kernel<1>), grid, block, 0, st, a);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }
@@ -274,7 +274,7 @@ int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slot
                              w.compact_bytes, st);
   if (rc != HADES_OK) return rc;
   const int64_t pad = id_bound > 0 ? id_bound : INT64_MAX;
-  hipLaunchKernelGGL(flush_gather_ids_kernel, dim3((unsigned)ceil_div(cap, kThreads)),
+  HADES_LAUNCH(flush_gather_ids_kernel, dim3((unsigned)ceil_div(cap, kThreads)),
                      dim3(kThreads), 0, st, keys, w.live_pos, w.live_count, cap, pad, w.ids, num_out,
                      status);
   HADES_LAUNCH_CHECK();
@@ -285,9 +285,9 @@ int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slot
   const dim3 grid(static_cast<unsigned>(ceil_div(cap, kRows))), block(kThreads);
   const bool vec4 = dim % 4 == 0 && (align_of_ptr(accum) % 16) == 0 && (align_of_ptr(out_sums) % 16) == 0;
   if (vec4)
-    hipLaunchKernelGGL((flush_emit_kernel<4>), grid, block, 0, st, a);
+    HADES_LAUNCH((flush_emit_kernel<4>), grid, block, 0, st, a);
   else
-    hipLaunchKernelGGL((flush_emit_kernel<1>), grid, block, 0, st, a);
+    HADES_LAUNCH((flush_emit_kernel<1>), grid, block, 0, st, a);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }

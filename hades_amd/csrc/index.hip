@@ -38,12 +38,53 @@ __global__ __launch_bounds__(kThreads) void upper_bound_kernel(const T* __restri
 }
 
 __global__ __launch_bounds__(kThreads) void lookup_sorted_kernel(const int64_t* __restrict__ q,
-                                                                int64_t n,
-                                                                const int64_t* __restrict__ sorted,
-                                                                int64_t num_hot,
+                                                                int64_t n, HotSet hs,
                                                                 int64_t* __restrict__ loc) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i < n) loc[i] = lookup_slot_dev(sorted, num_hot, q[i]);
+  if (i < n) loc[i] = hs.slot(q[i]);
+}
+
+// ---- bucket index over the sorted hot set ------------------------------------
+// header: shift such that (largest id >> shift) < buckets; valid only for non-negative ids
+__global__ void hot_index_header_kernel(const int64_t* __restrict__ sorted, int64_t num_hot,
+                                        int buckets_log2, uint32_t* __restrict__ index) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  uint32_t shift = 0, valid = 0;
+  if (num_hot > 0 && num_hot < (int64_t(1) << 32) && sorted[0] >= 0) {
+    const uint64_t mx = static_cast<uint64_t>(sorted[num_hot - 1]);
+    const int bits = mx == 0 ? 1 : 64 - __clzll(static_cast<long long>(mx));
+    shift = bits > buckets_log2 ? static_cast<uint32_t>(bits - buckets_log2) : 0u;
+    valid = 1;
+  }
+  index[0] = shift;
+  index[1] = static_cast<uint32_t>(buckets_log2);
+  index[2] = valid;
+  index[3] = 0;
+}
+
+__global__ __launch_bounds__(kThreads) void hot_index_table_kernel(const int64_t* __restrict__ sorted,
+                                                                  int64_t num_hot,
+                                                                  uint32_t* __restrict__ index) {
+  const int64_t b = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t buckets = int64_t(1) << index[1];
+  if (b > buckets) return;
+  if (index[2] == 0u) {
+    index[kHotIndexHeader + b] = 0;
+    return;
+  }
+  // first position whose id >= (b << shift): ids are >= 0, so this is upper_bound(key - 1)
+  // (the last entry closes the last bucket: every id is below buckets << shift)
+  const int64_t key = static_cast<int64_t>(static_cast<uint64_t>(b) << index[0]);
+  int64_t pos;
+  if (b == buckets) pos = num_hot;
+  else if (key <= 0) pos = 0;
+  else pos = upper_bound_dev<int64_t>(sorted, num_hot, key - 1);
+  index[kHotIndexHeader + b] = static_cast<uint32_t>(pos);
+}
+
+int hot_index_buckets_log2(int64_t num_hot) {
+  int l = ilog2_ceil(static_cast<uint64_t>(num_hot > 1 ? num_hot : 1));
+  return l > 30 ? 30 : l;
 }
 
 // ---- split: three masks from the int8 class table --------------------------
@@ -234,13 +275,13 @@ int run_compact(const Classifier& cf, int64_t n, int num_classes, const CompactO
   HADES_REQUIRE((align_of_ptr(workspace) & 255) == 0, "workspace must be 256-byte aligned");
   const int64_t nblocks = ceil_div(n > 0 ? n : 1, kTile);
   HADES_REQUIRE(nblocks < (int64_t(1) << 31), "n too large");
-  hipLaunchKernelGGL((classify_count_kernel<Classifier>), dim3((unsigned)nblocks), dim3(kThreads), 0,
+  HADES_LAUNCH((classify_count_kernel<Classifier>), dim3((unsigned)nblocks), dim3(kThreads), 0,
                      st, cf, n, w.cls, w.blk_cnt, nblocks);
   HADES_LAUNCH_CHECK();
-  hipLaunchKernelGGL(block_prefix_kernel, dim3(1), dim3(kThreads), 0, st, w.blk_cnt, w.blk_off,
+  HADES_LAUNCH(block_prefix_kernel, dim3(1), dim3(kThreads), 0, st, w.blk_cnt, w.blk_off,
                      nblocks, num_classes, counts);
   HADES_LAUNCH_CHECK();
-  hipLaunchKernelGGL(compact_kernel, dim3((unsigned)nblocks), dim3(kThreads), 0, st, w.cls,
+  HADES_LAUNCH(compact_kernel, dim3((unsigned)nblocks), dim3(kThreads), 0, st, w.cls,
                      w.blk_off, nblocks, n, num_classes, out);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
@@ -293,7 +334,7 @@ int hades_reminder(const void* in, int64_t local_num_gpus, void* out, int64_t n,
   HADES_REQUIRE(ceil_div(n, kThreads) < (int64_t(1) << 31), "n too large");
   return dispatch_itype(itype, [&](auto tag) {
     using T = decltype(tag);
-    hipLaunchKernelGGL((reminder_kernel<T>), dim3(grid_1d(n)), dim3(kThreads), 0,
+    HADES_LAUNCH((reminder_kernel<T>), dim3(grid_1d(n)), dim3(kThreads), 0,
                        static_cast<hipStream_t>(stream), static_cast<const T*>(in),
                        static_cast<T>(local_num_gpus), static_cast<T*>(out), n);
     HADES_LAUNCH_CHECK();
@@ -310,7 +351,7 @@ int hades_binary_search(const void* in, const void* range_partition, int64_t num
   HADES_REQUIRE(ceil_div(n, kThreads) < (int64_t(1) << 31), "n too large");
   return dispatch_itype(itype, [&](auto tag) {
     using T = decltype(tag);
-    hipLaunchKernelGGL((owner_rank_kernel<T>), dim3(grid_1d(n)), dim3(kThreads), 0,
+    HADES_LAUNCH((owner_rank_kernel<T>), dim3(grid_1d(n)), dim3(kThreads), 0,
                        static_cast<hipStream_t>(stream), static_cast<const T*>(in),
                        static_cast<const T*>(range_partition), num_part,
                        static_cast<T>(local_num_gpus), static_cast<T*>(out), n);
@@ -327,7 +368,7 @@ int hades_binary_search2(const void* in, const void* range, int64_t num_part, vo
   HADES_REQUIRE(ceil_div(n, kThreads) < (int64_t(1) << 31), "n too large");
   return dispatch_itype(itype, [&](auto tag) {
     using T = decltype(tag);
-    hipLaunchKernelGGL((upper_bound_kernel<T>), dim3(grid_1d(n)), dim3(kThreads), 0,
+    HADES_LAUNCH((upper_bound_kernel<T>), dim3(grid_1d(n)), dim3(kThreads), 0,
                        static_cast<hipStream_t>(stream), static_cast<const T*>(in),
                        static_cast<const T*>(range), num_part, static_cast<T*>(out), n);
     HADES_LAUNCH_CHECK();
@@ -336,13 +377,41 @@ int hades_binary_search2(const void* in, const void* range, int64_t num_part, vo
 }
 
 int hades_lookup_sorted(const int64_t* q, int64_t n, const int64_t* sorted_hot, int64_t num_hot,
-                        int64_t* loc, void* stream) {
+                        const void* hot_index, int64_t* loc, void* stream) {
   HADES_REQUIRE(n >= 0 && num_hot >= 0, "n and num_hot must be >= 0");
   if (n == 0) return HADES_OK;
   HADES_REQUIRE(q && loc && (num_hot == 0 || sorted_hot), "null pointer argument");
   HADES_REQUIRE(ceil_div(n, kThreads) < (int64_t(1) << 31), "n too large");
-  hipLaunchKernelGGL(lookup_sorted_kernel, dim3(grid_1d(n)), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(stream), q, n, sorted_hot, num_hot, loc);
+  HADES_LAUNCH(lookup_sorted_kernel, dim3(grid_1d(n)), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), q, n,
+                     HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}, loc);
+  HADES_LAUNCH_CHECK();
+  return HADES_OK;
+}
+
+size_t hades_hot_index_bytes(int64_t num_hot) {
+  if (num_hot < 0) return 0;
+  const int64_t buckets = int64_t(1) << hot_index_buckets_log2(num_hot);
+  return static_cast<size_t>(kHotIndexHeader + buckets + 1) * sizeof(uint32_t);
+}
+
+int hades_hot_index_build(const int64_t* sorted_hot, int64_t num_hot, void* hot_index,
+                          size_t hot_index_bytes, void* stream) {
+  HADES_REQUIRE(num_hot >= 0 && (num_hot == 0 || sorted_hot), "bad hot set");
+  HADES_REQUIRE(hot_index != nullptr && (align_of_ptr(hot_index) % 16) == 0,
+                "hot_index must be a 16-byte aligned device buffer");
+  if (hot_index_bytes < hades_hot_index_bytes(num_hot))
+    return set_error(HADES_ERR_WORKSPACE, "hot index buffer too small: need %zu bytes, got %zu",
+                     hades_hot_index_bytes(num_hot), hot_index_bytes);
+  const int l2 = hot_index_buckets_log2(num_hot);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t* index = static_cast<uint32_t*>(hot_index);
+  HADES_LAUNCH(hot_index_header_kernel, dim3(1), dim3(64), 0, st, sorted_hot, num_hot, l2,
+                     index);
+  HADES_LAUNCH_CHECK();
+  const int64_t entries = (int64_t(1) << l2) + 1;
+  HADES_LAUNCH(hot_index_table_kernel, dim3(grid_1d(entries)), dim3(kThreads), 0, st,
+                     sorted_hot, num_hot, index);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }
@@ -357,7 +426,7 @@ int hades_split(const void* ids, int id_type, const int8_t* class_table, int64_t
   HADES_REQUIRE(ceil_div(n, kThreads) < (int64_t(1) << 31), "n too large");
   return dispatch_split_id(id_type, [&](auto tag) {
     using T = decltype(tag);
-    hipLaunchKernelGGL((split_masks_kernel<T>), dim3(grid_1d(n)), dim3(kThreads), 0,
+    HADES_LAUNCH((split_masks_kernel<T>), dim3(grid_1d(n)), dim3(kThreads), 0,
                        static_cast<hipStream_t>(stream), static_cast<const T*>(ids), class_table, n,
                        local_mask, remote_hot_mask, remote_cold_mask);
     HADES_LAUNCH_CHECK();

@@ -78,11 +78,11 @@ struct AddrSetMap {
 };
 // loc = lookup(q[i]) in the sorted hot set; dst[i] = loc >= 0 ? hot[loc] : cold[q[i]]
 struct AddrFetchSorted {
-  const char* cold; const char* hot; const int64_t* q; const int64_t* sorted; int64_t num_hot;
+  const char* cold; const char* hot; const int64_t* q; HotSet hs;
   char* dst; int64_t* loc_out; int64_t row_bytes;
   __device__ __forceinline__ void operator()(int64_t i, const char*& s, char*& d) const {
     int64_t id = q[i];
-    int64_t loc = lookup_slot_dev(sorted, num_hot, id);
+    int64_t loc = hs.slot(id);
     if (loc_out) loc_out[i] = loc;
     s = (loc >= 0) ? hot + loc * row_bytes : cold + id * row_bytes;
     d = dst + i * row_bytes;
@@ -100,11 +100,10 @@ struct AddrFetchLoc {
 };
 // (loc >= 0 ? hot[loc] : cold[q[i]]) = src[i]
 struct AddrSetSorted {
-  const char* src; char* cold; char* hot; const int64_t* q; const int64_t* sorted;
-  int64_t num_hot; int64_t row_bytes;
+  const char* src; char* cold; char* hot; const int64_t* q; HotSet hs; int64_t row_bytes;
   __device__ __forceinline__ void operator()(int64_t i, const char*& s, char*& d) const {
     int64_t id = q[i];
-    int64_t loc = lookup_slot_dev(sorted, num_hot, id);
+    int64_t loc = hs.slot(id);
     s = src + i * row_bytes;
     d = (loc >= 0) ? hot + loc * row_bytes : cold + id * row_bytes;
   }
@@ -174,11 +173,11 @@ int launch_mover(const Addr& addr, int64_t n, int64_t row_bytes, int vec, hipStr
   HADES_REQUIRE(blocks < (int64_t(1) << 31), "too many rows: %lld", (long long)n);
   dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
   if (vec == 16) {
-    hipLaunchKernelGGL((row_move_kernel<u32x4, Addr>), grid, block, 0, stream, addr, n, cpr, shift);
+    HADES_LAUNCH((row_move_kernel<u32x4, Addr>), grid, block, 0, stream, addr, n, cpr, shift);
   } else if (vec == 8) {
-    hipLaunchKernelGGL((row_move_kernel<u32x2, Addr>), grid, block, 0, stream, addr, n, cpr, shift);
+    HADES_LAUNCH((row_move_kernel<u32x2, Addr>), grid, block, 0, stream, addr, n, cpr, shift);
   } else {
-    hipLaunchKernelGGL((row_move_kernel<uint32_t, Addr>), grid, block, 0, stream, addr, n, cpr, shift);
+    HADES_LAUNCH((row_move_kernel<uint32_t, Addr>), grid, block, 0, stream, addr, n, cpr, shift);
   }
   HADES_LAUNCH_CHECK();
   return HADES_OK;
@@ -294,14 +293,15 @@ int hades_set_with_cache(const void* src, void* cpu_dst, void* gpu_dst, const vo
 }
 
 int hades_cached_fetch(const void* cold_src, const void* hot_src, const int64_t* q, int64_t n,
-                       const int64_t* sorted_hot, int64_t num_hot, void* dst, int64_t* loc_out,
-                       int64_t dim, int dtype, void* stream) {
+                       const int64_t* sorted_hot, int64_t num_hot, const void* hot_index, void* dst,
+                       int64_t* loc_out, int64_t dim, int dtype, void* stream) {
   HADES_ROW_ARGS_CHECK();
   HADES_REQUIRE(num_hot >= 0, "num_hot must be >= 0");
   if (n == 0) return HADES_OK;
   HADES_REQUIRE(q && dst && (num_hot == 0 || (sorted_hot && hot_src)), "null pointer argument");
   const int vec = pick_vec(row_bytes, {cold_src, hot_src, dst});
-  AddrFetchSorted a{(const char*)cold_src, (const char*)hot_src, q, sorted_hot, num_hot,
+  AddrFetchSorted a{(const char*)cold_src, (const char*)hot_src, q,
+                    HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)},
                     (char*)dst, loc_out, row_bytes};
   return launch_mover(a, n, row_bytes, vec, static_cast<hipStream_t>(stream));
 }
@@ -318,15 +318,15 @@ int hades_cached_fetch_loc(const void* cold_src, const void* hot_src, const int6
 }
 
 int hades_cached_set(const void* src, void* cold_dst, void* hot_dst, const int64_t* q, int64_t n,
-                     const int64_t* sorted_hot, int64_t num_hot, int64_t dim, int dtype,
-                     void* stream) {
+                     const int64_t* sorted_hot, int64_t num_hot, const void* hot_index, int64_t dim,
+                     int dtype, void* stream) {
   HADES_ROW_ARGS_CHECK();
   HADES_REQUIRE(num_hot >= 0, "num_hot must be >= 0");
   if (n == 0) return HADES_OK;
   HADES_REQUIRE(src && q && (num_hot == 0 || (sorted_hot && hot_dst)), "null pointer argument");
   const int vec = pick_vec(row_bytes, {src, cold_dst, hot_dst});
-  AddrSetSorted a{(const char*)src, (char*)cold_dst, (char*)hot_dst, q, sorted_hot, num_hot,
-                  row_bytes};
+  AddrSetSorted a{(const char*)src, (char*)cold_dst, (char*)hot_dst, q,
+                  HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}, row_bytes};
   return launch_mover(a, n, row_bytes, vec, static_cast<hipStream_t>(stream));
 }
 

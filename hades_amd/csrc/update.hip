@@ -47,8 +47,7 @@ struct RowArgs {
   const int64_t* num_unique;
   int64_t max_rows;
   int64_t dim;
-  const int64_t* sorted_hot;
-  int64_t num_hot;
+  HotSet hs;
 };
 
 struct AdagradArgs {
@@ -73,7 +72,7 @@ __device__ __forceinline__ int resolve_rows(const RowArgs& a, int64_t* s_row, ui
   const int rows_here = left >= kRows ? kRows : (left > 0 ? static_cast<int>(left) : 0);
   for (int r = threadIdx.x; r < rows_here; r += kThreads) {
     const int64_t id = a.uids[row0 + r];
-    const int64_t loc = lookup_slot_dev(a.sorted_hot, a.num_hot, id);
+    const int64_t loc = a.hs.slot(id);
     s_row[r] = loc >= 0 ? loc : id;
     s_hot[r] = loc >= 0 ? 1 : 0;
   }
@@ -212,27 +211,28 @@ extern "C" {
 
 int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                          int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,
-                         float* hot_w, float* hot_s, float* cold_w, float* cold_s, float lr,
+                         const void* hot_index, float* hot_w, float* hot_s, float* cold_w, float* cold_s, float lr,
                          float eps, void* stream) {
   int rc = check_rows(uids, grad, max_rows, dim, sorted_hot, num_hot);
   if (rc != HADES_OK) return rc;
   if (max_rows == 0) return HADES_OK;
   HADES_REQUIRE(num_hot == 0 || (hot_w && hot_s), "hot tables are null but num_hot > 0");
-  AdagradArgs a{{uids, grad, num_unique, max_rows, dim, sorted_hot, num_hot},
+  AdagradArgs a{{uids, grad, num_unique, max_rows, dim,
+              HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}},
                 hot_w, hot_s, cold_w, cold_s, lr, eps};
   const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dim % 4 == 0 && aligned16({grad, hot_w, hot_s, cold_w, cold_s}))
-    hipLaunchKernelGGL((adagrad_kernel<4>), grid, block, 0, st, a);
+    HADES_LAUNCH((adagrad_kernel<4>), grid, block, 0, st, a);
   else
-    hipLaunchKernelGGL((adagrad_kernel<1>), grid, block, 0, st, a);
+    HADES_LAUNCH((adagrad_kernel<1>), grid, block, 0, st, a);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }
 
 int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                       int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,
-                      float* hot_w, float* hot_step, float* hot_m, float* hot_v, float* cold_w,
+                      const void* hot_index, float* hot_w, float* hot_step, float* hot_m, float* hot_v, float* cold_w,
                       float* cold_step, float* cold_m, float* cold_v, float lr, double beta1,
                       double beta2, float eps, void* stream) {
   int rc = check_rows(uids, grad, max_rows, dim, sorted_hot, num_hot);
@@ -245,15 +245,16 @@ int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num
   // 1 - float(0.999) would be off by 1.3e-5 relative
   const float omb1 = static_cast<float>(1.0 - beta1);
   const float omb2 = static_cast<float>(1.0 - beta2);
-  AdamArgs a{{uids, grad, num_unique, max_rows, dim, sorted_hot, num_hot},
+  AdamArgs a{{uids, grad, num_unique, max_rows, dim,
+              HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}},
              hot_w, hot_step, hot_m, hot_v, cold_w, cold_step, cold_m, cold_v,
              lr, static_cast<float>(beta1), static_cast<float>(beta2), omb1, omb2, eps};
   const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dim % 4 == 0 && aligned16({grad, hot_w, hot_m, hot_v, cold_w, cold_m, cold_v}))
-    hipLaunchKernelGGL((adam_kernel<4>), grid, block, 0, st, a);
+    HADES_LAUNCH((adam_kernel<4>), grid, block, 0, st, a);
   else
-    hipLaunchKernelGGL((adam_kernel<1>), grid, block, 0, st, a);
+    HADES_LAUNCH((adam_kernel<1>), grid, block, 0, st, a);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }

@@ -57,13 +57,45 @@ def _ws(device, kind):
     return _default_ws[key]
 
 
-# ---- lookup -------------------------------------------------------------------
+# ---- the hot set and lookup -----------------------------------------------------
+class HotSet:
+    """The ascending, duplicate-free hot ids on the device together with the bucket index that
+    turns a lookup into one table read plus a search over a handful of ids.  Every operator that
+    takes `sorted_hot` accepts either a plain int64 tensor (binary search) or a HotSet."""
+
+    def __init__(self, sorted_hot, device=None, build_index=True):
+        ids = torch.as_tensor(sorted_hot, dtype=torch.int64)
+        if device is not None:
+            ids = ids.to(device)
+        _i64(ids, "sorted_hot")
+        self.ids = ids
+        self.index = None
+        if build_index:
+            nbytes = _lib.query("hades_hot_index_bytes", ids.numel())
+            self.index = torch.empty(nbytes // 4, dtype=torch.int32, device=ids.device)
+            _lib.call("hades_hot_index_build", _ptr(ids), ids.numel(), _ptr(self.index), nbytes,
+                      _stream())
+
+    def numel(self):
+        return self.ids.numel()
+
+
+def _hot_args(sorted_hot):
+    """(ids pointer, count, index pointer) of a HotSet, a tensor or None."""
+    if sorted_hot is None:
+        return _NULL, 0, _NULL
+    if isinstance(sorted_hot, HotSet):
+        return _ptr(sorted_hot.ids), sorted_hot.ids.numel(), _opt(sorted_hot.index)
+    _i64(sorted_hot, "sorted_hot")
+    return _ptr(sorted_hot), sorted_hot.numel(), _NULL
+
+
 def lookup(ids, sorted_hot, out=None):
-    """loc[i] = slot of ids[i] in the ascending duplicate-free `sorted_hot`, or -1."""
-    _i64(ids, "ids"); _i64(sorted_hot, "sorted_hot")
+    """loc[i] = slot of ids[i] in the ascending duplicate-free hot set, or -1."""
+    _i64(ids, "ids")
+    hp, hn, hi = _hot_args(sorted_hot)
     loc = out if out is not None else torch.empty_like(ids)
-    _lib.call("hades_lookup_sorted", _ptr(ids), ids.numel(), _ptr(sorted_hot), sorted_hot.numel(),
-              _ptr(loc), _stream())
+    _lib.call("hades_lookup_sorted", _ptr(ids), ids.numel(), hp, hn, hi, _ptr(loc), _stream())
     return loc
 
 
@@ -130,7 +162,8 @@ def cached_fetch(cold, hot, ids, sorted_hot, out=None, return_loc=False):
 
     `cold` may be a device tensor or a pinned host tensor (read zero-copy).  The lookup runs
     inside the gather kernel."""
-    _i64(ids, "ids"); _i64(sorted_hot, "sorted_hot")
+    _i64(ids, "ids")
+    hp, hn, hi = _hot_args(sorted_hot)
     _dev_or_pinned(cold, "cold"); _dev(hot, "hot")
     dim = _table_dim(cold, hot)
     n = ids.numel()
@@ -141,8 +174,8 @@ def cached_fetch(cold, hot, ids, sorted_hot, out=None, return_loc=False):
         _dev(out, "out")
         _check(tuple(out.shape) == shape and out.dtype == hot.dtype, "out has the wrong shape/dtype")
     loc = torch.empty_like(ids) if return_loc else None
-    _lib.call("hades_cached_fetch", _ptr(cold), _ptr(hot), _ptr(ids), n, _ptr(sorted_hot),
-              sorted_hot.numel(), _ptr(out), _opt(loc), dim, _dcode(hot), _stream())
+    _lib.call("hades_cached_fetch", _ptr(cold), _ptr(hot), _ptr(ids), n, hp, hn, hi, _ptr(out),
+              _opt(loc), dim, _dcode(hot), _stream())
     return (out, loc) if return_loc else out
 
 
@@ -164,12 +197,13 @@ def cached_fetch_loc(cold, hot, ids, loc, out=None):
 def cached_set(src, cold, hot, ids, sorted_hot):
     """(hot[slot] if ids[i] in sorted_hot else cold[ids[i]]) = src[i]; ids must be duplicate-free
     for a defined result."""
-    _i64(ids, "ids"); _i64(sorted_hot, "sorted_hot")
+    _i64(ids, "ids")
+    hp, hn, hi = _hot_args(sorted_hot)
     _dev(src, "src"); _dev_or_pinned(cold, "cold"); _dev(hot, "hot")
     dim = _table_dim(cold, hot, src)
     _check(src.size(0) >= ids.numel(), "src has fewer rows than ids has entries")
     _lib.call("hades_cached_set", _ptr(src), _ptr(cold), _ptr(hot), _ptr(ids), ids.numel(),
-              _ptr(sorted_hot), sorted_hot.numel(), dim, _dcode(hot), _stream())
+              hp, hn, hi, dim, _dcode(hot), _stream())
 
 
 # ---- combine ------------------------------------------------------------------
@@ -228,7 +262,7 @@ def adagrad_update_(uids, grad, hot_w, hot_s, cold_w, cold_s, sorted_hot, lr, ep
     _i64(uids, "uids"); _dev(grad, "grad")
     _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
     dim = grad.size(1)
-    nh = 0 if sorted_hot is None else sorted_hot.numel()
+    hp, hn, hi = _hot_args(sorted_hot)
     for name, t in (("hot_w", hot_w), ("hot_s", hot_s)):
         if t is not None:
             _dev(t, name)
@@ -239,7 +273,7 @@ def adagrad_update_(uids, grad, hot_w, hot_s, cold_w, cold_s, sorted_hot, lr, ep
             _check(t.dtype == torch.float32 and t.size(1) == dim, "%s: wrong dtype/width" % name)
     _check(grad.size(0) >= uids.numel(), "grad has fewer rows than uids has entries")
     _lib.call("hades_adagrad_update", _ptr(uids), _ptr(grad), _opt(num_unique), uids.numel(), dim,
-              _opt(sorted_hot), nh, _opt(hot_w), _opt(hot_s), _opt(cold_w), _opt(cold_s),
+              hp, hn, hi, _opt(hot_w), _opt(hot_s), _opt(cold_w), _opt(cold_s),
               float(lr), float(eps), _stream())
 
 
@@ -247,10 +281,10 @@ def adam_update_(uids, grad, hot, cold, sorted_hot, lr, beta1, beta2, eps, num_u
     """SparseAdam row update in place.  `hot` and `cold` are (w, step, mem, power) tuples."""
     _i64(uids, "uids"); _dev(grad, "grad")
     dim = grad.size(1)
-    nh = 0 if sorted_hot is None else sorted_hot.numel()
+    hp, hn, hi = _hot_args(sorted_hot)
     hot = hot if hot is not None else (None, None, None, None)
     _lib.call("hades_adam_update", _ptr(uids), _ptr(grad), _opt(num_unique), uids.numel(), dim,
-              _opt(sorted_hot), nh, _opt(hot[0]), _opt(hot[1]), _opt(hot[2]), _opt(hot[3]),
+              hp, hn, hi, _opt(hot[0]), _opt(hot[1]), _opt(hot[2]), _opt(hot[3]),
               _opt(cold[0]), _opt(cold[1]), _opt(cold[2]), _opt(cold[3]),
               float(lr), float(beta1), float(beta2), float(eps), _stream())
 

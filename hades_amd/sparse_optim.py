@@ -46,6 +46,7 @@ class _SparseRowOptimizer:
         self.num_rows, self.dim = weight_cold.shape
         hot_ids = torch.as_tensor(hot_ids, dtype=torch.int64)
         self.hot_ids = hot_ids.to(self.device)
+        self.hot_set = ops.HotSet(self.hot_ids)
         self.hot_w = self._gather_hot(weight_cold)
         self._ws = ops.Workspace(self.device)
 
@@ -64,7 +65,7 @@ class _SparseRowOptimizer:
 
     def fetch(self, ids, out=None):
         """Forward fetch of embedding rows (cached_fetch)."""
-        return ops.cached_fetch(self.cold_w, self.hot_w, ids, self.hot_ids, out=out)
+        return ops.cached_fetch(self.cold_w, self.hot_w, ids, self.hot_set, out=out)
 
     def step(self, idx, grad, mode=ops.COMBINE_FAST):
         """combine the per-occurrence gradients, then update every distinct row once.
@@ -87,7 +88,7 @@ class SparseAdagrad(_SparseRowOptimizer):
 
     def update(self, uids, grad, num_unique=None):
         ops.adagrad_update_(uids, grad, self.hot_w, self.hot_s, self.cold_w, self.cold_s,
-                            self.hot_ids, self.lr, self.eps, num_unique)
+                            self.hot_set, self.lr, self.eps, num_unique)
 
 
 class SparseAdam(_SparseRowOptimizer):
@@ -106,5 +107,5 @@ class SparseAdam(_SparseRowOptimizer):
 
     def update(self, uids, grad, num_unique=None):
         ops.adam_update_(uids, grad, (self.hot_w, self.hot_step, self.hot_m, self.hot_v),
-                         (self.cold_w, self.cold_step, self.cold_m, self.cold_v), self.hot_ids,
+                         (self.cold_w, self.cold_step, self.cold_m, self.cold_v), self.hot_set,
                          self.lr, self.betas[0], self.betas[1], self.eps, num_unique)

@@ -136,7 +136,18 @@ int hades_split(const void* ids, int id_type, const int8_t* class_table, int64_t
  * Replaces the dense index_map probe (python/EmbCache/cache.py:163-171) and the CPU
  * IndexCache round trip (python/EmbCache/dist_emb.py:184-185).  q, sorted_hot, loc: int64. */
 int hades_lookup_sorted(const int64_t* q, int64_t n, const int64_t* sorted_hot, int64_t num_hot,
-                        int64_t* loc, void* stream);
+                        const void* hot_index, int64_t* loc, void* stream);
+
+/* Optional bucket index over the hot set: table[b] = first position whose id >= (b << shift), with
+ * about one bucket per hot id.  With it a lookup is one table read plus a search over the few ids
+ * of one bucket instead of log2(num_hot) dependent probes of the sorted array; results are
+ * identical.  Build it once per hot set (the reference builds its dense index_map once per cache,
+ * python/EmbCache/cache.py:163-171; this takes 4 bytes per hot id instead of 8 per table row) and
+ * pass it as `hot_index` to the operators below; NULL there means plain binary search.  The
+ * buffer is device memory, 16-byte aligned, hades_hot_index_bytes(num_hot) bytes. */
+size_t hades_hot_index_bytes(int64_t num_hot);
+int hades_hot_index_build(const int64_t* sorted_hot, int64_t num_hot, void* hot_index,
+                          size_t hot_index_bytes, void* stream);
 
 /* Hot/cold split of a looked-up batch with stable compaction (replaces cudaSplit + torch.nonzero,
  * python/EmbCache/dist_emb.py:174-191):  hot <=> loc[i] >= 0.
@@ -164,8 +175,8 @@ int hades_split3_compact(const void* ids, int id_type, const int8_t* class_table
  *   loc = lookup(q[i]);  dst[i, :] = loc >= 0 ? hot_src[loc, :] : cold_src[q[i], :]
  * loc_out (int64[n]) may be NULL.  cold_src may be device or pinned host memory. */
 int hades_cached_fetch(const void* cold_src, const void* hot_src, const int64_t* q, int64_t n,
-                       const int64_t* sorted_hot, int64_t num_hot, void* dst, int64_t* loc_out,
-                       int64_t dim, int dtype, void* stream);
+                       const int64_t* sorted_hot, int64_t num_hot, const void* hot_index,
+                       void* dst, int64_t* loc_out, int64_t dim, int dtype, void* stream);
 
 /* Same gather when the slots are already known (loc from hades_lookup_sorted). */
 int hades_cached_fetch_loc(const void* cold_src, const void* hot_src, const int64_t* q,
@@ -176,7 +187,7 @@ int hades_cached_fetch_loc(const void* cold_src, const void* hot_src, const int6
  * src/cuda/uva_set.cu:71-93):
  *   loc = lookup(q[i]);  (loc >= 0 ? hot_dst[loc, :] : cold_dst[q[i], :]) = src[i, :] */
 int hades_cached_set(const void* src, void* cold_dst, void* hot_dst, const int64_t* q, int64_t n,
-                     const int64_t* sorted_hot, int64_t num_hot,
+                     const int64_t* sorted_hot, int64_t num_hot, const void* hot_index,
                      int64_t dim, int dtype, void* stream);
 
 /* combine: sort + dedup + segment-sum of duplicate-ID gradient rows; the arithmetic of
@@ -189,8 +200,9 @@ int hades_cached_set(const void* src, void* cold_dst, void* hot_dst, const int64
  * Entries at and beyond U are left unspecified.  id_bound > 0 promises 0 <= idx[i] < id_bound
  * (fewer sort passes); id_bound == 0 sorts all 64 bits as signed integers.
  * mode: HADES_COMBINE_FAST or HADES_COMBINE_EXACT.  n must be < 2^30.
- * Optional outputs (may be NULL): perm = occurrence positions in sorted order (int32[n]);
- * inverse[i] = index of idx[i] in uids (int32[n]). */
+ * Optional output (may be NULL): inverse[i] = index of idx[i] in uids (int32[n]).
+ * The first int32 of the workspace is a sticky status word: bit 0 is set when an id violated
+ * id_bound (the result is then unspecified).  Zero-fill the workspace once before first use. */
 size_t hades_combine_workspace_bytes(int64_t n, int64_t dim);
 int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim, int64_t id_bound,
                   int mode, int64_t* uids, float* sums, int64_t* cnts, int64_t* num_unique,
@@ -212,7 +224,7 @@ int hades_rows_div_count(float* sums, const int64_t* cnts, const int64_t* num_un
  * sorted_hot may be NULL with num_hot == 0 (everything in the cold tables). */
 int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                          int64_t max_rows, int64_t dim,
-                         const int64_t* sorted_hot, int64_t num_hot,
+                         const int64_t* sorted_hot, int64_t num_hot, const void* hot_index,
                          float* hot_w, float* hot_s, float* cold_w, float* cold_s,
                          float lr, float eps, void* stream);
 
@@ -222,7 +234,7 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
  * step: float[N] / float[H]; m, v, w: float[., dim]. */
 int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                       int64_t max_rows, int64_t dim,
-                      const int64_t* sorted_hot, int64_t num_hot,
+                      const int64_t* sorted_hot, int64_t num_hot, const void* hot_index,
                       float* hot_w, float* hot_step, float* hot_m, float* hot_v,
                       float* cold_w, float* cold_step, float* cold_m, float* cold_v,
                       float lr, double beta1, double beta2, float eps, void* stream);

@@ -171,6 +171,32 @@ def test_lookup_sorted(lib, n, h):
         q[:4] = [hot[0], hot[-1], hot[0] - 1, hot[-1] + 1]
     loc = ops.lookup(dev(q), dev(hot))
     assert np.array_equal(loc.cpu().numpy(), O.lookup_sorted(q, hot))
+    # the bucket index changes the search, never the answer
+    loc = ops.lookup(dev(q), ops.HotSet(dev(hot)))
+    assert np.array_equal(loc.cpu().numpy(), O.lookup_sorted(q, hot))
+
+
+@pytest.mark.parametrize("kind", ["clustered", "huge_ids", "negative", "single", "dense", "zero"])
+def test_lookup_bucket_index_on_awkward_id_sets(lib, kind):
+    _, ops = lib
+    rng = np.random.default_rng(55)
+    if kind == "clustered":      # all hot ids in two narrow clusters of a wide id space
+        hot = np.unique(np.concatenate([rng.integers(10**9, 10**9 + 5000, 3000),
+                                        rng.integers(7, 300, 200)])).astype(np.int64)
+    elif kind == "huge_ids":     # ids that need 62 bits
+        hot = np.unique(rng.integers(2**61, 2**62, 4000)).astype(np.int64)
+    elif kind == "negative":     # not a node-id set: the index marks itself unusable, search still right
+        hot = np.unique(rng.integers(-5000, 5000, 3000)).astype(np.int64)
+    elif kind == "single":
+        hot = np.array([12345], np.int64)
+    elif kind == "zero":
+        hot = np.array([0], np.int64)
+    else:                        # every id of a range
+        hot = np.arange(1000, 6000, dtype=np.int64)
+    extra = np.array([0, 1, -1, hot[0] - 1, hot[-1] + 1, 2**62 + 5, 2**63 - 1, -(2**63)], np.int64)
+    q = np.concatenate([rng.choice(hot, 3000), rng.choice(hot, 3000) + rng.integers(-2, 3, 3000), extra])
+    loc = ops.lookup(dev(q), ops.HotSet(dev(hot)))
+    assert np.array_equal(loc.cpu().numpy(), O.lookup_sorted(q, hot))
 
 
 @pytest.mark.parametrize("n", [0, 1, 7, 2048, 2049, 100_003])
@@ -232,6 +258,8 @@ def test_cached_fetch_and_set_sorted(lib, dim, host_cold):
     else:
         t_cold = dev(cold)
     t_hot, t_q, t_ids = dev(hot), dev(q), dev(hot_ids)
+    if dim != 64:
+        t_ids = ops.HotSet(t_ids)       # with the bucket index; dim 64 keeps the plain binary search
     out, loc = ops.cached_fetch(t_cold, t_hot, t_q, t_ids, return_loc=True)
     assert np.array_equal(out.cpu().numpy(), O.cached_fetch(cold, hot, q, hot_ids))
     assert np.array_equal(loc.cpu().numpy(), O.lookup_sorted(q, hot_ids))
