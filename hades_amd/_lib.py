@@ -9,7 +9,9 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libhades_hip.so")
+# HADES_LIB_PATH selects another build of the same library (e.g. one compiled with other tuning
+# constants); by default the in-tree build is used.
+LIB_PATH = os.environ.get("HADES_LIB_PATH") or os.path.join(_HERE, "csrc", "libhades_hip.so")
 
 F32, F64 = 0, 1
 I32, I64, I16, I8, U8 = 0, 1, 2, 3, 4

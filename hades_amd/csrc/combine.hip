@@ -7,11 +7,10 @@
 //   1. stable LSD radix sort of (key = id, value = occurrence position), 8 bits per pass, only
 //      over the key bits that id_bound leaves significant.  Stability keeps the positions of
 //      equal ids ascending, which is what makes a sequential in-segment sum reproduce CPU
-//      index_add_.  Per pass ONE kernel: every block derives its own global digit offsets from the
-//      per-tile digit counts [tile][digit] (column sums over all tiles and over the tiles before
-//      it), ranks its keys stably through LDS, scatters, and counts the NEXT pass's per-tile
-//      digits with aggregated global atomics at the scattered position.  Only the first pass
-//      needs a counting kernel of its own.
+//      index_add_.  Per pass two kernels: per-tile digit counts [tile][digit], then a scatter in
+//      which every block derives its own global digit offsets from those counts (column sums over
+//      all tiles and over the tiles before it - no separate scan kernel), ranks its keys stably
+//      through LDS and writes them out.
 //   2. run boundaries -> uids, seg_start, seg_of (index of the run every sorted position is in).
 //   3. segmented sum of the gradient rows:
 //        EXACT: one lane group per distinct id walks its rows left to right.
@@ -71,18 +70,15 @@ __device__ __forceinline__ uint64_t match_any(uint32_t v, int nbits, uint64_t am
   return peers;
 }
 
-// ---- first pass only: per-tile digit counts, and zero-fill of the later passes' counts ----
-// counts layout: cnt[tile * kBins + digit]
-template <typename KeyT, int IPT>
-__global__ __launch_bounds__(kThreads) void radix_count0_kernel(
-    const int64_t* __restrict__ ids, int64_t n, uint32_t mask, uint32_t* __restrict__ cnt0,
-    uint32_t* __restrict__ cnt_later, int64_t cnt_later_len, int64_t id_bound,
-    int32_t* __restrict__ status) {
+// ---- per-tile digit counts of one pass ------------------------------------------------------
+// counts layout: cnt[tile * kBins + digit].  (Counting the next pass's digits with global atomics
+// from inside the scatter was measured at twice the cost of this kernel.)
+template <typename KeyT, bool FIRST, int IPT>
+__global__ __launch_bounds__(kThreads) void radix_count_kernel(
+    const void* __restrict__ keys_in, int64_t n, int shift, uint32_t mask,
+    uint32_t* __restrict__ cnt, int64_t id_bound, int32_t* __restrict__ status) {
   __shared__ uint32_t s_hist[kBins];
   for (int d = threadIdx.x; d < kBins; d += kThreads) s_hist[d] = 0;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < cnt_later_len;
-       i += static_cast<int64_t>(gridDim.x) * kThreads)
-    cnt_later[i] = 0;
   __syncthreads();
   const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * (kThreads * IPT);
   bool bad = false;
@@ -90,15 +86,18 @@ __global__ __launch_bounds__(kThreads) void radix_count0_kernel(
   for (int r = 0; r < IPT; ++r) {
     const int64_t i = tile0 + r * kThreads + threadIdx.x;
     if (i < n) {
-      const int64_t id = ids[i];
-      bad = bad || (id_bound > 0 && (id < 0 || id >= id_bound));
-      atomicAdd(&s_hist[static_cast<uint32_t>(key_from_id<KeyT>(id)) & mask], 1u);
+      if (FIRST) {
+        const int64_t id = static_cast<const int64_t*>(keys_in)[i];
+        bad = bad || (id_bound > 0 && (id < 0 || id >= id_bound));
+      }
+      const KeyT k = load_key<KeyT, FIRST>(keys_in, i);
+      atomicAdd(&s_hist[static_cast<uint32_t>(k >> shift) & mask], 1u);
     }
   }
-  if (bad) atomicOr(status, 1);
+  if (FIRST && bad) atomicOr(status, 1);
   __syncthreads();
   for (int d = threadIdx.x; d < kBins; d += kThreads)
-    cnt0[static_cast<int64_t>(blockIdx.x) * kBins + d] = s_hist[d];
+    cnt[static_cast<int64_t>(blockIdx.x) * kBins + d] = s_hist[d];
 }
 
 // ---- one radix pass ---------------------------------------------------------------------
@@ -108,8 +107,7 @@ template <typename KeyT, bool FIRST, int IPT>
 __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
     const void* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, int64_t n, int shift,
     uint32_t mask, int bits, const uint32_t* __restrict__ cnt_cur, int64_t ntiles,
-    KeyT* __restrict__ keys_out, uint32_t* __restrict__ vals_out, uint32_t* __restrict__ cnt_next,
-    int next_shift, uint32_t next_mask, int tile_shift, int cell_bits) {
+    KeyT* __restrict__ keys_out, uint32_t* __restrict__ vals_out) {
   __shared__ uint32_t s_cnt[kWaves][kBins];
   __shared__ uint32_t s_glob[kBins];
   __shared__ uint32_t s_scan[kWaves + 1];
@@ -197,21 +195,11 @@ __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
 #pragma unroll
   for (int r = 0; r < IPT; ++r) {
     const int64_t i = wave0 + r * kWave + lane;
-    const bool valid = i < n;
-    uint32_t pos = 0;
-    if (valid) {
+    if (i < n) {
       const uint32_t d = static_cast<uint32_t>(key[r] >> shift) & mask;
-      pos = s_glob[d] + s_cnt[wave][d] + rank[r];
+      const uint32_t pos = s_glob[d] + s_cnt[wave][d] + rank[r];
       keys_out[pos] = key[r];
       vals_out[pos] = val[r];
-    }
-    if (cnt_next != nullptr) {
-      // count this key for the next pass, in the tile it has just been written to; lanes with
-      // the same (tile, digit) send one atomic between them
-      const uint32_t nd = static_cast<uint32_t>(key[r] >> next_shift) & next_mask;
-      const uint32_t cell = ((pos >> tile_shift) << kRadixBits) | nd;
-      const uint64_t peers = match_any(cell, cell_bits, __ballot(valid));
-      if (valid && (peers & lt_mask) == 0) atomicAdd(&cnt_next[cell], __popcll(peers));
     }
   }
 }
@@ -632,7 +620,7 @@ struct SortWs {
   int32_t* status;
   void* keys[2];
   uint32_t* vals[2];
-  uint32_t* cnt;        // [passes][ntiles][kBins]
+  uint32_t* cnt;        // [ntiles][kBins], rewritten by every pass
   int64_t cnt_len;
   size_t bytes;
 };
@@ -642,10 +630,7 @@ void carve_sort(Carver& c, int64_t n, SortWs* w) {
   w->status = c.take<int32_t>(64);
   for (int i = 0; i < 2; ++i) w->keys[i] = c.take<uint64_t>(nn);  // sized for 64-bit keys
   for (int i = 0; i < 2; ++i) w->vals[i] = c.take<uint32_t>(nn);
-  // sized for the most passes and the most tiles any plan for this n can have
-  w->cnt_len = static_cast<int64_t>(kMaxPasses) * ceil_div(nn, kThreads * 4) * kBins;
-  if (ceil_div(nn, kThreads * 4) > 512)
-    w->cnt_len = static_cast<int64_t>(kMaxPasses) * make_plan(nn, 1, 0, true).ntiles * kBins;
+  w->cnt_len = make_plan(nn, 1, 0, true).ntiles * kBins;  // the tile count depends on n only
   w->cnt = c.take<uint32_t>(w->cnt_len);
   w->bytes = c.total();
 }
@@ -684,13 +669,6 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
     bits_of[pass] = base + (pass < extra ? 1 : 0);
     shift_of[pass + 1] = shift_of[pass] + bits_of[pass];
   }
-  const int tile_shift = ilog2_ceil(static_cast<uint64_t>(kThreads * IPT));
-  const int cell_bits = kRadixBits + ilog2_ceil(static_cast<uint64_t>(p.ntiles)) + 1;
-  const int64_t stride = p.ntiles * kBins;
-  HADES_LAUNCH((radix_count0_kernel<KeyT, IPT>), grid, block, 0, st, idx, n,
-                     (1u << bits_of[0]) - 1u, w.cnt, w.cnt + stride,
-                     static_cast<int64_t>(p.passes - 1) * stride, id_bound, w.status);
-  HADES_LAUNCH_CHECK();
   const void* kin = idx;
   const uint32_t* vin = nullptr;
   int cur = 0;
@@ -698,20 +676,17 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
     const uint32_t mask = (1u << bits_of[pass]) - 1u;
     KeyT* kout = static_cast<KeyT*>(w.keys[cur]);
     uint32_t* vout = w.vals[cur];
-    const bool last = pass + 1 == p.passes;
-    uint32_t* cnt_next = last ? nullptr : w.cnt + (pass + 1) * stride;
-    const int next_shift = last ? 0 : shift_of[pass + 1];
-    const uint32_t next_mask = last ? 0u : (1u << bits_of[pass + 1]) - 1u;
     if (pass == 0) {
+      HADES_LAUNCH((radix_count_kernel<KeyT, true, IPT>), grid, block, 0, st, kin, n,
+                   shift_of[pass], mask, w.cnt, id_bound, w.status);
       HADES_LAUNCH((radix_pass_kernel<KeyT, true, IPT>), grid, block, 0, st, kin, vin, n,
-                         shift_of[pass], mask, bits_of[pass], w.cnt + pass * stride, p.ntiles, kout,
-                         vout, cnt_next, next_shift, next_mask, tile_shift, cell_bits);
+                   shift_of[pass], mask, bits_of[pass], w.cnt, p.ntiles, kout, vout);
     } else {
+      HADES_LAUNCH((radix_count_kernel<KeyT, false, IPT>), grid, block, 0, st, kin, n,
+                   shift_of[pass], mask, w.cnt, id_bound, w.status);
       HADES_LAUNCH((radix_pass_kernel<KeyT, false, IPT>), grid, block, 0, st, kin, vin, n,
-                         shift_of[pass], mask, bits_of[pass], w.cnt + pass * stride, p.ntiles, kout,
-                         vout, cnt_next, next_shift, next_mask, tile_shift, cell_bits);
+                   shift_of[pass], mask, bits_of[pass], w.cnt, p.ntiles, kout, vout);
     }
-    HADES_LAUNCH_CHECK();
     kin = kout;
     vin = vout;
     cur ^= 1;
@@ -724,7 +699,7 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
 template <typename KeyT>
 int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
              hipStream_t st, const void** keys_out, const uint32_t** perm_out) {
-  HADES_REQUIRE(p.ntiles * kBins * static_cast<int64_t>(p.passes) <= w.cnt_len,
+  HADES_REQUIRE(p.ntiles * kBins <= w.cnt_len,
                 "internal: radix count buffer too small");
   switch (p.ipt) {
     case 4: return run_sort_ipt<KeyT, 4>(idx, n, id_bound, p, w, st, keys_out, perm_out);
