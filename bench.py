@@ -35,6 +35,14 @@ def parse_args():
     return ap.parse_args()
 
 
+def log(msg):
+    """Progress on stderr (stdout carries only the JSON line)."""
+    print("[bench %6.1fs] %s" % (time.perf_counter() - _T0, msg), file=sys.stderr, flush=True)
+
+
+_T0 = time.perf_counter()
+
+
 class Workload:
     """Tables, hot set and pre-generated batches of one configuration, resident on the device
     (cold table in pinned host memory for cfg3)."""
@@ -51,13 +59,22 @@ class Workload:
         self.n = cfg["batch"] * self.trainers
         self.host_cold = name == "cfg3"
         seed = 1234 + int(name[3:])
+        log("allocating the %d x %d table (%.1f GB, %s)" %
+            (N, D, N * D * 4 / 1e9, "pinned host" if self.host_cold else "HBM"))
         if self.host_cold:
             table = torch.empty((N, D), dtype=torch.float32, pin_memory=True)
         else:
             table = torch.empty((N, D), dtype=torch.float32, device=device)
-        synth.fill_normal_(table, 0.01, seed)
+        log("filling it")
+        synth.fill_normal_(table, 0.01, seed, progress=log if N > 50_000_000 else None)
         hot_ids = synth.hot_ids(N, H, device) if H else torch.empty(0, dtype=torch.int64, device=device)
-        self.opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=device)
+        log("hot copies and optimizer state")
+        # cfg3: the cold weights are the pinned host table; the cold Adagrad state stays in HBM
+        # (a second 57 GB page-locked allocation is refused on the benchmark box, and 288 GB of
+        # HBM have the room)
+        self.opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=device,
+                                 state_on_device=self.host_cold)
+        log("sampling %d batches of %d ids" % (nbatches, self.n))
         sampler = synth.ZipfSampler(N, cfg["zipf_s"], device)
         self.ids, self.grads = [], []
         for b in range(nbatches):
@@ -71,10 +88,13 @@ class Workload:
                          torch.empty((self.n, D), dtype=torch.float32, device=device),
                          torch.empty(self.n, dtype=torch.int64, device=device),
                          torch.empty(1, dtype=torch.int64, device=device))
+        log("workload ready")
 
     def describe(self):
         return ("%s: %d x %d fp32 table (%s), hot %d rows in HBM, %d ids/step zipf s=%.2f%s" %
-                (self.name, self.N, self.D, "cold rows in pinned host memory" if self.host_cold
+                (self.name, self.N, self.D,
+                 "cold weights in pinned host memory read zero-copy, cold Adagrad state in HBM"
+                 if self.host_cold
                  else "all in HBM", self.H, self.n, self.cfg["zipf_s"],
                  ", %d trainer batches concatenated" % self.trainers if self.trainers > 1 else ""))
 
@@ -90,7 +110,16 @@ def run_gpu(args):
     ws = ops.Workspace(dev)
     nb = len(wl.ids)
     phases = ("fetch", "combine", "update")
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+
+    def new_events(count):
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+        for e in evs:
+            e.record()          # torch creates the HIP event on first use
+        return evs
+
+    ev = [new_events(4) for _ in range(args.steps)]
+    kev = [new_events(2) for _ in range(args.steps)]
+    torch.cuda.synchronize()
 
     def step(i, events=None):
         q, g = wl.ids[i % nb], wl.grads[i % nb]
@@ -103,18 +132,39 @@ def run_gpu(args):
         opt.update(uids, sums, nu)
         if events: events[3].record()
 
+    # the three row-moving kernels of a step; the dominant one is found on a few untimed steps
+    kernels = {ops.KERNEL_CACHED_FETCH: "row_move_kernel<AddrFetchSorted> (hades_cached_fetch)",
+               ops.KERNEL_SEG_SUM: "seg_chunk_kernel (hades_combine)" if args.mode == "fast"
+               else "seg_exact_kernel (hades_combine)",
+               ops.KERNEL_ADAGRAD: "adagrad_kernel (hades_adagrad_update)"}
     for i in range(args.warmup):
         step(i)
+    probe_ms = {}
+    for kid in kernels:
+        acc = 0.0
+        for i in range(3):
+            ops.profile_kernel(kid, kev[i][0], kev[i][1])
+            step(i)
+        torch.cuda.synchronize()
+        for i in range(3):
+            acc += kev[i][0].elapsed_time(kev[i][1])
+        probe_ms[kid] = acc / 3
+    ops.profile_kernel(0)
+    dominant = max(kernels, key=lambda k: probe_ms[k])
+
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
+        ops.profile_kernel(dominant, kev[i][0], kev[i][1])
         step(i, ev[i])
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    ops.profile_kernel(0)
     ms_per_step = (t1 - t0) * 1e3 / args.steps
 
     phase_ms = {p: sum(ev[i][k].elapsed_time(ev[i][k + 1]) for i in range(args.steps)) / args.steps
                 for k, p in enumerate(phases)}
+    kernel_ms = sum(kev[i][0].elapsed_time(kev[i][1]) for i in range(args.steps)) / args.steps
     # distinct ids per step and hot-hit statistics of the batches actually used
     uniq, hot_hit, uniq_hot = [], [], []
     for q in wl.ids:
@@ -130,17 +180,22 @@ def run_gpu(args):
     U_hot = sum(uniq_hot) / len(uniq_hot)
     hit = sum(hot_hit) / len(hot_hit)
     n, D = wl.n, wl.D
-    # algorithmic bytes per launch of each phase (fp32): fetch 16 + 8D per query row;
-    # combine n(8+4D) read + U(16+4D) written; Adagrad 8 + 20D per distinct row
+    # algorithmic bytes per launch (fp32).  Phases: fetch 16 + 8D per query row; combine
+    # n(8+4D) read + U(16+4D) written; Adagrad 8 + 20D per distinct row.  Kernels: the fetch and
+    # Adagrad kernels are their whole phase; the segmented-sum kernel reads n rows plus 8 bytes of
+    # sort output per row and writes U rows.
     alg_bytes = {"fetch": n * (16 + 8 * D), "combine": n * (8 + 4 * D) + U * (16 + 4 * D),
                  "update": U * (8 + 20 * D)}
-    dominant = max(phases, key=lambda p: phase_ms[p])
-    kernel_of = {"fetch": "row_move_kernel<AddrFetchSorted>", "combine": "hades_combine (sort + runs + seg_chunk_kernel + seg_fixup_kernel)",
-                 "update": "adagrad_kernel"}
-    achieved = alg_bytes[dominant] / (phase_ms[dominant] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": kernel_of[dominant], "achieved": round(achieved, 1),
+    kernel_bytes = {ops.KERNEL_CACHED_FETCH: alg_bytes["fetch"],
+                    ops.KERNEL_SEG_SUM: n * (8 + 4 * D) + U * 4 * D,
+                    ops.KERNEL_ADAGRAD: alg_bytes["update"]}
+    achieved = kernel_bytes[dominant] / (kernel_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": kernels[dominant], "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": None}
+                "traffic": None, "kernel_us": round(kernel_ms * 1e3, 2),
+                "bytes_per_launch": int(kernel_bytes[dominant]),
+                "other_kernels_us": {kernels[k]: round(probe_ms[k] * 1e3, 2) for k in kernels
+                                     if k != dominant}}
     per_phase = {p: {"ms": round(phase_ms[p], 4),
                      "GB/s": round(alg_bytes[p] / (phase_ms[p] * 1e-3) / 1e9, 1),
                      "frac_hbm": round(alg_bytes[p] / (phase_ms[p] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
@@ -156,8 +211,9 @@ def run_gpu(args):
         cold_u = U - U_hot
         extra["pcie"] = {
             "fetch_GB/s": round(cold_q * 4 * D / (phase_ms["fetch"] * 1e-3) / 1e9, 2),
-            "update_read_GB/s": round(cold_u * 8 * D / (phase_ms["update"] * 1e-3) / 1e9, 2),
-            "update_write_GB/s": round(cold_u * 8 * D / (phase_ms["update"] * 1e-3) / 1e9, 2),
+            "update_read_GB/s": round(cold_u * 4 * D / (phase_ms["update"] * 1e-3) / 1e9, 2),
+            "update_write_GB/s": round(cold_u * 4 * D / (phase_ms["update"] * 1e-3) / 1e9, 2),
+            "cold_query_rows": round(cold_q, 1), "cold_unique_rows": round(cold_u, 1),
             "peak_per_direction": PCIE_PEAK_GBS}
     return wl, ms_per_step, roofline, extra
 

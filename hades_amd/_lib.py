@@ -21,7 +21,10 @@ _P = c_void_p
 _L = c_int64
 
 # name -> argument types; every function returns int unless listed in _RESTYPE
+KERNEL_NONE, KERNEL_CACHED_FETCH, KERNEL_SEG_SUM, KERNEL_ADAGRAD, KERNEL_RADIX_PASS = 0, 1, 2, 3, 4
+
 _SIGNATURES = {
+    "hades_profile_kernel": [c_int, _P, _P],
     "hades_pin": [_P, c_size_t],
     "hades_unpin": [_P],
     "hades_host_alloc": [ctypes.POINTER(c_void_p), c_size_t],

@@ -679,13 +679,15 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
     if (pass == 0) {
       HADES_LAUNCH((radix_count_kernel<KeyT, true, IPT>), grid, block, 0, st, kin, n,
                    shift_of[pass], mask, w.cnt, id_bound, w.status);
-      HADES_LAUNCH((radix_pass_kernel<KeyT, true, IPT>), grid, block, 0, st, kin, vin, n,
-                   shift_of[pass], mask, bits_of[pass], w.cnt, p.ntiles, kout, vout);
+      HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, true, IPT>), grid,
+                         block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
+                         p.ntiles, kout, vout);
     } else {
       HADES_LAUNCH((radix_count_kernel<KeyT, false, IPT>), grid, block, 0, st, kin, n,
                    shift_of[pass], mask, w.cnt, id_bound, w.status);
-      HADES_LAUNCH((radix_pass_kernel<KeyT, false, IPT>), grid, block, 0, st, kin, vin, n,
-                   shift_of[pass], mask, bits_of[pass], w.cnt, p.ntiles, kout, vout);
+      HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, false, IPT>), grid,
+                         block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
+                         p.ntiles, kout, vout);
     }
     kin = kout;
     vin = vout;
@@ -806,17 +808,21 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
     const int64_t blocks = ceil_div(n * p.group, kThreads);
     HADES_REQUIRE(blocks < (int64_t(1) << 31), "combine: too many rows");
     if (p.vec == 4)
-      HADES_LAUNCH((seg_exact_kernel<4>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
+      HADES_LAUNCH_TIMED(HADES_KERNEL_SEG_SUM, st, (seg_exact_kernel<4>), dim3((unsigned)blocks),
+                         dim3(kThreads), 0, st, a);
     else
-      HADES_LAUNCH((seg_exact_kernel<1>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
+      HADES_LAUNCH_TIMED(HADES_KERNEL_SEG_SUM, st, (seg_exact_kernel<1>), dim3((unsigned)blocks),
+                         dim3(kThreads), 0, st, a);
     HADES_LAUNCH_CHECK();
   } else {
     HADES_REQUIRE(p.nblocks_seg < (int64_t(1) << 31), "combine: too many rows");
     const dim3 grid(static_cast<unsigned>(p.nblocks_seg));
     if (p.vec == 4)
-      HADES_LAUNCH((seg_chunk_kernel<4>), grid, dim3(kThreads), 0, st, a);
+      HADES_LAUNCH_TIMED(HADES_KERNEL_SEG_SUM, st, (seg_chunk_kernel<4>), grid, dim3(kThreads), 0,
+                         st, a);
     else
-      HADES_LAUNCH((seg_chunk_kernel<1>), grid, dim3(kThreads), 0, st, a);
+      HADES_LAUNCH_TIMED(HADES_KERNEL_SEG_SUM, st, (seg_chunk_kernel<1>), grid, dim3(kThreads), 0,
+                         st, a);
     HADES_LAUNCH_CHECK();
     // one block per span of the chunk kernel, and at least one thread per sorted position so that
     // every u < U <= n gets its count written

@@ -41,6 +41,23 @@ int set_error(int code, const char* fmt, ...);
   } while (0)
 #define HADES_LAUNCH_CHECK() HADES_HIP_TRY(hipGetLastError())
 
+// Optional timing of one named kernel: hades_profile_kernel() arms a pair of HIP events that the
+// next launches of that kernel (on the calling thread) record around themselves, on the stream
+// the kernel is launched on.
+struct ProfileSlot {
+  int kernel_id = 0;
+  hipEvent_t start = nullptr, stop = nullptr;
+};
+extern thread_local ProfileSlot g_profile;
+
+#define HADES_LAUNCH_TIMED(kid, stream_, ...)                                        \
+  do {                                                                               \
+    const bool _timed = ::hades::g_profile.kernel_id == (kid);                       \
+    if (_timed) HADES_HIP_TRY(hipEventRecord(::hades::g_profile.start, (stream_)));  \
+    HADES_LAUNCH(__VA_ARGS__);                                                       \
+    if (_timed) HADES_HIP_TRY(hipEventRecord(::hades::g_profile.stop, (stream_)));   \
+  } while (0)
+
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
 inline int ilog2_ceil(uint64_t x) {  // smallest b with 2^b >= x

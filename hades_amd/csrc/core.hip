@@ -6,6 +6,7 @@
 namespace hades {
 
 static thread_local std::string g_last_error;
+thread_local ProfileSlot g_profile;
 
 int set_error(int code, const char* fmt, ...) {
   char buf[1024];
@@ -26,6 +27,15 @@ extern "C" {
 const char* hades_last_error(void) { return g_last_error.c_str(); }
 
 int hades_version(void) { return 100; }
+
+int hades_profile_kernel(int kernel_id, void* start_event, void* stop_event) {
+  HADES_REQUIRE(kernel_id >= 0 && kernel_id <= HADES_KERNEL_LAST, "unknown kernel id %d", kernel_id);
+  HADES_REQUIRE(kernel_id == 0 || (start_event && stop_event), "null event");
+  g_profile.kernel_id = kernel_id;
+  g_profile.start = static_cast<hipEvent_t>(start_event);
+  g_profile.stop = static_cast<hipEvent_t>(stop_event);
+  return HADES_OK;
+}
 
 int hades_pin(void* host_ptr, size_t bytes) {
   HADES_REQUIRE(host_ptr != nullptr, "hades_pin: null pointer");

@@ -162,7 +162,8 @@ int pick_vec(int64_t row_bytes, std::initializer_list<const void*> bases) {
 }
 
 template <typename Addr>
-int launch_mover(const Addr& addr, int64_t n, int64_t row_bytes, int vec, hipStream_t stream) {
+int launch_mover(const Addr& addr, int64_t n, int64_t row_bytes, int vec, hipStream_t stream,
+                 int kernel_id = -1) {
   if (n == 0) return HADES_OK;
   const int64_t cpr64 = row_bytes / vec;
   HADES_REQUIRE(cpr64 * kRowsPerBlock < (int64_t(1) << 30), "row of %lld bytes is too large",
@@ -173,7 +174,8 @@ int launch_mover(const Addr& addr, int64_t n, int64_t row_bytes, int vec, hipStr
   HADES_REQUIRE(blocks < (int64_t(1) << 31), "too many rows: %lld", (long long)n);
   dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
   if (vec == 16) {
-    HADES_LAUNCH((row_move_kernel<u32x4, Addr>), grid, block, 0, stream, addr, n, cpr, shift);
+    HADES_LAUNCH_TIMED(kernel_id, stream, (row_move_kernel<u32x4, Addr>), grid, block, 0, stream,
+                       addr, n, cpr, shift);
   } else if (vec == 8) {
     HADES_LAUNCH((row_move_kernel<u32x2, Addr>), grid, block, 0, stream, addr, n, cpr, shift);
   } else {
@@ -303,7 +305,8 @@ int hades_cached_fetch(const void* cold_src, const void* hot_src, const int64_t*
   AddrFetchSorted a{(const char*)cold_src, (const char*)hot_src, q,
                     HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)},
                     (char*)dst, loc_out, row_bytes};
-  return launch_mover(a, n, row_bytes, vec, static_cast<hipStream_t>(stream));
+  return launch_mover(a, n, row_bytes, vec, static_cast<hipStream_t>(stream),
+                      HADES_KERNEL_CACHED_FETCH);
 }
 
 int hades_cached_fetch_loc(const void* cold_src, const void* hot_src, const int64_t* q,

@@ -223,9 +223,9 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
   const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dim % 4 == 0 && aligned16({grad, hot_w, hot_s, cold_w, cold_s}))
-    HADES_LAUNCH((adagrad_kernel<4>), grid, block, 0, st, a);
+    HADES_LAUNCH_TIMED(HADES_KERNEL_ADAGRAD, st, (adagrad_kernel<4>), grid, block, 0, st, a);
   else
-    HADES_LAUNCH((adagrad_kernel<1>), grid, block, 0, st, a);
+    HADES_LAUNCH_TIMED(HADES_KERNEL_ADAGRAD, st, (adagrad_kernel<1>), grid, block, 0, st, a);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }

@@ -57,6 +57,24 @@ def _ws(device, kind):
     return _default_ws[key]
 
 
+# ---- kernel timing -------------------------------------------------------------
+KERNEL_CACHED_FETCH = _lib.KERNEL_CACHED_FETCH
+KERNEL_SEG_SUM = _lib.KERNEL_SEG_SUM
+KERNEL_ADAGRAD = _lib.KERNEL_ADAGRAD
+KERNEL_RADIX_PASS = _lib.KERNEL_RADIX_PASS
+
+
+def profile_kernel(kernel_id, start=None, stop=None):
+    """Arms (or with kernel_id 0 disarms) a pair of torch.cuda.Event(enable_timing=True) that the
+    library records around every later launch of that kernel, on the kernel's own stream.  The
+    events must have been recorded once before, so that torch has created their handles."""
+    if not kernel_id:
+        _lib.call("hades_profile_kernel", 0, _NULL, _NULL)
+        return
+    _lib.call("hades_profile_kernel", int(kernel_id), ctypes.c_void_p(start.cuda_event),
+              ctypes.c_void_p(stop.cuda_event))
+
+
 # ---- the hot set and lookup -----------------------------------------------------
 class HotSet:
     """The ascending, duplicate-free hot ids on the device together with the bucket index that

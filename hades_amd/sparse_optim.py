@@ -9,7 +9,7 @@ an EmbCache-style (hot, cold) table pair.  The cross-trainer all-to-all of the r
 """
 import torch
 
-from . import ops
+from . import EmbCacheLib, ops
 
 
 def only_unique_grads(idx, grad, id_bound=0, mode=ops.COMBINE_FAST):
@@ -39,8 +39,12 @@ class _SparseRowOptimizer:
     """State shared by the two optimizers: weights and state as (hot, cold) pairs keyed by the
     ascending hot-ID set.  `weight_cold` is [N, D] on the device or pinned on the host."""
 
-    def __init__(self, weight_cold, hot_ids, lr, device="cuda"):
+    def __init__(self, weight_cold, hot_ids, lr, device="cuda", state_on_device=False):
         self.device = torch.device(device)
+        # cold optimizer state normally lives where the cold weights live; with state_on_device
+        # it is kept in HBM even when the weights are a pinned host table (288 GB of HBM hold the
+        # state of tables whose weights are served from the host)
+        self.state_on_device = state_on_device
         self.lr = lr
         self.cold_w = weight_cold
         self.num_rows, self.dim = weight_cold.shape
@@ -51,16 +55,27 @@ class _SparseRowOptimizer:
         self._ws = ops.Workspace(self.device)
 
     def _gather_hot(self, cold):
+        """Hot copy of the rows named by hot_ids; a pinned host table is read zero-copy by the
+        gather kernel instead of being indexed on the CPU."""
         if cold.is_cuda:
             return cold[self.hot_ids].contiguous()
-        return cold[self.hot_ids.cpu()].to(self.device)
+        out = torch.empty((self.hot_ids.numel(),) + tuple(cold.shape[1:]), dtype=cold.dtype,
+                          device=self.device)
+        EmbCacheLib.cudaFetch2(cold, self.hot_ids, out)
+        return out
 
     def _new_state_like(self, cold, shape=None):
         shape = shape or tuple(cold.shape)
-        if cold.is_cuda:
-            return torch.zeros(shape, dtype=torch.float32, device=cold.device)
+        if cold.is_cuda or self.state_on_device:
+            return torch.zeros(shape, dtype=torch.float32, device=self.device)
         t = torch.empty(shape, dtype=torch.float32, pin_memory=True)
-        t.zero_()
+        # zero it from the device in slices (a 57 GB memset on one host core takes far longer)
+        flat = t.view(-1)
+        step = 1 << 28
+        zeros = torch.zeros(min(step, flat.numel()), dtype=torch.float32, device=self.device)
+        for i in range(0, flat.numel(), step):
+            m = min(step, flat.numel() - i)
+            flat[i:i + m].copy_(zeros[:m])
         return t
 
     def fetch(self, ids, out=None):
@@ -80,8 +95,9 @@ class SparseAdagrad(_SparseRowOptimizer):
     """s += g*g;  w -= lr * g / (sqrt(s) + eps) on the rows a step touches
     (torch.optim.Adagrad with lr_decay = weight_decay = initial_accumulator_value = 0)."""
 
-    def __init__(self, weight_cold, hot_ids, lr=0.01, eps=1e-10, device="cuda"):
-        super().__init__(weight_cold, hot_ids, lr, device)
+    def __init__(self, weight_cold, hot_ids, lr=0.01, eps=1e-10, device="cuda",
+                 state_on_device=False):
+        super().__init__(weight_cold, hot_ids, lr, device, state_on_device)
         self.eps = eps
         self.cold_s = self._new_state_like(weight_cold)
         self.hot_s = torch.zeros_like(self.hot_w)
@@ -94,8 +110,9 @@ class SparseAdagrad(_SparseRowOptimizer):
 class SparseAdam(_SparseRowOptimizer):
     """The reference's SparseAdam.update (python/EmbCache/sparse_optim.py:590-685) as one kernel."""
 
-    def __init__(self, weight_cold, hot_ids, lr=0.01, betas=(0.9, 0.999), eps=1e-8, device="cuda"):
-        super().__init__(weight_cold, hot_ids, lr, device)
+    def __init__(self, weight_cold, hot_ids, lr=0.01, betas=(0.9, 0.999), eps=1e-8, device="cuda",
+                 state_on_device=False):
+        super().__init__(weight_cold, hot_ids, lr, device, state_on_device)
         self.betas, self.eps = betas, eps
         n, h = self.num_rows, self.hot_ids.numel()
         self.cold_step = self._new_state_like(weight_cold, (n,))

@@ -68,7 +68,7 @@ def make_grads(n, dim, seed, device="cpu"):
     return (torch.randn(n, dim, generator=g, dtype=torch.float32) * 1e-3).to(device)
 
 
-def fill_normal_(t, std, seed, chunk_rows=1 << 20):
+def fill_normal_(t, std, seed, chunk_rows=1 << 20, progress=None):
     """In-place N(0, std) fill, chunk-wise so that pinned host tables of tens of GB can be filled
     from the device without a second full-size buffer."""
     if t.is_cuda:
@@ -80,10 +80,12 @@ def fill_normal_(t, std, seed, chunk_rows=1 << 20):
         dev = torch.device("cuda")
         g = torch.Generator(device=dev).manual_seed(seed)
         buf = torch.empty((chunk_rows,) + tuple(t.shape[1:]), dtype=t.dtype, device=dev)
-        for r0 in range(0, t.size(0), chunk_rows):
+        for k, r0 in enumerate(range(0, t.size(0), chunk_rows)):
             rows = min(chunk_rows, t.size(0) - r0)
             buf[:rows].normal_(0.0, std, generator=g)
             t[r0:r0 + rows].copy_(buf[:rows])
+            if progress and k % 16 == 15:
+                progress("filled %d of %d rows" % (r0 + rows, t.size(0)))
         return t
     g = torch.Generator().manual_seed(seed)
     return t.normal_(0.0, std, generator=g)

@@ -55,6 +55,18 @@ extern "C" {
 const char* hades_last_error(void);
 int hades_version(void);
 
+/* Kernel timing hook (no counterpart in the reference, whose scripts time whole calls from the
+ * host: test/test_cached_fetch.py:51-56).  Arms a pair of hipEvent_t handles; from then on every
+ * launch of the named kernel made by the calling thread records start_event before and
+ * stop_event after itself, on the stream it is launched on.  kernel_id 0 disarms. */
+#define HADES_KERNEL_NONE 0
+#define HADES_KERNEL_CACHED_FETCH 1 /* row mover launched by hades_cached_fetch */
+#define HADES_KERNEL_SEG_SUM 2      /* segmented row sum of hades_combine (FAST: chunk kernel; EXACT: exact kernel) */
+#define HADES_KERNEL_ADAGRAD 3      /* hades_adagrad_update */
+#define HADES_KERNEL_RADIX_PASS 4   /* scatter passes of the sort in hades_combine (the pair keeps the last pass) */
+#define HADES_KERNEL_LAST 4
+int hades_profile_kernel(int kernel_id, void* start_event, void* stop_event);
+
 /* ------------------------------------------------------------------------- */
 /* Group 1: one entry point per function bound in src/pybind.cc:46-70          */
 /* ------------------------------------------------------------------------- */

@@ -351,6 +351,8 @@ def torch_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps):
     reference's CPU-side code has: searchsorted for the lookup, indexed reads, torch.unique +
     index_add_ for the combine (python/EmbCache/sparse_optim.py:132-139), element-wise update."""
     def lookup(ids):
+        if sorted_hot.numel() == 0:
+            return torch.full_like(ids, -1)
         pos = torch.searchsorted(sorted_hot, ids, right=True)
         prev = sorted_hot[(pos - 1).clamp_(min=0)]
         return torch.where((pos > 0) & (prev == ids), pos - 1, torch.full_like(pos, -1))
