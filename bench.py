@@ -40,6 +40,10 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
+    ap.add_argument("--schedule", default="serial", choices=["serial", "overlap"],
+                    help="serial: every kernel of the step on one stream (the default: measured "
+                         "faster); overlap: the sort of the ids runs on a side stream next to the "
+                         "fetch")
     ap.add_argument("--batches", type=int, default=4, help="distinct pre-generated id batches")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -135,13 +139,25 @@ def run_gpu(args):
     kev = [new_events(2) for _ in range(args.steps)]
     torch.cuda.synchronize()
 
+    uids_o, sums_o, cnts_o, nu_o = wl.comb_out
+    overlap = args.schedule == "overlap"
+
     def step(i, events=None):
+        """fetch -> combine -> update of batch i.  With the overlapped schedule the id-only half
+        of the combine (sort + run boundaries) is issued on a side stream before the fetch, as a
+        trainer that knows the ids at forward time would do; everything that touches rows stays
+        on the main stream in program order."""
         q, g = wl.ids[i % nb], wl.grads[i % nb]
+        if overlap:
+            plan = opt.prepare(q, out=(uids_o, nu_o))
         if events: events[0].record()
         ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_set, out=wl.rows_out)
         if events: events[1].record()
-        uids, sums, cnts, nu = ops.combine_padded(q, g, id_bound=wl.N, mode=mode, workspace=ws,
-                                                  out=wl.comb_out)
+        if overlap:
+            torch.cuda.current_stream().wait_event(plan.ready)
+        else:
+            plan = ops.combine_plan(q, wl.D, id_bound=wl.N, workspace=opt._ws, out=(uids_o, nu_o))
+        uids, sums, cnts, nu = ops.combine_apply(plan, g, mode, out=(sums_o, cnts_o))
         if events: events[2].record()
         opt.update(uids, sums, nu)
         if events: events[3].record()
@@ -302,7 +318,9 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": wl.describe(), "combine_mode": args.mode,
-                   "optimizer": "sparse Adagrad lr=0.01 eps=1e-10"},
+                   "optimizer": "sparse Adagrad lr=0.01 eps=1e-10",
+                   "schedule": "sort of the step's ids on a side stream, concurrent with its fetch"
+                   if args.schedule == "overlap" else "one stream"},
         "roofline": roofline,
     }
     line.update(extra)

@@ -103,7 +103,9 @@ __global__ __launch_bounds__(kThreads) void adagrad_kernel(AdagradArgs a) {
         const int64_t off = s_row[r] * a.r.dim + col;
         sp[k] = reinterpret_cast<V*>((s_hot[r] ? a.hot_s : a.cold_s) + off);
         wp[k] = reinterpret_cast<V*>((s_hot[r] ? a.hot_w : a.cold_w) + off);
-        g[k] = *reinterpret_cast<const V*>(a.r.grad + (row0 + r) * a.r.dim + col);
+        // the gradient row is read once; the state and weight rows of hot ids come back next step
+        g[k] = __builtin_nontemporal_load(
+            reinterpret_cast<const V*>(a.r.grad + (row0 + r) * a.r.dim + col));
         s[k] = *sp[k];
         w[k] = *wp[k];
       }

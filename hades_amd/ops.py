@@ -256,6 +256,54 @@ def combine_padded(idx, grad, id_bound=0, mode=COMBINE_FAST, return_inverse=Fals
     return uids, sums, cnts, num_unique
 
 
+class CombinePlan:
+    """The id-only half of a combine: sort permutation and run boundaries (kept in `workspace`),
+    the distinct ids and their number.  Made by combine_plan, consumed by combine_apply."""
+
+    def __init__(self, n, dim, id_bound, uids, num_unique, inverse, workspace):
+        self.n, self.dim, self.id_bound = n, dim, id_bound
+        self.uids, self.num_unique, self.inverse = uids, num_unique, inverse
+        self.workspace = workspace
+
+
+def combine_plan(idx, dim, id_bound=0, return_inverse=False, workspace=None, out=None):
+    """Sorts the ids and finds the runs; needs no gradients, so it can run as soon as the ids of a
+    batch are known (e.g. at forward time, on another stream).  `workspace` is a Workspace that must
+    not be used by anything else until combine_apply has consumed the plan.  `out` = (uids int64[n],
+    num_unique int64[1]) to write into preallocated tensors."""
+    _i64(idx, "idx")
+    n, dev = idx.numel(), idx.device
+    if out is None:
+        uids = torch.empty(n, dtype=torch.int64, device=dev)
+        num_unique = torch.empty(1, dtype=torch.int64, device=dev)
+    else:
+        uids, num_unique = out
+    inverse = torch.empty(n, dtype=torch.int32, device=dev) if return_inverse else None
+    workspace = workspace or Workspace(dev)
+    ws = workspace.get(_lib.query("hades_combine_workspace_bytes", n, int(dim)))
+    _lib.call("hades_combine_plan", _ptr(idx), n, int(dim), int(id_bound), _ptr(uids),
+              _ptr(num_unique), _opt(inverse), _ptr(ws), ws.numel(), _stream())
+    return CombinePlan(n, int(dim), int(id_bound), uids, num_unique, inverse, workspace)
+
+
+def combine_apply(plan, grad, mode=COMBINE_FAST, out=None):
+    """Segmented row sums of `grad` under a plan.  Returns (uids, sums, cnts, num_unique) like
+    combine_padded; `out` = (sums float32[n, D], cnts int64[n]) to write into preallocated tensors."""
+    _dev(grad, "grad")
+    _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
+    _check(grad.size(0) == plan.n and grad.size(1) == plan.dim, "grad does not match the plan")
+    dev = grad.device
+    if out is None:
+        sums = torch.empty((plan.n, plan.dim), dtype=torch.float32, device=dev)
+        cnts = torch.empty(plan.n, dtype=torch.int64, device=dev)
+    else:
+        sums, cnts = out
+    ws = plan.workspace.get(_lib.query("hades_combine_workspace_bytes", plan.n, plan.dim))
+    _lib.call("hades_combine_apply", _ptr(grad), plan.n, plan.dim, plan.id_bound, int(mode),
+              _ptr(sums), _ptr(cnts), _ptr(plan.num_unique), _ptr(ws), ws.numel(), _stream())
+    return plan.uids, sums, cnts, plan.num_unique
+
+
 def combine(idx, grad, id_bound=0, mode=COMBINE_FAST, workspace=None):
     """As combine_padded, trimmed to the number of distinct ids (one host synchronisation)."""
     uids, sums, cnts, num_unique = combine_padded(idx, grad, id_bound, mode, workspace=workspace)

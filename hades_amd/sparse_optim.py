@@ -53,6 +53,7 @@ class _SparseRowOptimizer:
         self.hot_set = ops.HotSet(self.hot_ids)
         self.hot_w = self._gather_hot(weight_cold)
         self._ws = ops.Workspace(self.device)
+        self._side = None
 
     def _gather_hot(self, cold):
         """Hot copy of the rows named by hot_ids; a pinned host table is read zero-copy by the
@@ -82,11 +83,37 @@ class _SparseRowOptimizer:
         """Forward fetch of embedding rows (cached_fetch)."""
         return ops.cached_fetch(self.cold_w, self.hot_w, ids, self.hot_set, out=out)
 
-    def step(self, idx, grad, mode=ops.COMBINE_FAST):
+    def prepare(self, idx, stream=None, out=None):
+        """Starts the id-only half of the next step's combine (sort + run boundaries) on a side
+        stream and returns its plan.  The ids of a batch are known at forward time - the reference
+        saves them in its trace (python/EmbCache/dist_emb.py:276-288) - so this work can hide
+        behind the fetch and the model's forward/backward; step(..., plan=plan) waits for it.
+        One plan may be outstanding per optimizer (it lives in the optimizer's workspace)."""
+        cur = torch.cuda.current_stream()
+        if out is None:   # allocated on the caller's stream, which is where they are consumed
+            out = (torch.empty(idx.numel(), dtype=torch.int64, device=self.device),
+                   torch.empty(1, dtype=torch.int64, device=self.device))
+        if stream is None:
+            if self._side is None:
+                self._side = torch.cuda.Stream(device=self.device)
+            stream = self._side
+        # everything queued so far (the ids, and the previous step that used the workspace) first
+        stream.wait_stream(cur)
+        with torch.cuda.stream(stream):
+            plan = ops.combine_plan(idx, self.dim, id_bound=self.num_rows, workspace=self._ws,
+                                    out=out)
+            plan.ready = torch.cuda.Event()
+            plan.ready.record(stream)
+        return plan
+
+    def step(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None):
         """combine the per-occurrence gradients, then update every distinct row once.
-        No host synchronisation."""
-        uids, sums, cnts, nu = ops.combine_padded(idx, grad, id_bound=self.num_rows, mode=mode,
-                                                  workspace=self._ws)
+        No host synchronisation.  `plan` = what prepare(idx) returned, if it was called."""
+        if plan is None:
+            plan = ops.combine_plan(idx, self.dim, id_bound=self.num_rows, workspace=self._ws)
+        else:
+            torch.cuda.current_stream().wait_event(plan.ready)
+        uids, sums, cnts, nu = ops.combine_apply(plan, grad, mode, out=out)
         self.update(uids, sums, nu)
         return uids, sums, cnts, nu
 

@@ -220,6 +220,19 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
                   int mode, int64_t* uids, float* sums, int64_t* cnts, int64_t* num_unique,
                   int32_t* inverse, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same in two halves.  The sort and the run boundaries depend on the ids alone, which a
+ * trainer knows at forward time (python/EmbCache/dist_emb.py:276-288 saves them for the optimizer),
+ * long before the gradients exist: hades_combine_plan can run then, on another stream, and
+ * hades_combine_apply (the segmented row sums; also writes cnts) when the gradients arrive.
+ * The plan lives in the workspace: apply must get the same n, dim, id_bound and workspace, after the
+ * plan has finished, and the workspace must not be reused in between. */
+int hades_combine_plan(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bound, int64_t* uids,
+                       int64_t* num_unique, int32_t* inverse, void* workspace,
+                       size_t workspace_bytes, void* stream);
+int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bound, int mode,
+                        float* sums, int64_t* cnts, const int64_t* num_unique, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
 /* unique_grads (python/EmbCache/sparse_optim.py:142-157): in-place division of the first
  * num_unique[0] rows of sums by cnts (plus `one_plus` added to the divisor: the reference starts
  * the count from ones when a cnt vector is supplied, :145-148). */

@@ -287,6 +287,7 @@ CASES = [  # (n, dim, id space, kind)
     (32, 7, 10, "zipf"), (33, 128, 50, "zipf"), (1000, 64, 1, "same"), (4096, 128, 10**9, "distinct"),
     (5000, 100, 300, "zipf"), (20_000, 128, 2_400_000, "zipf"), (70_001, 260, 5000, "zipf"),
     (65_536, 64, 1_000_000, "zipf"),
+    (3000, 7, 3, "zipf"), (2500, 1, 2, "zipf"), (40_000, 128, 40, "zipf"),   # very long runs
 ]
 
 
@@ -514,3 +515,40 @@ def test_full_size_step_properties(lib):
     assert torch.equal(hot_changed, torch.sort(uloc[uloc >= 0]).values)
     g = sums[:U][uloc < 0]
     assert torch.equal(opt.cold_s[cold_u], g * g)      # first step from a zero accumulator
+
+
+def test_combine_plan_then_apply_and_side_stream_schedule(lib):
+    """The two halves of combine give what the whole gives; a plan made on a side stream while the
+    main stream fetches gives the same optimizer step as the one-stream order."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad
+    rng = np.random.default_rng(77)
+    n_rows, dim, n = 60_000, 64, 50_000
+    idx = zipfish(rng, n, n_rows)
+    grad = (rng.standard_normal((n, dim)) * 1e-3).astype(np.float32)
+    t_idx, t_grad = dev(idx), dev(grad)
+    for mode in (ops.COMBINE_EXACT, ops.COMBINE_FAST):
+        whole = ops.combine_padded(t_idx, t_grad, n_rows, mode)
+        plan = ops.combine_plan(t_idx, dim, n_rows)
+        halves = ops.combine_apply(plan, t_grad, mode)
+        U = int(whole[3].item())
+        assert U == int(halves[3].item())
+        for a, b in zip(whole[:3], halves[:3]):
+            assert torch.equal(a[:U], b[:U])
+    table = (rng.standard_normal((n_rows, dim)) * 0.01).astype(np.float32)
+    hot_ids = np.sort(rng.choice(n_rows, 6000, replace=False)).astype(np.int64)
+    a = SparseAdagrad(dev(table), torch.from_numpy(hot_ids))
+    b = SparseAdagrad(dev(table), torch.from_numpy(hot_ids))
+    for step in range(3):
+        idx = zipfish(rng, n, n_rows)
+        t_idx = dev(idx)
+        t_grad = dev((rng.standard_normal((n, dim)) * 1e-3).astype(np.float32))
+        a.fetch(t_idx)
+        a.step(t_idx, t_grad)
+        plan = b.prepare(t_idx)          # side stream
+        rows = b.fetch(t_idx)            # main stream, concurrently
+        b.step(t_idx, t_grad, plan=plan)
+        del rows
+    torch.cuda.synchronize()
+    for x, y in ((a.cold_w, b.cold_w), (a.cold_s, b.cold_s), (a.hot_w, b.hot_w), (a.hot_s, b.hot_s)):
+        assert torch.equal(x, y)
