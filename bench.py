@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
     ap.add_argument("--schedule", default="serial", choices=["serial", "overlap"],
                     help="serial: every kernel of the step on one stream (the default: measured "
@@ -256,6 +256,131 @@ def run_gpu(args):
     return wl, ms_per_step, roofline, extra
 
 
+def run_cfg4(args):
+    """Cold-gradient accumulator with a delayed write-back: every step combines a batch of cold
+    ids and adds the distinct rows to the hash table in HBM; every `flush_every` steps the live
+    entries leave the table in id order and go through sparse Adagrad on the pinned-host table.
+    Prints its own JSON line (the step is not the headline fetch+combine+update step)."""
+    import torch
+    from hades_amd import ops, synth
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = synth.CONFIGS["cfg4"]
+    N, D, H, n = cfg["num_rows"], cfg["dim"], cfg["num_hot"], cfg["batch"]
+    slots, every = cfg["num_slots"], cfg["flush_every"]
+    seed = 1234 + 4
+    nb = every
+    log("allocating the %d x %d pinned host table (%.1f GB)" % (N, D, N * D * 4 / 1e9))
+    cold_w = torch.empty((N, D), dtype=torch.float32, pin_memory=True)
+    log("filling it")
+    synth.fill_normal_(cold_w, 0.01, seed, progress=log)
+    cold_s = torch.zeros((N, D), dtype=torch.float32, device=dev)
+    log("sampling %d batches of %d cold ids" % (nb, n))
+    # a Zipf law of its own over the cold ranks: cold rank k is global rank H + k
+    sampler = synth.ZipfSampler(N - H, cfg["zipf_s"], dev)
+    ids = [synth.make_ids(sampler, N, n, seed * 1000 + b, rank_offset=H) for b in range(nb)]
+    grads = [synth.make_grads(n, D, seed * 2000 + b, dev) for b in range(nb)]
+    del sampler
+    acc = ops.ColdGradAccumulator(slots, D, id_bound=N, device=dev)
+    ws = ops.Workspace(dev)
+    comb_out = (torch.empty(n, dtype=torch.int64, device=dev),
+                torch.empty((n, D), dtype=torch.float32, device=dev),
+                torch.empty(n, dtype=torch.int64, device=dev),
+                torch.empty(1, dtype=torch.int64, device=dev))
+    cap = slots
+    flush_out = (torch.empty(cap, dtype=torch.int64, device=dev),
+                 torch.empty((cap, D), dtype=torch.float32, device=dev),
+                 torch.empty(cap, dtype=torch.int64, device=dev),
+                 torch.empty(1, dtype=torch.int64, device=dev))
+    log("workload ready")
+
+    def new_events(count):
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+        for e in evs:
+            e.record()
+        return evs
+
+    ev = [new_events(5) for _ in range(args.steps)]
+    kev = [new_events(2) for _ in range(args.steps)]
+    live_at_flush = []
+
+    def step(i, events=None):
+        q, g = ids[i % nb], grads[i % nb]
+        if events: events[0].record()
+        uids, sums, cnts, nu = ops.combine_padded(q, g, id_bound=N, workspace=ws, out=comb_out)
+        if events: events[1].record()
+        acc.accumulate(uids, sums, cnts, num_rows=nu)
+        if events: events[2].record()
+        if (i + 1) % every == 0:
+            fi, fs, fc, fn = acc.flush_padded(cap, out=flush_out)
+            if events: events[3].record()
+            ops.adagrad_update_(fi, fs, None, None, cold_w, cold_s, None, 0.01, 1e-10,
+                                num_unique=fn)
+            if events: events[4].record()
+            return fn
+        return None
+
+    warm = max(every, (args.warmup + every - 1) // every * every)   # ends on a flush
+    for i in range(warm):
+        step(i)
+    torch.cuda.synchronize()
+    assert int(acc.status.item()) == 0, "accumulator overflow during warm-up"
+    log("warm-up of %d steps done" % warm)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        ops.profile_kernel(ops.KERNEL_HASH_ACCUMULATE, kev[i][0], kev[i][1])
+        fn = step(i, ev[i])
+        if fn is not None:
+            live_at_flush.append(fn.clone())
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ops.profile_kernel(0)
+    assert int(acc.status.item()) == 0, "accumulator overflow"
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    K = args.steps
+    flush_steps = [i for i in range(K) if (i + 1) % every == 0]
+    comb_ms = sum(ev[i][0].elapsed_time(ev[i][1]) for i in range(K)) / K
+    acc_ms = sum(ev[i][1].elapsed_time(ev[i][2]) for i in range(K)) / K
+    kern_ms = sum(kev[i][0].elapsed_time(kev[i][1]) for i in range(K)) / K
+    U = sum(int(torch.unique(q).numel()) for q in ids) / nb
+    live = [int(x.item()) for x in live_at_flush]
+    L = sum(live) / max(1, len(live))
+    line = {
+        "metric": "cold gradient rows/s (combine + accumulate, flush + Adagrad write-back every %d steps)" % every,
+        "value": round(n / (ms_per_step * 1e-3), 1), "unit": "rows/s", "n_gpus": 1,
+        "steps": K, "warmup": warm, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cfg4: %d cold ids/step zipf s=%.2f over ranks %d..%d of a %d x %d "
+                               "pinned-host table, %d-slot accumulator in HBM, flush every %d steps"
+                               % (n, cfg["zipf_s"], H + 1, N, N, D, slots, every)},
+        "unique_per_step": round(U, 1), "live_keys_at_flush": round(L, 1),
+        "load_at_flush": round(L / slots, 4),
+        "phases": {"combine_ms": round(comb_ms, 4), "accumulate_ms": round(acc_ms, 4)},
+    }
+    # accumulate kernel: per distinct row 8 B id + 8 B count + 4D gradient read, 8 B key probe,
+    # 8 B count and 4D accumulator read-modify-write (2 x 4D)
+    kbytes = U * (16 + 4 * D + 8 + 16 + 8 * D)
+    achieved = kbytes / (kern_ms * 1e-3) / 1e9
+    line["roofline"] = {"bound": "hbm", "kernel": "hash_accumulate_kernel (hades_hash_accumulate)",
+                        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                        "kernel_us": round(kern_ms * 1e3, 2), "bytes_per_launch": int(kbytes)}
+    if flush_steps:
+        fl_ms = sum(ev[i][2].elapsed_time(ev[i][3]) for i in flush_steps) / len(flush_steps)
+        ap_ms = sum(ev[i][3].elapsed_time(ev[i][4]) for i in flush_steps) / len(flush_steps)
+        line["phases"]["flush_ms_per_flush"] = round(fl_ms, 4)
+        line["phases"]["apply_ms_per_flush"] = round(ap_ms, 4)
+        # flush: scan of all keys, then per live entry key+count+row out of the table, row zeroed,
+        # and id+count+row written
+        fbytes = slots * 8 + L * (16 + 4 * D) * 2 + L * 4 * D
+        line["flush_GB/s"] = round(fbytes / (fl_ms * 1e-3) / 1e9, 1)
+        line["pcie"] = {"apply_read_GB/s": round(L * 4 * D / (ap_ms * 1e-3) / 1e9, 2),
+                        "apply_write_GB/s": round(L * 4 * D / (ap_ms * 1e-3) / 1e9, 2),
+                        "peak_per_direction": PCIE_PEAK_GBS}
+    print(json.dumps(line))
+
+
 def run_cpu_baseline(wl_name, seconds):
     """The same step with the CPU oracle (torch CPU ops, all host threads), on a bounded sample:
     the benchmark's own batches at full table size when that fits the host, repeated for about
@@ -301,6 +426,9 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (the all-to-all "
               "gradient exchange is out of scope); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "cfg4":
+        run_cfg4(args)
+        return
     wl, ms_per_step, roofline, extra = run_gpu(args)
     n = wl.n
     line = {

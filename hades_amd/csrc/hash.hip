@@ -242,10 +242,11 @@ int hades_hash_accumulate(int64_t* keys, float* accum, int64_t* cnt, int64_t num
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec4 = dim % 4 == 0 && (align_of_ptr(accum) % 16) == 0 && (align_of_ptr(grad) % 16) == 0;
   if (vec4)
-    HADES_LAUNCH((hash_accumulate_kernel<4>), grid, block, 0, st, a);
+    HADES_LAUNCH_TIMED(HADES_KERNEL_HASH_ACCUMULATE, st, (hash_accumulate_kernel<4>), grid, block, 0,
+                       st, a);
   else
-    HADES_LAUNCH((hash_accumulate_kernel<1>), grid, block, 0, st, a);
-  HADES_LAUNCH_CHECK();
+    HADES_LAUNCH_TIMED(HADES_KERNEL_HASH_ACCUMULATE, st, (hash_accumulate_kernel<1>), grid, block, 0,
+                       st, a);
   return HADES_OK;
 }
 

@@ -62,6 +62,7 @@ KERNEL_CACHED_FETCH = _lib.KERNEL_CACHED_FETCH
 KERNEL_SEG_SUM = _lib.KERNEL_SEG_SUM
 KERNEL_ADAGRAD = _lib.KERNEL_ADAGRAD
 KERNEL_RADIX_PASS = _lib.KERNEL_RADIX_PASS
+KERNEL_HASH_ACCUMULATE = _lib.KERNEL_HASH_ACCUMULATE
 
 
 def profile_kernel(kernel_id, start=None, stop=None):
@@ -387,13 +388,19 @@ class ColdGradAccumulator:
                   self.num_slots, _ptr(ids), _ptr(grad), _opt(cnt), _opt(num_rows), ids.numel(),
                   self.dim, _ptr(self.status), _stream())
 
-    def flush_padded(self, cap):
-        """Returns (ids int64[cap], sums float32[cap, dim], cnts int64[cap], num_out int64[1])."""
+    def flush_padded(self, cap, out=None):
+        """Returns (ids int64[cap], sums float32[cap, dim], cnts int64[cap], num_out int64[1]);
+        `out` may bring these four tensors to avoid their allocation."""
         dev = self.device
-        out_ids = torch.empty(cap, dtype=torch.int64, device=dev)
-        out_sums = torch.empty((cap, self.dim), dtype=torch.float32, device=dev)
-        out_cnts = torch.empty(cap, dtype=torch.int64, device=dev)
-        num_out = torch.empty(1, dtype=torch.int64, device=dev)
+        if out is not None:
+            out_ids, out_sums, out_cnts, num_out = out
+            _check(out_ids.numel() >= cap and out_sums.size(0) >= cap and out_cnts.numel() >= cap,
+                   "flush outputs smaller than cap")
+        else:
+            out_ids = torch.empty(cap, dtype=torch.int64, device=dev)
+            out_sums = torch.empty((cap, self.dim), dtype=torch.float32, device=dev)
+            out_cnts = torch.empty(cap, dtype=torch.int64, device=dev)
+            num_out = torch.empty(1, dtype=torch.int64, device=dev)
         nbytes = _lib.query("hades_hash_flush_workspace_bytes", self.num_slots, cap)
         ws = self._ws.get(nbytes)
         _lib.call("hades_hash_flush", _ptr(self.keys), _ptr(self.accum), _ptr(self.cnt),

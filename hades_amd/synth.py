@@ -58,9 +58,11 @@ def hot_ids(num_rows, num_hot, device="cpu"):
     return torch.sort(rank_to_id(ranks, num_rows)).values
 
 
-def make_ids(sampler, num_rows, n, seed):
+def make_ids(sampler, num_rows, n, seed, rank_offset=0):
+    """n ids drawn from the sampler's ranks; rank_offset shifts them (H: a Zipf law of its own
+    over the cold ranks H+1..N)."""
     g = torch.Generator().manual_seed(seed)
-    return rank_to_id(sampler.sample_ranks(n, g), num_rows)
+    return rank_to_id(sampler.sample_ranks(n, g) + rank_offset, num_rows)
 
 
 def make_grads(n, dim, seed, device="cpu"):

@@ -64,7 +64,8 @@ int hades_version(void);
 #define HADES_KERNEL_SEG_SUM 2      /* segmented row sum of hades_combine (FAST: chunk kernel; EXACT: exact kernel) */
 #define HADES_KERNEL_ADAGRAD 3      /* hades_adagrad_update */
 #define HADES_KERNEL_RADIX_PASS 4   /* scatter passes of the sort in hades_combine (the pair keeps the last pass) */
-#define HADES_KERNEL_LAST 4
+#define HADES_KERNEL_HASH_ACCUMULATE 5 /* hades_hash_accumulate */
+#define HADES_KERNEL_LAST 5
 int hades_profile_kernel(int kernel_id, void* start_event, void* stop_event);
 
 /* ------------------------------------------------------------------------- */
