@@ -31,6 +31,7 @@ constexpr int kWaves = kThreads / kWave;
 constexpr int kRadixBits = 8;
 constexpr int kBins = 1 << kRadixBits;
 constexpr int kMaxPasses = 8;
+constexpr int kGroup = 4;  // tiles counted by one block of the count kernel
 
 // ---- key transforms ---------------------------------------------------------
 template <typename KeyT>
@@ -73,31 +74,43 @@ __device__ __forceinline__ uint64_t match_any(uint32_t v, int nbits, uint64_t am
 // ---- per-tile digit counts of one pass ------------------------------------------------------
 // counts layout: cnt[tile * kBins + digit].  (Counting the next pass's digits with global atomics
 // from inside the scatter was measured at twice the cost of this kernel.)
+// A block counts kGroup consecutive tiles and also writes their sum, gcnt[group * kBins + digit]:
+// the scatter then adds up one row per group plus the few tile rows inside its own group instead
+// of one row per tile.
 template <typename KeyT, bool FIRST, int IPT>
-__global__ __launch_bounds__(kThreads) void radix_count_kernel(
+__global__ __launch_bounds__(kGroup * kThreads) void radix_count_kernel(
     const void* __restrict__ keys_in, int64_t n, int shift, uint32_t mask,
-    uint32_t* __restrict__ cnt, int64_t id_bound, int32_t* __restrict__ status) {
-  __shared__ uint32_t s_hist[kBins];
-  for (int d = threadIdx.x; d < kBins; d += kThreads) s_hist[d] = 0;
+    uint32_t* __restrict__ cnt, uint32_t* __restrict__ gcnt, int64_t ntiles, int64_t id_bound,
+    int32_t* __restrict__ status) {
+  __shared__ uint32_t s_hist[kGroup][kBins];
+  const int g = threadIdx.x / kThreads;  // the tile of the group this thread counts
+  const int t = threadIdx.x % kThreads;  // kThreads == kBins: also the digit it writes out
+  s_hist[g][t] = 0;
   __syncthreads();
-  const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * (kThreads * IPT);
+  const int64_t tile = static_cast<int64_t>(blockIdx.x) * kGroup + g;
+  const int64_t tile0 = tile * (kThreads * IPT);
   bool bad = false;
 #pragma unroll
   for (int r = 0; r < IPT; ++r) {
-    const int64_t i = tile0 + r * kThreads + threadIdx.x;
+    const int64_t i = tile0 + r * kThreads + t;
     if (i < n) {
       if (FIRST) {
         const int64_t id = static_cast<const int64_t*>(keys_in)[i];
         bad = bad || (id_bound > 0 && (id < 0 || id >= id_bound));
       }
       const KeyT k = load_key<KeyT, FIRST>(keys_in, i);
-      atomicAdd(&s_hist[static_cast<uint32_t>(k >> shift) & mask], 1u);
+      atomicAdd(&s_hist[g][static_cast<uint32_t>(k >> shift) & mask], 1u);
     }
   }
   if (FIRST && bad) atomicOr(status, 1);
   __syncthreads();
-  for (int d = threadIdx.x; d < kBins; d += kThreads)
-    cnt[static_cast<int64_t>(blockIdx.x) * kBins + d] = s_hist[d];
+  if (tile < ntiles) cnt[tile * kBins + t] = s_hist[g][t];
+  if (g == 0) {
+    uint32_t sum = 0;
+#pragma unroll
+    for (int k = 0; k < kGroup; ++k) sum += s_hist[k][t];  // tiles past the end counted nothing
+    gcnt[static_cast<int64_t>(blockIdx.x) * kBins + t] = sum;
+  }
 }
 
 // ---- one radix pass ---------------------------------------------------------------------
@@ -106,8 +119,9 @@ __global__ __launch_bounds__(kThreads) void radix_count_kernel(
 template <typename KeyT, bool FIRST, int IPT>
 __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
     const void* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, int64_t n, int shift,
-    uint32_t mask, int bits, const uint32_t* __restrict__ cnt_cur, int64_t ntiles,
-    KeyT* __restrict__ keys_out, uint32_t* __restrict__ vals_out) {
+    uint32_t mask, int bits, const uint32_t* __restrict__ cnt_cur,
+    const uint32_t* __restrict__ gcnt, int64_t ngroups, KeyT* __restrict__ keys_out,
+    uint32_t* __restrict__ vals_out) {
   __shared__ uint32_t s_cnt[kWaves][kBins];
   __shared__ uint32_t s_glob[kBins];
   __shared__ uint32_t s_scan[kWaves + 1];
@@ -115,27 +129,45 @@ __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
 
+  // the tile's keys are requested first, so that their latency overlaps the column sums
+  const int64_t wave0 = static_cast<int64_t>(blockIdx.x) * (kThreads * IPT) + wave * (IPT * kWave);
+  KeyT key[IPT];
+  uint32_t val[IPT];
+#pragma unroll
+  for (int r = 0; r < IPT; ++r) {
+    const int64_t i = wave0 + r * kWave + lane;
+    const bool valid = i < n;
+    key[r] = valid ? load_key<KeyT, FIRST>(keys_in, i) : KeyT(0);
+    val[r] = valid ? (FIRST ? static_cast<uint32_t>(i) : vals_in[i]) : 0u;
+  }
+
   // global offset of (digit, this tile): all keys with a smaller digit, plus the keys with this
   // digit in the tiles before this one.  Thread d owns digit d (kThreads == kBins).
-  // The column sums are latency-bound: wave w takes the tiles t = w (mod kWaves), lane l the four
-  // digits 4l..4l+3 of a tile row as one 16-byte load, eight rows in flight.
+  // Rows to add up: one per group of tiles (all of them for the totals, those before this tile's
+  // group for the prefix), then the tile rows of this group before this tile.  The sums are
+  // latency-bound: wave w takes the rows v = w (mod kWaves), lane l the four digits 4l..4l+3 of a
+  // row as one 16-byte load, sixteen rows in flight.
   {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int kInFlight = 16;
     const int64_t me = blockIdx.x;
+    const int64_t my_group = me / kGroup;
+    const int64_t nrows = ngroups + (me - my_group * kGroup);
     u32x4 tot4 = {0, 0, 0, 0}, pre4 = {0, 0, 0, 0};
-    for (int64_t t = wave; t < ntiles; t += kWaves * 8) {
-      u32x4 h[8];
+    for (int64_t v0 = wave; v0 < nrows; v0 += kWaves * kInFlight) {
+      u32x4 h[kInFlight];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int64_t tt = t + static_cast<int64_t>(k) * kWaves;
-        h[k] = tt < ntiles ? reinterpret_cast<const u32x4*>(cnt_cur + tt * kBins)[lane]
-                           : u32x4{0, 0, 0, 0};
+      for (int k = 0; k < kInFlight; ++k) {
+        const int64_t v = v0 + static_cast<int64_t>(k) * kWaves;
+        const uint32_t* row = v < ngroups ? gcnt + v * kBins
+                                          : cnt_cur + (my_group * kGroup + (v - ngroups)) * kBins;
+        h[k] = v < nrows ? reinterpret_cast<const u32x4*>(row)[lane] : u32x4{0, 0, 0, 0};
       }
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int64_t tt = t + static_cast<int64_t>(k) * kWaves;
-        tot4 += h[k];
-        if (tt < me) pre4 += h[k];
+      for (int k = 0; k < kInFlight; ++k) {
+        const int64_t v = v0 + static_cast<int64_t>(k) * kWaves;
+        if (v < ngroups) tot4 += h[k];
+        if (v < my_group || v >= ngroups) pre4 += h[k];
       }
     }
     // s_cnt doubles as scratch here: rows 0..3 hold the per-wave totals; the per-wave prefixes
@@ -158,17 +190,12 @@ __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
   }
   __syncthreads();
 
-  const int64_t wave0 = static_cast<int64_t>(blockIdx.x) * (kThreads * IPT) + wave * (IPT * kWave);
-  KeyT key[IPT];
-  uint32_t val[IPT];
   uint32_t rank[IPT];
   const uint64_t lt_mask = (uint64_t(1) << lane) - 1;
 #pragma unroll
   for (int r = 0; r < IPT; ++r) {
     const int64_t i = wave0 + r * kWave + lane;
     const bool valid = i < n;
-    key[r] = valid ? load_key<KeyT, FIRST>(keys_in, i) : KeyT(0);
-    val[r] = valid ? (FIRST ? static_cast<uint32_t>(i) : vals_in[i]) : 0u;
     const uint32_t d = static_cast<uint32_t>(key[r] >> shift) & mask;
     const uint64_t peers = match_any(d, bits, __ballot(valid));
     uint32_t old = 0;
@@ -709,6 +736,7 @@ struct SortWs {
   void* keys[2];
   uint32_t* vals[2];
   uint32_t* cnt;        // [ntiles][kBins], rewritten by every pass
+  uint32_t* gcnt;       // [ceil(ntiles / kGroup)][kBins]: sums of kGroup consecutive rows of cnt
   int64_t cnt_len;
   size_t bytes;
 };
@@ -720,6 +748,7 @@ void carve_sort(Carver& c, int64_t n, SortWs* w) {
   for (int i = 0; i < 2; ++i) w->vals[i] = c.take<uint32_t>(nn);
   w->cnt_len = make_plan(nn, 1, 0, true).ntiles * kBins;  // the tile count depends on n only
   w->cnt = c.take<uint32_t>(w->cnt_len);
+  w->gcnt = c.take<uint32_t>(ceil_div(w->cnt_len / kBins, kGroup) * kBins);
   w->bytes = c.total();
 }
 
@@ -749,7 +778,9 @@ Ws carve(void* ws, int64_t n, int64_t dim) {
 template <typename KeyT, int IPT>
 int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
                  hipStream_t st, const void** keys_out, const uint32_t** perm_out) {
-  const dim3 grid(static_cast<unsigned>(p.ntiles)), block(kThreads);
+  const int64_t ngroups = ceil_div(p.ntiles, kGroup);
+  const dim3 grid(static_cast<unsigned>(p.ntiles)), cgrid(static_cast<unsigned>(ngroups)),
+      block(kThreads), cblock(kGroup * kThreads);
   const int base = p.key_bits / p.passes, extra = p.key_bits % p.passes;
   int bits_of[kMaxPasses], shift_of[kMaxPasses + 1];
   shift_of[0] = 0;
@@ -765,17 +796,17 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
     KeyT* kout = static_cast<KeyT*>(w.keys[cur]);
     uint32_t* vout = w.vals[cur];
     if (pass == 0) {
-      HADES_LAUNCH((radix_count_kernel<KeyT, true, IPT>), grid, block, 0, st, kin, n,
-                   shift_of[pass], mask, w.cnt, id_bound, w.status);
+      HADES_LAUNCH((radix_count_kernel<KeyT, true, IPT>), cgrid, cblock, 0, st, kin, n,
+                   shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.status);
       HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, true, IPT>), grid,
                          block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
-                         p.ntiles, kout, vout);
+                         w.gcnt, ngroups, kout, vout);
     } else {
-      HADES_LAUNCH((radix_count_kernel<KeyT, false, IPT>), grid, block, 0, st, kin, n,
-                   shift_of[pass], mask, w.cnt, id_bound, w.status);
+      HADES_LAUNCH((radix_count_kernel<KeyT, false, IPT>), cgrid, cblock, 0, st, kin, n,
+                   shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.status);
       HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, false, IPT>), grid,
                          block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
-                         p.ntiles, kout, vout);
+                         w.gcnt, ngroups, kout, vout);
     }
     kin = kout;
     vin = vout;
