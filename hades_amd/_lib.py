@@ -57,12 +57,15 @@ _SIGNATURES = {
     "hades_hash_clear": [_P, _P, _P, _L, _L, _P],
     "hades_hash_accumulate": [_P, _P, _P, _L, _P, _P, _P, _P, _L, _L, _P, _P],
     "hades_hash_flush": [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P, _P, c_size_t, _P],
+    "hades_bucket_by_owner": [_P, _L, _P, _L, _L, _L, _P, _L, c_int, _P, _P, _P, _P, _P, _P, _P,
+                              c_size_t, _P],
 }
 _SIZE_QUERIES = {
     "hades_split_compact_workspace_bytes": [_L],
     "hades_hot_index_bytes": [_L],
     "hades_combine_workspace_bytes": [_L, _L],
     "hades_hash_flush_workspace_bytes": [_L, _L],
+    "hades_bucket_workspace_bytes": [_L],
 }
 
 _lib = None

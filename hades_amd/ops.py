@@ -420,3 +420,51 @@ class ColdGradAccumulator:
             raise RuntimeError("cold-gradient accumulator overflow (status %d): table full or "
                                "flush capacity too small" % st)
         return ids[:n], sums[:n], cnts[:n]
+
+
+# ---- pre-exchange bucketing ------------------------------------------------------
+def bucket_by_owner(ids, grad=None, cnt=None, partition_range=None, local_num_gpus=1,
+                    num_owners=None, return_perm=False, workspace=None):
+    """Groups a batch by the rank that owns each id, as swap_gradients does before its all-to-all
+    (python/EmbCache/sparse_optim.py:33-50), without a host synchronisation.
+
+    owner = id % local_num_gpus, plus (index of the id's range in partition_range) * local_num_gpus
+    when a partition range is given.  Returns (ids_out, grad_out, cnt_out, split_sizes[, perm]):
+    the inputs stably sorted by owner (None where the input was None), split_sizes int64[num_owners]
+    on the device, and perm int64[n] (input position of every output row) when asked.
+    """
+    _i64(ids, "ids")
+    n = ids.numel()
+    dev = ids.device
+    if partition_range is not None:
+        _i64(partition_range, "partition_range")
+        num_part = partition_range.numel()
+        _check(num_part >= 1, "partition_range must not be empty")
+    else:
+        num_part = 0
+    if num_owners is None:
+        num_owners = max(1, num_part) * int(local_num_gpus)
+    dim, dcode = 1, _lib.F32
+    grad_out = cnt_out = perm = None
+    if grad is not None:
+        _dev(grad, "grad")
+        _check(grad.dim() == 2 and grad.size(0) == n, "grad must be [len(ids), dim]")
+        dim, dcode = grad.size(1), _dcode(grad)
+        grad_out = torch.empty_like(grad)
+    if cnt is not None:
+        _i64(cnt, "cnt")
+        _check(cnt.numel() == n, "cnt must have one entry per id")
+        cnt_out = torch.empty_like(cnt)
+    if return_perm:
+        perm = torch.empty(n, dtype=torch.int64, device=dev)
+    ids_out = torch.empty_like(ids)
+    split_sizes = torch.empty(int(num_owners), dtype=torch.int64, device=dev)
+    nbytes = _lib.query("hades_bucket_workspace_bytes", n)
+    ws = (workspace or _ws(dev, "bucket")).get(nbytes)
+    _lib.call("hades_bucket_by_owner", _ptr(ids), n, _opt(partition_range), num_part,
+              int(local_num_gpus), int(num_owners), _opt(grad), dim, dcode, _opt(cnt),
+              _ptr(ids_out), _opt(grad_out), _opt(cnt_out), _ptr(split_sizes), _opt(perm),
+              _ptr(ws), ws.numel(), _stream())
+    if return_perm:
+        return ids_out, grad_out, cnt_out, split_sizes, perm
+    return ids_out, grad_out, cnt_out, split_sizes

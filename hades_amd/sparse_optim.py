@@ -12,6 +12,18 @@ import torch
 from . import EmbCacheLib, ops
 
 
+def bucket_gradients(idics, grads, partition_range, num_parts, num_trainers_per_part,
+                     grads_cnt=None):
+    """The part of swap_gradients that precedes its all-to-all (python/EmbCache/sparse_optim.py:
+    33-62), argument names as there: ids, gradient rows and counts grouped by owning trainer, and
+    the per-trainer row counts.  Returns (ids, grads, grads_cnt, input_splits_tensor) with
+    input_splits_tensor int64[num_parts * num_trainers_per_part] on the device (the reference
+    then calls .tolist() on it for the exchange, :52)."""
+    num_owners = int(num_parts * num_trainers_per_part)
+    return ops.bucket_by_owner(idics, grads, grads_cnt, partition_range,
+                               int(num_trainers_per_part), num_owners)
+
+
 def only_unique_grads(idx, grad, id_bound=0, mode=ops.COMBINE_FAST):
     """(unique ids ascending, per-id summed float32 grads, per-id counts) - python/EmbCache/sparse_optim.py:132-139."""
     return ops.combine(idx, grad, id_bound=id_bound, mode=mode)

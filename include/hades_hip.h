@@ -288,6 +288,25 @@ int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slot
                      int64_t* num_out, int64_t cap, int32_t* status,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* Pre-exchange bucketing: what swap_gradients does on one GPU before the all-to-all
+ * (python/EmbCache/sparse_optim.py:33-50), in one call and without a host synchronisation:
+ *   owner[i] = ids[i] % local_num_gpus                               when range_partition == NULL (:36)
+ *            = (upper_bound(range_partition, ids[i]) - 1) * local_num_gpus
+ *              + ids[i] % local_num_gpus                             otherwise (:38-39)
+ *   stable sort by owner (:41); ids_out / cnt_out / grad_out = inputs in that order (:42-45);
+ *   split_sizes[g] = number of rows owned by g, g in [0, num_owners) (:48-52, int64 on the device)
+ *   perm_out[j] (optional) = input position of output row j.
+ * grad (dim columns of dtype) and cnt are optional, each together with its output.
+ * Rows keep their input order inside a bucket.  An owner outside [0, num_owners) sets bit 0 of the
+ * first workspace word and makes the result unspecified. */
+size_t hades_bucket_workspace_bytes(int64_t n);
+int hades_bucket_by_owner(const int64_t* ids, int64_t n, const int64_t* range_partition,
+                          int64_t num_part, int64_t local_num_gpus, int64_t num_owners,
+                          const void* grad, int64_t dim, int dtype, const int64_t* cnt,
+                          int64_t* ids_out, void* grad_out, int64_t* cnt_out,
+                          int64_t* split_sizes, int64_t* perm_out, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -70,6 +70,23 @@ def split_sizes(sorted_owner, num_owners):
     return ub
 
 
+def bucket_by_owner(ids, partition_range, local_num_gpus, num_owners, grad=None, cnt=None):
+    """The pre-exchange half of swap_gradients (python/EmbCache/sparse_optim.py:33-52): owner of
+    every id (cudaReminder without a partition range, cudaBinarySearch with one), sort by owner,
+    reorder ids / grads / counts, split sizes.  torch.sort(split) (:41) leaves the order of equal
+    owners unspecified; this restatement fixes it as the stable one (input order inside a bucket).
+    Returns (ids, grad, cnt, split_sizes, perm)."""
+    ids = np.asarray(ids, dtype=np.int64)
+    if partition_range is None:
+        owner = c_remainder(ids, local_num_gpus)
+    else:
+        owner = owner_rank(ids, np.asarray(partition_range, dtype=np.int64), local_num_gpus)
+    perm = np.argsort(owner, kind="stable").astype(np.int64)
+    sizes = split_sizes(owner[perm], num_owners)
+    return (ids[perm], None if grad is None else np.asarray(grad)[perm],
+            None if cnt is None else np.asarray(cnt)[perm], sizes, perm)
+
+
 # ---------------------------------------------------------------------------
 # lookup against the sorted hot set (closed form over BinarySearchKernel2)
 # ---------------------------------------------------------------------------

@@ -159,6 +159,59 @@ def test_routing_ops(lib, idt):
     assert E.cudaReminder(torch.empty(0, dtype=idt, device="cuda"), 4).numel() == 0
 
 
+# ---- pre-exchange bucketing (swap_gradients before its all-to-all) ---------------------------
+@pytest.mark.parametrize("n,num_part,local,dim,fdt", [
+    (10_001, 2, 4, 16, torch.float32),     # partition range, 8 owners
+    (50_000, 1, 8, 128, torch.float32),    # remainder only (partition_range=None)
+    (7_777, 5, 64, 3, torch.float64),      # 320 owners: two sort passes
+    (1, 1, 1, 4, torch.float32),           # one row, one owner
+    (300_000, 4, 8, 8, torch.float32),     # several tiles per group
+])
+def test_bucket_by_owner(lib, n, num_part, local, dim, fdt):
+    _, ops = lib
+    rng = np.random.default_rng(n + local)
+    n_rows = 3_000_000
+    ids = rng.integers(0, n_rows, n).astype(np.int64)
+    grad = rng.standard_normal((n, dim)).astype(NP_F[fdt])
+    cnt = rng.integers(1, 100, n).astype(np.int64)
+    ranged = num_part > 1
+    rp = np.array([i * n_rows // num_part for i in range(num_part + 1)], np.int64) if ranged else None
+    G = num_part * local
+    want = O.bucket_by_owner(ids, rp, local, G, grad, cnt)
+    got = ops.bucket_by_owner(dev(ids), dev(grad), dev(cnt), dev(rp) if ranged else None, local, G,
+                              return_perm=True)
+    for w, g in zip(want, got):
+        assert w.dtype == g.cpu().numpy().dtype and np.array_equal(w, g.cpu().numpy())
+    # ids only
+    ids_out, g_out, c_out, sizes = ops.bucket_by_owner(dev(ids), None, None,
+                                                       dev(rp) if ranged else None, local, G)
+    assert g_out is None and c_out is None
+    assert np.array_equal(ids_out.cpu().numpy(), want[0]) and np.array_equal(sizes.cpu().numpy(), want[3])
+
+
+def test_bucket_by_owner_reference_names_and_empty(lib):
+    _, ops = lib
+    from hades_amd import sparse_optim
+    rng = np.random.default_rng(77)
+    ids = rng.integers(0, 1000, 4096).astype(np.int64)
+    grad = rng.standard_normal((ids.size, 8)).astype(np.float32)
+    rp = np.array([0, 400, 1000], np.int64)
+    b_ids, b_grad, b_cnt, splits = sparse_optim.bucket_gradients(dev(ids), dev(grad), dev(rp), 2, 4)
+    want = O.bucket_by_owner(ids, rp, 4, 8, grad)
+    assert b_cnt is None
+    assert np.array_equal(b_ids.cpu().numpy(), want[0]) and np.array_equal(b_grad.cpu().numpy(), want[1])
+    assert splits.tolist() == want[3].tolist() and sum(splits.tolist()) == ids.size
+    # empty batch: all sizes zero (python/EmbCache/sparse_optim.py:54-62)
+    e_ids, e_grad, _, e_splits = ops.bucket_by_owner(
+        torch.empty(0, dtype=torch.int64, device="cuda"),
+        torch.empty((0, 8), dtype=torch.float32, device="cuda"), None, None, 4, 4)
+    assert e_ids.numel() == 0 and e_grad.shape == (0, 8) and e_splits.tolist() == [0, 0, 0, 0]
+    # an owner outside [0, num_owners) is reported in the workspace status word
+    ws = ops.Workspace("cuda")
+    ops.bucket_by_owner(dev(np.array([5, -3, 7], np.int64)), None, None, None, 4, 4, workspace=ws)
+    assert int(ws.buf[:4].view(torch.int32).item()) & 1
+
+
 # ---- lookup / split -----------------------------------------------------------------------
 @pytest.mark.parametrize("n,h", [(0, 10), (1, 1), (1000, 0), (4097, 511), (200_000, 48_000)])
 def test_lookup_sorted(lib, n, h):

@@ -53,6 +53,32 @@ def test_owner_rank_and_split_sizes_recipe():
     assert sizes.sum() == index.size
 
 
+@pytest.mark.parametrize("ranged", [False, True])
+def test_bucket_by_owner_is_the_reference_recipe_made_stable(ranged):
+    # swap_gradients (python/EmbCache/sparse_optim.py:33-52) with torch's own sort, stable
+    rng = np.random.default_rng(21)
+    num_part, local = (3, 4) if ranged else (1, 8)
+    ids = rng.integers(0, 90_000, size=5000).astype(np.int64)
+    grad = rng.standard_normal((ids.size, 4)).astype(np.float32)
+    cnt = rng.integers(1, 9, ids.size).astype(np.int64)
+    rp = np.array([i * 90_000 // num_part for i in range(num_part + 1)], np.int64) if ranged else None
+    G = num_part * local
+    b_ids, b_grad, b_cnt, sizes, perm = O.bucket_by_owner(ids, rp, local, G, grad, cnt)
+    split = torch.from_numpy(O.owner_rank(ids, rp, local) if ranged else O.c_remainder(ids, local))
+    value, indices = torch.sort(split, stable=True)
+    assert np.array_equal(perm, indices.numpy())
+    assert np.array_equal(b_ids, ids[indices.numpy()]) and np.array_equal(b_grad, grad[indices.numpy()])
+    assert np.array_equal(b_cnt, cnt[indices.numpy()])
+    assert np.array_equal(sizes, torch.bincount(split, minlength=G).numpy())
+    # brute force: bucket g holds exactly the rows owned by g, in input order
+    start = 0
+    for g in range(G):
+        rows = [i for i in range(ids.size) if int(split[i]) == g]
+        assert perm[start:start + len(rows)].tolist() == rows
+        start += len(rows)
+    assert start == ids.size
+
+
 # ---- lookup -----------------------------------------------------------------------
 def test_lookup_sorted_brute_force_and_edges():
     rng = np.random.default_rng(3)
