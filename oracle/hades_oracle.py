@@ -360,6 +360,110 @@ class ColdGradAccumulatorModel:
 
 
 # ---------------------------------------------------------------------------
+# set-associative index cache: src/cache/cache.h, src/cache/cache_line.h, src/cache/lookup.cu
+# ---------------------------------------------------------------------------
+class SACacheIndexModel:
+    """SACacheIndex<int64, int64> (src/cache/cache.h:11-259) over 8-entry lines
+    (CACHE_LINE_SIZE, src/cache/cache_line.h:5), batches processed in input order (the reference's
+    OpenMP loops give that order with one thread; with more, the outcome for ids that share a line
+    depends on thread timing).  Pure-Python loops: for small cases.  Ids must be >= 0
+    (`id % index_size` indexes the line array, cache.h:27).
+
+    State: ids[line, entry] (-1 = empty) and age[line, entry] (the access table)."""
+    LINE = 8
+
+    def __init__(self, cache_size):
+        self.lines = (int(cache_size) + self.LINE - 1) // self.LINE       # cache.h:139
+        self.ids = np.full((self.lines, self.LINE), -1, dtype=np.int64)    # cache_line.h:13-18
+        self.age = np.zeros((self.lines, self.LINE), dtype=np.int32)
+
+    def get_capacity(self):                                               # cache.h:187-189
+        return self.lines * self.LINE
+
+    def get_valid_entries_num(self):                                      # cache.h:180-185
+        return int((self.ids != -1).sum())
+
+    def _set_id(self, ln, e, v):                                          # cache_line.h:20-24
+        self.ids[ln, e] = v
+        self.age[ln, e] = 0
+
+    def _find(self, ln, v):                                               # cache_line.h:48-56
+        for e in range(self.LINE):
+            if self.ids[ln, e] == v:
+                return e
+        return -1
+
+    def add(self, ids):
+        """_add (cache.h:51-91): the id's entry if present; else the LAST empty entry of its line
+        (find_or_empty_entry keeps overwriting idx, cache_line.h:66-77); else the entry with the
+        largest non-zero age (find_lru, cache_line.h:91-102: strictly greater than entry 0's, so
+        ties go to the lowest entry), or -1 when every age is 0."""
+        ids = np.asarray(ids, dtype=np.int64)
+        locs = np.full(ids.shape, -1, dtype=np.int64)
+        for i, v in enumerate(ids.tolist()):
+            ln = v % self.lines
+            idx, exist = -1, False
+            for e in range(self.LINE):
+                cur = self.ids[ln, e]
+                if cur == v:
+                    idx, exist = e, True
+                    break
+                if cur == -1:
+                    idx = e
+            if idx >= 0:
+                if not exist:
+                    self._set_id(ln, idx, v)
+                locs[i] = ln * self.LINE + idx                            # compute_loc :31-33
+                continue
+            lru, tmp = 0, int(self.age[ln, 0])
+            for e in range(self.LINE):
+                a = int(self.age[ln, e])
+                if a > tmp and a != 0:
+                    lru, tmp = e, a
+            if tmp != 0:
+                self._set_id(ln, lru, v)
+                locs[i] = ln * self.LINE + lru
+        return locs
+
+    def lookup(self, ids):
+        """_lookup (cache.h:93-107): loc or -1; a hit ages every entry of the line by one and
+        zeroes the hit entry (access_loc, cache_line.h:79-85)."""
+        ids = np.asarray(ids, dtype=np.int64)
+        locs = np.full(ids.shape, -1, dtype=np.int64)
+        for i, v in enumerate(ids.tolist()):
+            ln = v % self.lines
+            e = self._find(ln, v)
+            if e >= 0:
+                locs[i] = ln * self.LINE + e
+                self.age[ln] += 1
+                self.age[ln, e] = 0
+        return locs
+
+    def cudalookup(self, ids):
+        """lookupkernel2 (src/cache/lookup.cu:15-45): the same search on a copy of the line, so no
+        aging; misses keep the -1 the output was filled with (cache.h:222-231)."""
+        ids = np.asarray(ids, dtype=np.int64)
+        ln = ids % self.lines
+        hit = self.ids[ln] == ids[:, None]
+        e = hit.argmax(axis=1)
+        return np.where(hit.any(axis=1), ln * self.LINE + e, -1).astype(np.int64)
+
+    def reset(self, ids):
+        """_reset (cache.h:109-121): an id that is present gives its entry back."""
+        for v in np.asarray(ids, dtype=np.int64).tolist():
+            ln = v % self.lines
+            e = self._find(ln, v)
+            if e >= 0:
+                self._set_id(ln, e, -1)
+
+    def getall(self, length):
+        """_getall (cache.h:123-137): live (id, loc) pairs in line order, at most `length`."""
+        flat = self.ids.reshape(-1)
+        locs = np.nonzero(flat != -1)[0][:length].astype(np.int64)
+        return flat[locs].copy(), locs
+
+
+# ---------------------------------------------------------------------------
 # the whole step, for smoke tests and the CPU baseline (torch CPU, as the reference's CPU path)
 # ---------------------------------------------------------------------------
 def torch_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps):

@@ -440,3 +440,56 @@ def test_torch_step_agrees_with_numpy_pieces():
     O.sparse_adagrad_step(cw, cs, hw, hs, hot, u, s, 0.01, 1e-10)
     for a, b in zip(t, (cw, cs, hw, hs)):
         assert np.allclose(a.numpy(), b, rtol=1e-5, atol=1e-9)
+
+
+# ---- set-associative index cache ------------------------------------------------------------
+def test_sacache_model_known_answers():
+    # worked by hand from src/cache/cache_line.h: 2 lines of 8 entries, ids with id % 2 == 0 -> line 0
+    m = O.SACacheIndexModel(16)
+    assert m.lines == 2 and m.get_capacity() == 16
+    # empty line: the LAST empty entry is taken (find_or_empty_entry keeps the last -1 it sees)
+    assert m.add([0, 2, 4]).tolist() == [7, 6, 5]
+    assert m.add([2]).tolist() == [6]                       # already present: same loc, no change
+    assert m.add([1]).tolist() == [8 + 7]                   # line 1
+    assert m.cudalookup([4, 6, 1, 3]).tolist() == [5, -1, 15, -1]
+    assert m.add([6, 8, 10, 12, 14]).tolist() == [4, 3, 2, 1, 0]     # line 0 now full
+    # nothing has been looked up yet: every age is 0 -> no victim -> -1
+    assert m.add([16]).tolist() == [-1]
+    # a hit ages every entry of the line by one and zeroes the hit
+    assert m.lookup([0, 0]).tolist() == [7, 7]
+    assert m.age[0].tolist() == [2, 2, 2, 2, 2, 2, 2, 0]
+    # victim: the largest non-zero age, ties to the lowest entry -> entry 0 (id 14)
+    assert m.add([16]).tolist() == [0]
+    assert m.cudalookup([14, 16]).tolist() == [-1, 0]
+    assert m.age[0].tolist() == [0, 2, 2, 2, 2, 2, 2, 0]
+    assert m.add([18]).tolist() == [1]                      # next victim: entry 1 (id 12)
+    m.reset([16, 99])                                       # absent ids are ignored
+    assert m.cudalookup([16]).tolist() == [-1] and m.get_valid_entries_num() == 8
+    assert m.add([20]).tolist() == [0]                      # the freed entry is reused
+    ids, locs = m.getall(100)
+    assert locs.tolist() == [0, 1, 2, 3, 4, 5, 6, 7, 15]
+    assert ids.tolist() == [20, 18, 10, 8, 6, 4, 2, 0, 1]
+    assert m.getall(3)[1].tolist() == [0, 1, 2]
+
+
+@pytest.mark.parametrize("cache_size,id_range,seed", [(64, 400, 1), (1000, 3000, 2), (8, 50, 3)])
+def test_sacache_model_matches_reference_cache_line(sacache_ref, cache_size, id_range, seed):
+    # the model against the reference's own cache_line class on random operation sequences
+    rng = np.random.default_rng(seed)
+    m, r = O.SACacheIndexModel(cache_size), sacache_ref(cache_size)
+    assert m.lines == r.lines
+    for step in range(60):
+        ids = rng.integers(0, id_range, int(rng.integers(1, 200))).astype(np.int64)
+        op = step % 4
+        if op == 0:
+            assert np.array_equal(m.add(ids), r.add(ids))
+        elif op == 1:
+            assert np.array_equal(m.lookup(ids), r.lookup(ids))
+        elif op == 2:
+            assert np.array_equal(m.cudalookup(ids), r.cudalookup(ids))
+            assert np.array_equal(m.add(np.unique(ids)), r.add(np.unique(ids)))
+        else:
+            m.reset(ids[:20]); r.reset(ids[:20])
+        assert m.get_valid_entries_num() == r.get_valid_entries_num()
+        a, b = m.getall(m.get_capacity()), r.getall(m.get_capacity())
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
