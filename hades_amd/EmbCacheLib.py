@@ -239,3 +239,12 @@ def cudaBinarySearch2(*args, **kwargs):
     _lib.call("hades_binary_search2", _ptr(in_), _ptr(range_), range_.size(0), _ptr(out),
               in_.size(0), _itype(in_, "in"), _stream())
     return out
+
+
+def __getattr__(name):
+    """EmbCacheLib.IndexCache (src/pybind.cc:17-36), resolved on first use: the class lives in
+    hades_amd.index_cache, which itself imports this module."""
+    if name == "IndexCache":
+        from .index_cache import IndexCache
+        return IndexCache
+    raise AttributeError("module %r has no attribute %r" % (__name__, name))

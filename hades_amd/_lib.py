@@ -59,6 +59,12 @@ _SIGNATURES = {
     "hades_hash_flush": [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P, _P, c_size_t, _P],
     "hades_bucket_by_owner": [_P, _L, _P, _L, _L, _L, _P, _L, c_int, _P, _P, _P, _P, _P, _P, _P,
                               c_size_t, _P],
+    "hades_sacache_init": [_P, _P, _L, _P],
+    "hades_sacache_add": [_P, _P, _L, _P, _L, _P, _P, c_size_t, _P],
+    "hades_sacache_lookup": [_P, _L, _P, _L, _P, _P],
+    "hades_sacache_lookup_touch": [_P, _P, _L, _P, _L, _P, _P, c_size_t, _P],
+    "hades_sacache_reset": [_P, _P, _L, _P, _L, _P],
+    "hades_sacache_getall": [_P, _L, _P, _P, _P, _P, _L, _P, c_size_t, _P],
 }
 _SIZE_QUERIES = {
     "hades_split_compact_workspace_bytes": [_L],
@@ -66,6 +72,8 @@ _SIZE_QUERIES = {
     "hades_combine_workspace_bytes": [_L, _L],
     "hades_hash_flush_workspace_bytes": [_L, _L],
     "hades_bucket_workspace_bytes": [_L],
+    "hades_sacache_workspace_bytes": [_L],
+    "hades_sacache_getall_workspace_bytes": [_L],
 }
 
 _lib = None

@@ -307,6 +307,38 @@ int hades_bucket_by_owner(const int64_t* ids, int64_t n, const int64_t* range_pa
                           int64_t* split_sizes, int64_t* perm_out, void* workspace,
                           size_t workspace_bytes, void* stream);
 
+/* Set-associative index cache on the device: SACacheIndex<int64, int64> of src/cache/cache.h:11-259
+ * over the 8-entry lines of src/cache/cache_line.h (bound as EmbCacheLib.IndexCache,
+ * src/pybind.cc:17-36).  State is two caller-owned device arrays:
+ *   line_ids int64[lines * 8]  (-1 = empty entry),  line_age int32[lines * 8]  (LRU ages);
+ * an id lives in line id % lines and its loc is line * 8 + entry.  Negative ids are never cached
+ * (loc -1).  Batches are handled in input order line by line, which is what the reference's
+ * loops give with one OpenMP thread.
+ *   init          constructor + _init_cache (cache.h:41-48, cache_line.h:13-18)
+ *   add           _add (cache.h:51-91): loc of each id after insertion, -1 if its line has no victim
+ *   lookup        lookupkernel2 (src/cache/lookup.cu:15-45): loc or -1, the cache is not changed
+ *   lookup_touch  _lookup (cache.h:93-107): loc or -1, a hit ages its line (access_loc)
+ *   reset         _reset (cache.h:109-121): ids that are present give their entry back
+ *   getall        _getall (cache.h:123-137) + get_valid_entries_ (:180-185): live (id, loc) pairs in
+ *                 loc order, at most cap; num_out[0] = pairs written, num_valid[0] = live entries
+ *                 (either may be NULL, not both) */
+int hades_sacache_init(int64_t* line_ids, int32_t* line_age, int64_t lines, void* stream);
+size_t hades_sacache_workspace_bytes(int64_t n); /* add and lookup_touch */
+int hades_sacache_add(int64_t* line_ids, int32_t* line_age, int64_t lines, const int64_t* ids,
+                      int64_t n, int64_t* locs, void* workspace, size_t workspace_bytes,
+                      void* stream);
+int hades_sacache_lookup(const int64_t* line_ids, int64_t lines, const int64_t* ids, int64_t n,
+                         int64_t* locs, void* stream);
+int hades_sacache_lookup_touch(int64_t* line_ids, int32_t* line_age, int64_t lines,
+                               const int64_t* ids, int64_t n, int64_t* locs, void* workspace,
+                               size_t workspace_bytes, void* stream);
+int hades_sacache_reset(int64_t* line_ids, int32_t* line_age, int64_t lines, const int64_t* ids,
+                        int64_t n, void* stream);
+size_t hades_sacache_getall_workspace_bytes(int64_t lines);
+int hades_sacache_getall(const int64_t* line_ids, int64_t lines, int64_t* ids_out,
+                         int64_t* locs_out, int64_t* num_out, int64_t* num_valid, int64_t cap,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

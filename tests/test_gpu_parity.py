@@ -212,6 +212,82 @@ def test_bucket_by_owner_reference_names_and_empty(lib):
     assert int(ws.buf[:4].view(torch.int32).item()) & 1
 
 
+# ---- set-associative index cache (EmbCacheLib.IndexCache) ----------------------------------
+def _same_cache_state(ic, model_or_ref):
+    cap = ic.get_capacity()
+    ids, locs, num = ic.getall_padded(cap)
+    k = int(num.item())
+    want_ids, want_locs = model_or_ref.getall(cap)
+    assert k == want_ids.size == model_or_ref.get_valid_entries_num() == ic.get_valid_entries_num()
+    assert np.array_equal(ids[:k].cpu().numpy(), want_ids)
+    assert np.array_equal(locs[:k].cpu().numpy(), want_locs)
+
+
+@pytest.mark.parametrize("cache_size,id_range,seed", [(64, 400, 1), (1000, 3000, 2), (8, 50, 3)])
+def test_index_cache_random_sequences_vs_model(lib, cache_size, id_range, seed):
+    import hades_amd.EmbCacheLib as E
+    rng = np.random.default_rng(seed)
+    ic, m = E.IndexCache(cache_size, "unused", True), O.SACacheIndexModel(cache_size)
+    assert ic.get_capacity() == m.get_capacity() and ic.get_size() == m.get_capacity()
+    assert ic.get_space() == m.lines * 96
+    for step in range(40):
+        ids = rng.integers(0, id_range, int(rng.integers(1, 300))).astype(np.int64)
+        op = step % 4
+        if op == 0:
+            assert np.array_equal(ic.add(dev(ids)).cpu().numpy(), m.add(ids))
+        elif op == 1:
+            assert np.array_equal(ic.lookup(dev(ids)).cpu().numpy(), m.lookup(ids))
+        elif op == 2:
+            assert np.array_equal(ic.cudalookup(dev(ids)).cpu().numpy(), m.cudalookup(ids))
+            u = np.unique(ids)
+            assert np.array_equal(ic.add(dev(u)).cpu().numpy(), m.add(u))
+        else:
+            ic.reset(dev(ids[:20])); m.reset(ids[:20])
+        _same_cache_state(ic, m)
+        assert np.array_equal(ic.line_age.cpu().numpy().reshape(-1, 8), m.age)
+
+
+def test_index_cache_known_answers_and_edges(lib):
+    from hades_amd.index_cache import LocalCache
+    t = lambda *v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    c = LocalCache("unused", 16, True)
+    assert c.get_num_entries() == 16
+    assert c.add(t(0, 2, 4)).tolist() == [7, 6, 5]           # last empty entry first
+    assert c.add(t(2)).tolist() == [6]
+    assert c.add(t(6, 8, 10, 12, 14)).tolist() == [4, 3, 2, 1, 0]
+    assert c.add(t(16)).tolist() == [-1]                     # full line, all ages 0: no victim
+    assert c.lookup(t(0, 0)).tolist() == [7, 7]
+    assert c.add(t(16)).tolist() == [0]                      # oldest entry, lowest index on ties
+    assert c.cudalookup(t(14, 16, 1, -5, -1)).tolist() == [-1, 0, -1, -1, -1]
+    assert c.add(t(-5, 18)).tolist() == [-1, 1]              # negative ids are never cached
+    c.reset(t(16, 99, -1))
+    assert c.cudalookup(t(16)).tolist() == [-1]
+    ids, locs = c._idx_cache.getall(3)
+    assert locs.tolist() == [1, 2, 3] and ids.tolist() == [18, 10, 8]
+    ids, locs = c._idx_cache.getall(12)                      # padded like the reference: 0 / -1
+    assert locs.tolist()[7:] == [-1] * 5 and ids.tolist()[7:] == [0] * 5
+    assert c.add(torch.empty(0, dtype=torch.int64, device="cuda")).numel() == 0
+
+
+@pytest.mark.parametrize("cache_size,id_range,batch", [(100_000, 1_000_000, 60_000),
+                                                       (4096, 50_000, 200_000)])
+def test_index_cache_large_vs_reference_cache_line(lib, sacache_ref, cache_size, id_range, batch):
+    # the reference's own cache_line class (oracle/_ref) on batches far larger than a line:
+    # long per-line sequences, evictions, re-insertions
+    import hades_amd.EmbCacheLib as E
+    rng = np.random.default_rng(cache_size)
+    ic, r = E.IndexCache(cache_size, "unused", True), sacache_ref(cache_size)
+    for step in range(6):
+        ids = rng.integers(0, id_range, batch).astype(np.int64)
+        assert np.array_equal(ic.add(dev(ids)).cpu().numpy(), r.add(ids))
+        probe = rng.integers(0, id_range, batch).astype(np.int64)
+        assert np.array_equal(ic.cudalookup(dev(probe)).cpu().numpy(), r.cudalookup(probe))
+        assert np.array_equal(ic.lookup(dev(probe)).cpu().numpy(), r.lookup(probe))
+        gone = np.unique(ids[: batch // 10])                  # reset takes distinct ids
+        ic.reset(dev(gone)); r.reset(gone)
+        _same_cache_state(ic, r)
+
+
 # ---- lookup / split -----------------------------------------------------------------------
 @pytest.mark.parametrize("n,h", [(0, 10), (1, 1), (1000, 0), (4097, 511), (200_000, 48_000)])
 def test_lookup_sorted(lib, n, h):
