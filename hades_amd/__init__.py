@@ -3,7 +3,9 @@
     hades_amd.EmbCacheLib   drop-in for the reference's extension module (same operator names)
     hades_amd.ops           fused operators: lookup, split, cached_fetch/set, combine, optimizers
     hades_amd.cache         EmbCache: hot-row cache keyed by the sorted hot-ID set
-    hades_amd.sparse_optim  only_unique_grads / unique_grads / SparseAdagrad / SparseAdam
+    hades_amd.sparse_optim  only_unique_grads / unique_grads / bucket_gradients / SparseAdagrad / SparseAdam
+    hades_amd.index_cache   IndexCache / LocalCache: the set-associative index cache, in HBM
+    hades_amd.cold_cache    ColdDataCache: the cache server's gradient path with its staleness rule
 
 All device work is done by csrc/libhades_hip.so (hand-written HIP, C ABI in include/hades_hip.h),
 built in-tree with `python -m hades_amd.build`.  There is no CPU fallback: without the library

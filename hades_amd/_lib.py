@@ -65,6 +65,10 @@ _SIGNATURES = {
     "hades_sacache_lookup_touch": [_P, _P, _L, _P, _L, _P, _P, c_size_t, _P],
     "hades_sacache_reset": [_P, _P, _L, _P, _L, _P],
     "hades_sacache_getall": [_P, _L, _P, _P, _P, _P, _L, _P, c_size_t, _P],
+    "hades_coldcache_insert": [_P, _P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _P],
+    "hades_coldcache_accumulate": [_P, _P, _P, _L, _L, _L, _L, _P, _P, _P, _P, _P, _P],
+    "hades_coldcache_flush": [_L, _L, c_int, _L, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P,
+                              _L, _P, c_size_t, _P],
 }
 _SIZE_QUERIES = {
     "hades_split_compact_workspace_bytes": [_L],
@@ -74,6 +78,7 @@ _SIZE_QUERIES = {
     "hades_bucket_workspace_bytes": [_L],
     "hades_sacache_workspace_bytes": [_L],
     "hades_sacache_getall_workspace_bytes": [_L],
+    "hades_coldcache_flush_workspace_bytes": [_L],
 }
 
 _lib = None

@@ -339,6 +339,44 @@ int hades_sacache_getall(const int64_t* line_ids, int64_t lines, int64_t* ids_ou
                          int64_t* locs_out, int64_t* num_out, int64_t* num_valid, int64_t cap,
                          void* workspace, size_t workspace_bytes, void* stream);
 
+/* Gradient side of the cold-data cache with the reference's per-row staleness rule: the
+ * arithmetic of the cache server over slot arrays in device memory.  A slot is a loc of the index
+ * cache above (remote part) or id - id_offset (dense local part, locs == NULL, grad_idx == NULL).
+ * Slot arrays: emb_buf / grad_buf float[num_slots, dim], grad_cnt / iter_count / iter_threshold
+ * int32[num_slots], grad_idx int64[num_slots].
+ *   insert      _update_cache (python/EmbCache/server.py:499-544): locs = what hades_sacache_add
+ *               returned for ids, line_ids = the index cache after that add.  For rows with
+ *               locs[r] >= 0 whose id holds that entry (an id evicted later in the same batch does
+ *               not): emb_buf[loc] = rows[r]; grad_buf[loc] = 0; grad_cnt[loc] = 0; grad_idx[loc] = -1
+ *   accumulate  _accumulate_gradients_cold_remote (:546-562) / _cold_local (:564-574): for rows
+ *               with a slot: grad_idx[s] = id; iter_threshold[s] = threshold[id] (if given);
+ *               grad_buf[s] += grad[r]; grad_cnt[s] += 1.  Rows must name distinct slots.
+ *   flush       _send_staled_gradients (:346-419, :421-497): slots with grad_cnt > 0 and
+ *               (iter_count >= iter_threshold or grad_cnt >= cnt_threshold) are written out in slot
+ *               order as (id, gradient row, count); they are zeroed, iter_count = 0, and their id is
+ *               taken out of the index cache (line_ids / line_age, may be NULL); every other slot
+ *               with grad_cnt > 0 ages by one.  num_out[0] = rows written (<= out_cap; if more were
+ *               due, bit 1 of the first workspace word is set and the rest leaves with the next
+ *               flush).
+ * The reference zeroes gradient rows through a temporary copy (:414, :489, :537), which leaves them
+ * unchanged; the evident intent, zeroing, is what these entry points do. */
+int hades_coldcache_insert(const int64_t* locs, const int64_t* ids, const int64_t* line_ids,
+                           const float* rows, int64_t n, int64_t dim, int64_t num_slots,
+                           float* emb_buf, float* grad_buf, int32_t* grad_cnt, int64_t* grad_idx,
+                           void* stream);
+int hades_coldcache_accumulate(const int64_t* locs, const int64_t* ids, const float* grad,
+                               int64_t n, int64_t dim, int64_t id_offset, int64_t num_slots,
+                               const int32_t* threshold, float* grad_buf, int32_t* grad_cnt,
+                               int64_t* grad_idx, int32_t* iter_threshold, void* stream);
+size_t hades_coldcache_flush_workspace_bytes(int64_t num_slots);
+int hades_coldcache_flush(int64_t num_slots, int64_t dim, int32_t cnt_threshold,
+                          int64_t id_offset, float* grad_buf, int32_t* grad_cnt,
+                          const int64_t* grad_idx, int32_t* iter_count,
+                          const int32_t* iter_threshold, int64_t* line_ids, int32_t* line_age,
+                          int64_t lines, int64_t* out_ids, float* out_grads, int64_t* out_cnts,
+                          int64_t* num_out, int64_t out_cap, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

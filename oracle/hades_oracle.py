@@ -463,6 +463,92 @@ class SACacheIndexModel:
         return flat[locs].copy(), locs
 
 
+class ColdCacheServerModel:
+    """Gradient path of EmbCacheServer (python/EmbCache/server.py) with the same torch CPU calls,
+    over SACacheIndexModel: _create_cache buffers (:76-166), _update_cache for one client
+    (:510-541), _accumulate_gradients_cold_remote (:546-562), _accumulate_gradients_cold_local
+    (:564-574) and both halves of _send_staled_gradients (:346-419, :421-497) up to the point
+    where rows are handed to the clients.  One deliberate difference: the reference's
+    `buf[index][:] = 0` (:414, :489, :537) assigns into a temporary and zeroes nothing; the rows
+    are zeroed here (the evident intent)."""
+
+    def __init__(self, cache_size, dim, hotness, cnt_threshold=16, part_start=0, part_nnodes=0):
+        hotness = torch.as_tensor(hotness, dtype=torch.float32)
+        self.cnt_threshold = int(cnt_threshold)
+        self.threshold = (1 / (0.001 + hotness)).ceil().int().clamp(max=100)      # :87-88
+        self.index = SACacheIndexModel(cache_size)
+        S = self.index.get_capacity()                                              # :98
+        self.emb = torch.zeros((S, dim))
+        self.grad = torch.zeros((S, dim))                                          # :108-112
+        self.cnt = torch.zeros(S, dtype=torch.int32)                               # :115-121
+        self.iter = torch.zeros(S, dtype=torch.int32)                              # :124-125
+        self.iter_thr = torch.zeros(S, dtype=torch.int32)                          # :127
+        self.idx = torch.full((S,), -1, dtype=torch.int64)                         # :132-139
+        self.part_start = int(part_start)
+        self.l_grad = torch.zeros((part_nnodes, dim))                              # :144-149
+        self.l_cnt = torch.zeros(part_nnodes, dtype=torch.int32)                   # :151-157
+        self.l_iter = torch.zeros(part_nnodes, dtype=torch.int32)                  # :160-161
+        self.l_thr = self.threshold[part_start:part_start + part_nnodes]           # :164-166
+
+    def update_cache(self, ids, embs):
+        ids, embs = torch.as_tensor(ids), torch.as_tensor(embs)
+        locs = torch.from_numpy(self.index.add(ids.numpy()))                       # :513
+        valid_index = torch.nonzero(locs >= 0).flatten()                           # :519-520
+        valid_locs = locs[valid_index]
+        # an id already cached at a loc and a later id of the batch that evicts it both report
+        # that loc; index assignment with a repeated index keeps the row written last, made
+        # explicit here (torch leaves the order of repeated indices unspecified)
+        _, first_rev = np.unique(valid_locs.numpy()[::-1], return_index=True)
+        keep = torch.from_numpy(np.sort(valid_locs.numel() - 1 - first_rev))
+        valid_index, valid_locs = valid_index[keep], valid_locs[keep]
+        self.emb[valid_locs] = embs[valid_index]                                   # :531
+        self.grad[valid_locs] = 0                                                  # :537 (intent)
+        self.cnt[valid_locs] = 0                                                   # :538
+        self.idx[valid_locs] = -1                                                  # :539
+        return locs.numpy()
+
+    def accumulate_gradients_cold_remote(self, id, grad):
+        id, grad = torch.as_tensor(id), torch.as_tensor(grad)
+        locs = torch.from_numpy(self.index.lookup(id.numpy()))                     # :550
+        cache_idx = torch.nonzero(locs >= 0).flatten()                             # :551-552
+        if cache_idx.numel() > 0:
+            tmp = locs[cache_idx]
+            self.idx[tmp] = id[cache_idx]                                          # :556
+            self.iter_thr[tmp] = self.threshold[id[cache_idx]]                     # :557
+            self.grad[tmp] += grad[cache_idx]                                      # :558
+            self.cnt[tmp] += 1                                                     # :559
+        return locs.numpy()
+
+    def accumulate_gradients_cold_local(self, id, grad):
+        id, grad = torch.as_tensor(id), torch.as_tensor(grad)
+        if id.numel() > 0:
+            local_id = id - self.part_start                                        # :569
+            self.l_grad[local_id] += grad                                          # :570
+            self.l_cnt[local_id] += 1                                              # :571
+
+    def _staled(self, grad, cnt, it, thr):
+        cnt_index = torch.nonzero(cnt > 0).flatten()                               # :350-351
+        mask = (it[cnt_index] >= thr[cnt_index]) | (cnt[cnt_index] >= self.cnt_threshold)  # :352-355
+        staled_index = cnt_index[mask]                                             # :357
+        out_grads = grad[staled_index].clone()                                     # :362
+        out_cnt = cnt[staled_index].long()                                         # :363, sent as int64 (:384-386)
+        grad[staled_index] = 0                                                     # :414 (intent)
+        cnt[staled_index] = 0                                                      # :415
+        it[cnt_index] += 1                                                         # :418
+        it[staled_index] = 0                                                       # :419
+        return staled_index, out_grads, out_cnt
+
+    def staled_gradients_remote(self):
+        staled_index, grads, cnts = self._staled(self.grad, self.cnt, self.iter, self.iter_thr)
+        ids = self.idx[staled_index].clone()                                       # :361
+        self.index.reset(ids.numpy())                                              # :413
+        return ids.numpy(), grads.numpy(), cnts.numpy()
+
+    def staled_gradients_local(self):
+        staled_index, grads, cnts = self._staled(self.l_grad, self.l_cnt, self.l_iter, self.l_thr)
+        return (staled_index + self.part_start).numpy(), grads.numpy(), cnts.numpy()   # :437
+
+
 # ---------------------------------------------------------------------------
 # the whole step, for smoke tests and the CPU baseline (torch CPU, as the reference's CPU path)
 # ---------------------------------------------------------------------------

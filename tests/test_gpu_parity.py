@@ -288,6 +288,75 @@ def test_index_cache_large_vs_reference_cache_line(lib, sacache_ref, cache_size,
         _same_cache_state(ic, r)
 
 
+# ---- cold-data cache: the server's gradient path with its staleness rule -------------------
+def _cold_state_equal(c, m):
+    assert np.array_equal(c.emb_cache_buff.cpu().numpy(), m.emb.numpy())
+    assert np.array_equal(c.grad_cache_buff.cpu().numpy(), m.grad.numpy())
+    assert np.array_equal(c.grad_cnt_cache_buff.cpu().numpy(), m.cnt.numpy())
+    assert np.array_equal(c.grad_iter_count.cpu().numpy(), m.iter.numpy())
+    live = m.cnt.numpy() > 0                       # ids and thresholds matter where gradients wait
+    assert np.array_equal(c.grad_idx_cache_buff.cpu().numpy()[live], m.idx.numpy()[live])
+    assert np.array_equal(c.grad_iter_threshold.cpu().numpy()[live], m.iter_thr.numpy()[live])
+    assert np.array_equal(c.index.line_ids.cpu().numpy().reshape(-1, 8), m.index.ids)
+    assert np.array_equal(c.index.line_age.cpu().numpy().reshape(-1, 8), m.index.age)
+
+
+@pytest.mark.parametrize("cache_size,n_ids,dim,seed", [(256, 600, 8, 1), (64, 2000, 128, 2),
+                                                       (1024, 1500, 3, 3)])
+def test_cold_data_cache_vs_server_model(lib, cache_size, n_ids, dim, seed):
+    from hades_amd.cold_cache import ColdDataCache
+    rng = np.random.default_rng(seed)
+    hotness = rng.choice([0.0, 0.02, 0.3, 1.0, 5.0], n_ids).astype(np.float32)
+    part_start, part_n = 100, 300
+    c = ColdDataCache(cache_size, dim, dev(hotness), cnt_threshold=3, part_start=part_start,
+                      part_nnodes=part_n)
+    m = O.ColdCacheServerModel(cache_size, dim, hotness, cnt_threshold=3, part_start=part_start,
+                               part_nnodes=part_n)
+    assert np.array_equal(c.threshold.cpu().numpy(), m.threshold.numpy())
+    for step in range(30):
+        if step % 3 == 0:                          # new rows arrive: evictions once the cache is full
+            ids = rng.choice(n_ids, int(rng.integers(1, cache_size)), replace=False).astype(np.int64)
+            embs = rng.standard_normal((ids.size, dim)).astype(np.float32)
+            assert np.array_equal(c.update_cache(dev(ids), dev(embs)).cpu().numpy(),
+                                  m.update_cache(ids, embs))
+        ids = rng.choice(n_ids, int(rng.integers(1, 400)), replace=False).astype(np.int64)
+        g = rng.standard_normal((ids.size, dim)).astype(np.float32)
+        assert np.array_equal(c.accumulate_gradients_cold_remote(dev(ids), dev(g)).cpu().numpy(),
+                              m.accumulate_gradients_cold_remote(ids, g))
+        lids = (part_start + rng.choice(part_n, int(rng.integers(1, 100)), replace=False)).astype(np.int64)
+        lg = rng.standard_normal((lids.size, dim)).astype(np.float32)
+        c.accumulate_gradients_cold_local(dev(lids), dev(lg))
+        m.accumulate_gradients_cold_local(lids, lg)
+        _cold_state_equal(c, m)
+        for got, want in ((c.staled_gradients_remote(), m.staled_gradients_remote()),
+                          (c.staled_gradients_local(), m.staled_gradients_local())):
+            for a, b in zip(got, want):
+                assert a.cpu().numpy().dtype == b.dtype and np.array_equal(a.cpu().numpy(), b)
+        _cold_state_equal(c, m)
+        assert np.array_equal(c.local_grad_buff.cpu().numpy(), m.l_grad.numpy())
+        assert np.array_equal(c.local_grad_cnt_buff.cpu().numpy(), m.l_cnt.numpy())
+        assert np.array_equal(c.local_grad_iter_count.cpu().numpy(), m.l_iter.numpy())
+
+
+def test_cold_data_cache_small_flush_capacity(lib):
+    # more rows due than the output holds: the rest stays due and leaves with the next flush
+    from hades_amd.cold_cache import ColdDataCache
+    rng = np.random.default_rng(5)
+    c = ColdDataCache(64, 4, torch.full((100,), 1000.0), cnt_threshold=1)
+    ids = np.arange(40, dtype=np.int64)
+    c.update_cache(dev(ids), dev(np.zeros((40, 4), np.float32)))
+    g = rng.standard_normal((40, 4)).astype(np.float32)
+    c.accumulate_gradients_cold_remote(dev(ids), dev(g))
+    a_ids, a_g, a_c, a_n = c.staled_gradients_remote_padded(cap=25)
+    b_ids, b_g, b_c, b_n = c.staled_gradients_remote_padded(cap=25)
+    assert int(a_n) == 25 and int(b_n) == 15
+    got = np.concatenate([a_ids[:25].cpu().numpy(), b_ids[:15].cpu().numpy()])
+    rows = np.concatenate([a_g[:25].cpu().numpy(), b_g[:15].cpu().numpy()])
+    order = np.argsort(got)
+    assert np.array_equal(got[order], ids) and np.array_equal(rows[order], g)
+    assert c.index.get_valid_entries_num() == 0 and int(c.grad_cnt_cache_buff.sum()) == 0
+
+
 # ---- lookup / split -----------------------------------------------------------------------
 @pytest.mark.parametrize("n,h", [(0, 10), (1, 1), (1000, 0), (4097, 511), (200_000, 48_000)])
 def test_lookup_sorted(lib, n, h):

@@ -493,3 +493,53 @@ def test_sacache_model_matches_reference_cache_line(sacache_ref, cache_size, id_
         assert m.get_valid_entries_num() == r.get_valid_entries_num()
         a, b = m.getall(m.get_capacity()), r.getall(m.get_capacity())
         assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+
+
+def test_cold_cache_server_model_against_per_id_bookkeeping():
+    # The slot-array model against plain per-id bookkeeping in a setting without evictions
+    # (at most 8 ids per line): what leaves at which flush, with which sum and count.
+    rng = np.random.default_rng(31)
+    n_ids, dim, lines = 400, 4, 64
+    ids_all = np.arange(n_ids, dtype=np.int64)                   # id % 64: 6-7 ids per line
+    hotness = rng.choice([0.0, 0.05, 0.3, 1.0, 5.0], n_ids).astype(np.float32)
+    thr = np.minimum(np.ceil(1.0 / (np.float32(0.001) + hotness)), 100).astype(np.int64)
+    m = O.ColdCacheServerModel(lines * 8, dim, hotness, cnt_threshold=3)
+    assert np.array_equal(m.threshold.numpy(), thr)
+    cached, pend, cnt, it = set(), {}, {}, {}
+    for step in range(60):
+        if step % 7 == 0:                                        # (re-)insert everything
+            locs = m.update_cache(ids_all, rng.standard_normal((n_ids, dim)).astype(np.float32))
+            assert (locs >= 0).all()
+            for i in range(n_ids):
+                cached.add(i); pend[i] = np.zeros(dim, np.float32); cnt[i] = 0; it.setdefault(i, 0)
+        batch = rng.choice(n_ids, 90, replace=False).astype(np.int64)
+        g = rng.standard_normal((batch.size, dim)).astype(np.float32)
+        locs = m.accumulate_gradients_cold_remote(batch, g)
+        for r, i in enumerate(batch.tolist()):
+            assert (locs[r] >= 0) == (i in cached)
+            if i in cached:
+                pend[i] = (pend[i] + g[r]).astype(np.float32); cnt[i] += 1
+        out_ids, out_g, out_c = m.staled_gradients_remote()
+        want = {}
+        for i in sorted(cached):
+            if cnt[i] > 0:
+                if it[i] >= thr[i] or cnt[i] >= 3:
+                    want[i] = (pend[i].copy(), cnt[i])
+                    pend[i][:] = 0; cnt[i] = 0; it[i] = 0
+                else:
+                    it[i] += 1
+        cached -= set(want)
+        assert sorted(out_ids.tolist()) == sorted(want)
+        for r, i in enumerate(out_ids.tolist()):
+            assert np.array_equal(out_g[r], want[i][0]) and out_c[r] == want[i][1]
+        assert m.index.get_valid_entries_num() == len(cached)
+    # the dense local part: same rule, ids = slot + part_start
+    m = O.ColdCacheServerModel(64, dim, hotness, cnt_threshold=2, part_start=100, part_nnodes=50)
+    lid = np.array([100, 149, 120], np.int64)
+    lg = rng.standard_normal((3, dim)).astype(np.float32)
+    m.accumulate_gradients_cold_local(lid, lg)
+    m.accumulate_gradients_cold_local(lid[:1], lg[:1])
+    out_ids, out_g, out_c = m.staled_gradients_local()
+    due0 = [int(i) for i in (120, 149) if thr[i] <= 0]           # first flush: iter 0 >= thr never
+    assert out_ids.tolist() == sorted([100] + due0)              # id 100 reached cnt_threshold
+    assert np.array_equal(out_g[0], (lg[0] + lg[0]).astype(np.float32)) and out_c[0] == 2
