@@ -1,6 +1,8 @@
 """Benchmark of the embedding-cache hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5] [--mode fast|exact]
+    python bench.py --workload cfg4          cold-gradient accumulator with delayed write-back
+    python bench.py --workload neighbours    pre-exchange bucketing, index cache, cold-data cache
 
 One step = lookup + cached_fetch of the query rows, combine of the per-query gradients, and the
 sparse Adagrad update of every distinct row, on one batch of synthetic Zipf ids that is already
@@ -38,7 +40,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
     ap.add_argument("--schedule", default="serial", choices=["serial", "overlap"],
                     help="serial: every kernel of the step on one stream (the default: measured "
@@ -399,6 +401,110 @@ def run_cfg4(args):
     print(json.dumps(line))
 
 
+def run_neighbours(args):
+    """The operators either side of the step, each timed on its own over `steps` calls after
+    `warmup` (wall clock around a synchronised loop, so launch overheads count): the pre-exchange
+    bucketing of a cfg5-sized batch, and the set-associative index cache / cold-data cache with
+    the staleness rule at cfg4's size.  Prints its own JSON line."""
+    import torch
+    from hades_amd import ops, synth
+    from hades_amd.cold_cache import ColdDataCache
+    from hades_amd.index_cache import IndexCache
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    K, W = args.steps, args.warmup
+
+    def timed(fn, setup=None):
+        for _ in range(W):
+            if setup: setup()
+            fn()
+        torch.cuda.synchronize()
+        total = 0.0
+        for _ in range(K):
+            if setup:
+                setup()
+                torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            total += time.perf_counter() - t0
+        return total / K * 1e3
+
+    out = {}
+    # ---- pre-exchange bucketing: 1 M ids x 64 floats, 4 machines x 8 trainers ----
+    cfg = synth.CONFIGS["cfg5"]
+    N, D, n = cfg["num_rows"], cfg["dim"], cfg["batch"] * cfg["trainers"]
+    sampler = synth.ZipfSampler(N, cfg["zipf_s"], dev)
+    ids = synth.make_ids(sampler, N, n, 99)
+    del sampler
+    grad = synth.make_grads(n, D, 98, dev)
+    cnt = torch.ones(n, dtype=torch.int64, device=dev)
+    rp = torch.tensor([i * N // 4 for i in range(5)], dtype=torch.int64, device=dev)
+    ws = ops.Workspace(dev)
+    ms = timed(lambda: ops.bucket_by_owner(ids, grad, cnt, rp, 8, 32, workspace=ws))
+    moved = n * (8 + 8 + 4 * D) * 2                       # ids, counts and rows read and written
+    out["bucket_by_owner"] = {"rows": n, "dim": D, "owners": 32, "ms": round(ms, 4),
+                              "rows/s": round(n / ms * 1e3, 1),
+                              "GB/s": round(moved / ms / 1e6, 1),
+                              "frac_hbm": round(moved / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    log("bucket_by_owner %.3f ms" % ms)
+    del grad, cnt
+
+    # ---- index cache: 4 M entries, 512 K-id batches of cold ids ----
+    c4 = synth.CONFIGS["cfg4"]
+    N4, H4, n4, D4 = c4["num_rows"], c4["num_hot"], c4["batch"], c4["dim"]
+    sampler = synth.ZipfSampler(N4 - H4, c4["zipf_s"], dev)
+    batches = [torch.unique(synth.make_ids(sampler, N4, n4, 500 + b, rank_offset=H4)) for b in range(4)]
+    del sampler
+    ic = IndexCache(c4["num_slots"], device=dev)
+    state = {"b": 0}
+
+    def nxt():
+        state["b"] = (state["b"] + 1) % len(batches)
+        return batches[state["b"]]
+    u = sum(b.numel() for b in batches) / len(batches)
+    ms_add = timed(lambda: ic.add(nxt()))
+    ms_look = timed(lambda: ic.cudalookup(nxt()))
+    ms_touch = timed(lambda: ic.lookup(nxt()))
+    out["index_cache"] = {"entries": ic.get_capacity(), "ids_per_call": round(u, 1),
+                          "valid_entries": ic.get_valid_entries_num(),
+                          "add_ms": round(ms_add, 4), "cudalookup_ms": round(ms_look, 4),
+                          "lookup_with_aging_ms": round(ms_touch, 4),
+                          "cudalookup_ids/s": round(u / ms_look * 1e3, 1),
+                          # per id: 8 B id + 64 B line + 8 B loc
+                          "cudalookup_GB/s": round(u * 80 / ms_look / 1e6, 1)}
+    log("index cache add %.3f lookup %.3f aging lookup %.3f ms" % (ms_add, ms_look, ms_touch))
+    del ic
+
+    # ---- cold-data cache: insert, accumulate and staleness flush at the same size ----
+    hot = torch.rand(N4, device=dev) * 0.2               # thresholds between 5 and 100 iterations
+    cc = ColdDataCache(c4["num_slots"], D4, hot, cnt_threshold=16)
+    del hot
+    rows = [synth.make_grads(b.numel(), D4, 700 + i, dev) for i, b in enumerate(batches)]
+
+    def pair():
+        state["b"] = (state["b"] + 1) % len(batches)
+        return batches[state["b"]], rows[state["b"]]
+    ms_ins = timed(lambda: cc.update_cache(*pair()))
+    ms_acc = timed(lambda: cc.accumulate_gradients_cold_remote(*pair()))
+    cap = c4["num_slots"]
+    ms_flush = timed(lambda: cc.staled_gradients_remote_padded(cap),
+                     setup=lambda: cc.accumulate_gradients_cold_remote(*pair()))
+    out["cold_data_cache"] = {"slots": cc.num_slots, "dim": D4, "rows_per_call": round(u, 1),
+                              "update_cache_ms": round(ms_ins, 4),
+                              "accumulate_ms": round(ms_acc, 4),
+                              "staleness_flush_ms": round(ms_flush, 4),
+                              # per accumulated row: gradient read, slot row read and written
+                              "accumulate_GB/s": round(u * 12 * D4 / ms_acc / 1e6, 1)}
+    log("cold cache insert %.3f accumulate %.3f flush %.3f ms" % (ms_ins, ms_acc, ms_flush))
+    line = {"metric": "neighbouring operators, ms per call", "unit": "ms", "n_gpus": 1,
+            "steps": K, "warmup": W, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "bucket_by_owner on a cfg5 batch; index cache and cold-data "
+                                   "cache at cfg4's size"}}
+    line.update(out)
+    print(json.dumps(line))
+
+
 def run_cpu_baseline(wl_name, seconds):
     """The same step with the CPU oracle (torch CPU ops, all host threads), on a bounded sample:
     the benchmark's own batches at full table size when that fits the host, repeated for about
@@ -446,6 +552,9 @@ def main():
         sys.exit(2)
     if args.workload == "cfg4":
         run_cfg4(args)
+        return
+    if args.workload == "neighbours":
+        run_neighbours(args)
         return
     wl, ms_per_step, roofline, extra = run_gpu(args)
     n = wl.n
