@@ -247,4 +247,7 @@ def __getattr__(name):
     if name == "IndexCache":
         from .index_cache import IndexCache
         return IndexCache
+    if name in ("create_shared_mem", "open_shared_mem", "release_shared_mem", "open_shared_tensor"):
+        from . import shm                      # src/pybind.cc:38-45
+        return getattr(shm, name)
     raise AttributeError("module %r has no attribute %r" % (__name__, name))

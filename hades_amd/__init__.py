@@ -6,6 +6,7 @@
     hades_amd.sparse_optim  only_unique_grads / unique_grads / bucket_gradients / SparseAdagrad / SparseAdam
     hades_amd.index_cache   IndexCache / LocalCache: the set-associative index cache, in HBM
     hades_amd.cold_cache    ColdDataCache: the cache server's gradient path with its staleness rule
+    hades_amd.shm           shared-memory segments and tensors, ShmTensorPool
 
 All device work is done by csrc/libhades_hip.so (hand-written HIP, C ABI in include/hades_hip.h),
 built in-tree with `python -m hades_amd.build`.  There is no CPU fallback: without the library

@@ -30,6 +30,10 @@ _SIGNATURES = {
     "hades_unpin": [_P],
     "hades_host_alloc": [ctypes.POINTER(c_void_p), c_size_t],
     "hades_host_free": [_P],
+    "hades_shm_create": [c_char_p, _L, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int64)],
+    "hades_shm_open": [c_char_p, _L, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int64)],
+    "hades_shm_release": [c_char_p, _L, _P, _L, c_int],
+    "hades_shm_exists": [c_char_p],
     "hades_fetch": [_P, _P, _P, _P, _L, _L, c_int, c_int, _P],
     "hades_fetch2": [_P, _P, _P, _L, _L, c_int, c_int, _P],
     "hades_fetch_with_cache2": [_P, _P, _P, _P, _P, _L, _L, c_int, c_int, _P],

@@ -83,6 +83,17 @@ int hades_unpin(void* host_ptr);
 int hades_host_alloc(void** out_ptr, size_t bytes);
 int hades_host_free(void* ptr);
 
+/* create_shared_mem / open_shared_mem / release_shared_mem (src/shm/shared_memory.h:14-58):
+ * a POSIX shared-memory segment mapped read-write; pin != 0 also registers the mapping with the
+ * HIP runtime (cudaHostRegister in the reference).  create sizes the segment, open refuses a
+ * segment smaller than `size`; release unregisters, unmaps, closes and unlinks.  On any failure
+ * nothing stays mapped, open or (for create) linked, and an error code comes back where the
+ * reference ends the process.  hades_shm_exists: SharedMemory::Exist (:104-112), 1 or 0. */
+int hades_shm_create(const char* name, int64_t size, int pin, void** out_ptr, int64_t* out_fd);
+int hades_shm_open(const char* name, int64_t size, int pin, void** out_ptr, int64_t* out_fd);
+int hades_shm_release(const char* name, int64_t size, void* ptr, int64_t fd, int pin);
+int hades_shm_exists(const char* name);
+
 /* cudaFetch: CUDAFetch (src/cuda/uva_fetch.cu:28-45)
  *   dst[dst_index[i], :] = src[src_index[i], :]            for i in [0, n) */
 int hades_fetch(const void* src, const void* src_index, void* dst, const void* dst_index,
