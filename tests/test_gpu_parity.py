@@ -715,6 +715,57 @@ def test_full_size_step_properties(lib):
     assert torch.equal(opt.cold_s[cold_u], g * g)      # first step from a zero accumulator
 
 
+def test_full_size_local_aggregation_and_accumulator_round_trip(lib):
+    """cfg5's shape (four trainers' 256 K-id batches over a 244 M-row id space, 64 columns) and
+    cfg4's (512 K cold ids per step into a 4 M-slot accumulator), through properties that need no
+    oracle: agreement with torch's own device unique / index_add_, combine(concat(batches)) ==
+    combine(concat(combine(batch_t))), and flush(accumulate(batches)) == combine(concat(batches))."""
+    _, ops = lib
+    from hades_amd import synth
+    c5 = synth.CONFIGS["cfg5"]
+    N, D, T, b = c5["num_rows"], c5["dim"], c5["trainers"], c5["batch"]
+    sampler = synth.ZipfSampler(N, c5["zipf_s"], "cuda")
+    qs = [synth.make_ids(sampler, N, b, 40 + t) for t in range(T)]
+    gs = [synth.make_grads(b, D, 50 + t, "cuda") for t in range(T)]
+    del sampler
+    q, g = torch.cat(qs), torch.cat(gs)
+    uids, sums, cnts = ops.combine(q, g, id_bound=N)
+    tu, tinv, tc = torch.unique(q, return_inverse=True, return_counts=True)
+    assert torch.equal(uids, tu) and torch.equal(cnts, tc) and int(cnts.sum()) == T * b
+    ref = torch.zeros((tu.numel(), D), dtype=torch.float64, device="cuda").index_add_(0, tinv, g.double())
+    scale = ref.abs().max().item()
+    assert (sums.double() - ref).abs().max().item() <= 1e-5 * scale
+    # two-level aggregation: per-trainer combine first, then the combine of the partial results
+    parts = [ops.combine(qs[t], gs[t], id_bound=N) for t in range(T)]
+    u2, s2, _ = ops.combine(torch.cat([p[0] for p in parts]), torch.cat([p[1] for p in parts]), id_bound=N)
+    assert torch.equal(u2, uids)
+    assert (s2.double() - ref).abs().max().item() <= 1e-5 * scale
+    del ref, sums, s2, parts, q, g, qs, gs
+
+    c4 = synth.CONFIGS["cfg4"]
+    N4, H4, D4, n4 = c4["num_rows"], c4["num_hot"], c4["dim"], c4["batch"]
+    sampler = synth.ZipfSampler(N4 - H4, c4["zipf_s"], "cuda")
+    acc = ops.ColdGradAccumulator(c4["num_slots"], D4, id_bound=N4, device="cuda")
+    all_ids, all_g, all_c = [], [], []
+    for step in range(c4["flush_every"]):
+        ids = synth.make_ids(sampler, N4, n4, 60 + step, rank_offset=H4)
+        grad = synth.make_grads(n4, D4, 70 + step, "cuda")
+        u, s, c = ops.combine(ids, grad, id_bound=N4, mode=ops.COMBINE_EXACT)
+        acc.accumulate(u, s, c)
+        all_ids.append(u); all_g.append(s); all_c.append(c)
+    f_ids, f_sums, f_cnts = acc.flush()
+    cat_ids, cat_g, cat_c = torch.cat(all_ids), torch.cat(all_g), torch.cat(all_c)
+    tu, tinv = torch.unique(cat_ids, return_inverse=True)
+    assert torch.equal(f_ids, tu) and (f_ids >= 0).all()
+    want_c = torch.zeros(tu.numel(), dtype=torch.int64, device="cuda").index_add_(0, tinv, cat_c)
+    assert torch.equal(f_cnts, want_c) and int(f_cnts.sum()) == c4["flush_every"] * n4
+    # one add per slot per step in step order: the same float32 chain as combining the
+    # concatenated per-step results in EXACT mode
+    e_ids, e_sums, _ = ops.combine(cat_ids, cat_g, id_bound=N4, mode=ops.COMBINE_EXACT)
+    assert torch.equal(e_ids, f_ids) and torch.equal(e_sums, f_sums)
+    assert acc.flush()[0].numel() == 0                      # the table is empty again
+
+
 def test_combine_plan_then_apply_and_side_stream_schedule(lib):
     """The two halves of combine give what the whole gives; a plan made on a side stream while the
     main stream fetches gives the same optimizer step as the one-stream order."""
