@@ -559,8 +559,11 @@ __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
 // EXACT: strictly left to right from +0.0f, one accumulator chain per id.
 // Runs shorter than kLongRun: one lane group per distinct id.  Longer runs (a heavy-hitter id can
 // have tens of thousands of occurrences) are left to seg_exact_long_kernel.
-constexpr int kLongRun = kThreads;
-constexpr int kLongRows = 16;  // rows every lane group stages per batch in the long-run kernel
+constexpr int kLongRun = 64;    // shortest run the long-run kernel takes
+constexpr int kLongThreads = 1024;  // the long-run kernel's block: one CU has to pull a whole run
+                                    // through, so it keeps as many row loads in flight as it can
+constexpr int kLongRows = 8;    // rows every lane group stages per batch in the long-run kernel
+constexpr int kLongSlice = 32;  // floats of a row one block of the long-run kernel sums (128 bytes)
 
 template <int VEC>
 __global__ __launch_bounds__(kThreads) void seg_exact_kernel(SegArgs a) {
@@ -599,13 +602,13 @@ __global__ __launch_bounds__(kThreads) void seg_exact_kernel(SegArgs a) {
 // EXACT, long runs: block c takes the run that begins inside positions [c*kLongRun, (c+1)*kLongRun)
 // and is at least kLongRun long (there is at most one: it must cover the last position of that
 // span).  All lane groups of the block stage rows into LDS, kLongRows each per batch, with the
-// next batch's loads already in flight; lane group 0 alone adds the staged rows in order, so the
-// sum is the same single chain ((0 + g1) + g2) + ... as for a short run.
+// next batch's loads already in flight; one thread per float column adds the staged rows in order,
+// so every element's sum is the same single chain ((0 + g1) + g2) + ... as for a short run.
 template <int VEC>
-__global__ __launch_bounds__(kThreads) void seg_exact_long_kernel(SegArgs a) {
+__global__ __launch_bounds__(kLongThreads) void seg_exact_long_kernel(SegArgs a) {
   typedef typename RowVec<VEC>::type V;
   extern __shared__ __align__(16) unsigned char s_raw[];
-  V* s_rows = reinterpret_cast<V*>(s_raw);   // [ngroups * kLongRows][G]
+  V* s_rows = reinterpret_cast<V*>(s_raw);   // [rows of a batch][kLongSlice floats]
   const int64_t c = blockIdx.x;
   const int64_t span0 = c * kLongRun;
   if (span0 >= a.n) return;
@@ -615,63 +618,70 @@ __global__ __launch_bounds__(kThreads) void seg_exact_long_kernel(SegArgs a) {
   const int64_t end = a.seg_start[u + 1];
   if (start < span0 || end - start < kLongRun) return;
 
-  const int G = a.group;
-  const int ngroups = kThreads / G;
+  // A block takes a 32-float slice of the columns (blockIdx.y): every element's chain is
+  // independent of the other columns, and one CU alone cannot pull whole rows of a long run fast
+  // enough, so the slices of a run are summed on different CUs at once.
+  constexpr int G = kLongSlice / VEC;          // lanes per row slice
+  constexpr int ngroups = kLongThreads / G;
+  constexpr int batch = ngroups * kLongRows;
   const int g = threadIdx.x / G;
   const int gl = threadIdx.x & (G - 1);
-  const int batch = ngroups * kLongRows;
-  for (int ct = 0; ct < a.col_tiles; ++ct) {
-    const int64_t col = (static_cast<int64_t>(ct) * G + gl) * VEC;
-    const bool col_ok = col < a.dim;
-    V acc = RowVec<VEC>::zero();
-    V row[kLongRows];
-    // rows of a batch are dealt to the groups in blocks of kLongRows: group g stages batch rows
-    // [g*kLongRows, (g+1)*kLongRows)
-    // Two loads deep: while batch b is added, the rows of batch b+1 and the sort positions of
-    // batch b+2 are in flight.
-    uint32_t pos[kLongRows];
-    auto load_pos = [&](int64_t base) {
+  const int64_t col = static_cast<int64_t>(blockIdx.y) * kLongSlice + gl * VEC;
+  const bool col_ok = col < a.dim;
+  // the adders: thread t < kLongSlice owns one float column of the slice and adds the staged
+  // rows in order - one dependent add per row and lane
+  const float* s_f = reinterpret_cast<const float*>(s_raw);
+  float accf = 0.f;
+  V row[kLongRows];
+  // rows of a batch are dealt to the groups in blocks of kLongRows: group g stages batch rows
+  // [g*kLongRows, (g+1)*kLongRows)
+  // Two loads deep: while batch b is added, the rows of batch b+1 and the sort positions of
+  // batch b+2 are in flight.
+  uint32_t pos[kLongRows];
+  auto load_pos = [&](int64_t base) {
 #pragma unroll
-      for (int k = 0; k < kLongRows; ++k) {
-        int64_t j = base + g * kLongRows + k;
-        if (j >= end) j = end - 1;
-        pos[k] = a.perm[j];
-      }
-    };
-    auto issue_rows = [&]() {
-#pragma unroll
-      for (int k = 0; k < kLongRows; ++k)
-        row[k] = col_ok ? __builtin_nontemporal_load(reinterpret_cast<const V*>(
-                              a.grad + static_cast<int64_t>(pos[k]) * a.dim + col))
-                        : RowVec<VEC>::zero();
-    };
-    load_pos(start);
-    issue_rows();
-    load_pos(start + batch);
-    for (int64_t base = start; base < end; base += batch) {
-#pragma unroll
-      for (int k = 0; k < kLongRows; ++k) s_rows[(g * kLongRows + k) * G + gl] = row[k];
-      __syncthreads();
-      if (base + batch < end) {
-        issue_rows();
-        load_pos(base + 2 * batch);
-      }
-      if (g == 0) {
-        const int64_t left = end - base;
-        const int rows_here = left < batch ? static_cast<int>(left) : batch;
-        int r = 0;
-        for (; r + 16 <= rows_here; r += 16) {   // LDS reads issued 16 at a time, adds in order
-          V t[16];
-#pragma unroll
-          for (int k = 0; k < 16; ++k) t[k] = s_rows[(r + k) * G + gl];
-#pragma unroll
-          for (int k = 0; k < 16; ++k) acc += t[k];
-        }
-        for (; r < rows_here; ++r) acc += s_rows[r * G + gl];
-      }
-      __syncthreads();
+    for (int k = 0; k < kLongRows; ++k) {
+      int64_t j = base + g * kLongRows + k;
+      if (j >= end) j = end - 1;
+      pos[k] = a.perm[j];
     }
-    if (g == 0 && col_ok) *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(u) * a.dim + col) = acc;
+  };
+  auto issue_rows = [&]() {
+#pragma unroll
+    for (int k = 0; k < kLongRows; ++k)
+      row[k] = col_ok ? __builtin_nontemporal_load(reinterpret_cast<const V*>(
+                            a.grad + static_cast<int64_t>(pos[k]) * a.dim + col))
+                      : RowVec<VEC>::zero();
+  };
+  load_pos(start);
+  issue_rows();
+  load_pos(start + batch);
+  for (int64_t base = start; base < end; base += batch) {
+#pragma unroll
+    for (int k = 0; k < kLongRows; ++k) s_rows[(g * kLongRows + k) * G + gl] = row[k];
+    __syncthreads();
+    if (base + batch < end) {
+      issue_rows();
+      load_pos(base + 2 * batch);
+    }
+    if (threadIdx.x < kLongSlice) {
+      const int64_t left = end - base;
+      const int rows_here = left < batch ? static_cast<int>(left) : batch;
+      int r = 0;
+      for (; r + 16 <= rows_here; r += 16) {   // LDS reads issued 16 at a time, adds in order
+        float t[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) t[k] = s_f[(r + k) * kLongSlice + threadIdx.x];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) accf += t[k];
+      }
+      for (; r < rows_here; ++r) accf += s_f[r * kLongSlice + threadIdx.x];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x < kLongSlice) {
+    const int64_t c_out = static_cast<int64_t>(blockIdx.y) * kLongSlice + threadIdx.x;
+    if (c_out < a.dim) a.sums[static_cast<int64_t>(u) * a.dim + c_out] = accf;
   }
 }
 
@@ -945,15 +955,23 @@ int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bo
     // short runs, then the long ones; the timing hook brackets the pair
     const bool timed = g_profile.kernel_id == HADES_KERNEL_SEG_SUM;
     if (timed) HADES_HIP_TRY(hipEventRecord(g_profile.start, st));
-    const dim3 lgrid(static_cast<unsigned>(ceil_div(n, kLongRun)));
+    const dim3 lgrid(static_cast<unsigned>(ceil_div(n, kLongRun)),
+                     static_cast<unsigned>(ceil_div(dim, kLongSlice)));
     if (p.vec == 4) {
+      // 128 KB of dynamic LDS: above the default limit, which has to be raised once
+      constexpr int kLongLds = kLongThreads * kLongRows * sizeof(f32x4);  // a batch of row slices
+      static bool raised = false;
+      if (!raised) {
+        HADES_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&seg_exact_long_kernel<4>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, kLongLds));
+        raised = true;
+      }
       HADES_LAUNCH((seg_exact_kernel<4>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
-      HADES_LAUNCH((seg_exact_long_kernel<4>), lgrid, dim3(kThreads),
-                   kThreads * kLongRows * sizeof(f32x4), st, a);
+      HADES_LAUNCH((seg_exact_long_kernel<4>), lgrid, dim3(kLongThreads), kLongLds, st, a);
     } else {
       HADES_LAUNCH((seg_exact_kernel<1>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
-      HADES_LAUNCH((seg_exact_long_kernel<1>), lgrid, dim3(kThreads),
-                   kThreads * kLongRows * sizeof(float), st, a);
+      HADES_LAUNCH((seg_exact_long_kernel<1>), lgrid, dim3(kLongThreads),
+                   kLongThreads * kLongRows * sizeof(float), st, a);
     }
     if (timed) HADES_HIP_TRY(hipEventRecord(g_profile.stop, st));
   } else {
