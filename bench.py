@@ -248,6 +248,8 @@ def run_gpu(args):
                 "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.mode, dominant)),
                 "kernel_us": round(kernel_ms * 1e3, 2),
                 "launches_timed": "%d of the %d in the timed region" % (len(sampled), args.steps),
+                "timing": "HIP events recorded on the launch stream right before and after the "
+                          "launch: the kernel plus about 3 us of dispatch latency",
                 "bytes_per_launch": int(kernel_bytes[dominant]),
                 "other_kernels_us": {kernels[k]: round(probe_ms[k] * 1e3, 2) for k in kernels
                                      if k != dominant}}
