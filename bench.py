@@ -42,10 +42,12 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
-    ap.add_argument("--schedule", default="serial", choices=["serial", "overlap"],
+    ap.add_argument("--schedule", default="serial", choices=["serial", "overlap", "graph"],
                     help="serial: every kernel of the step on one stream (the default: measured "
                          "faster); overlap: the sort of the ids runs on a side stream next to the "
-                         "fetch")
+                         "fetch; graph: every step is the replay of a HIP graph captured once per "
+                         "batch (no kernel inside a replay can be bracketed with events, so the "
+                         "roofline time is taken from eager steps before the timed region)")
     ap.add_argument("--batches", type=int, default=4, help="distinct pre-generated id batches")
     ap.add_argument("--event-every", type=int, default=4,
                     help="bracket every n-th launch of the dominant kernel with HIP events inside "
@@ -199,19 +201,45 @@ def run_gpu(args):
     # here and the per-phase events are taken in a second, untimed pass over the same steps.
     every = max(1, args.event_every)
     sampled = [i for i in range(args.steps) if i % every == 0]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        if i % every == 0:
-            ops.profile_kernel(dominant, kev[i][0], kev[i][1])
-        elif i % every == 1:
-            ops.profile_kernel(0)
-        step(i)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ops.profile_kernel(0)
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    kernel_ms = sum(kev[i][0].elapsed_time(kev[i][1]) for i in sampled) / len(sampled)
+    if args.schedule == "graph":
+        # one captured graph per pre-generated batch (the library allocates nothing and clears
+        # memory with kernels only, so a step captures as it is); launches inside a replay cannot
+        # be bracketed, so the dominant kernel's time is that of the eager probe steps above
+        graphs = []
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for b in range(nb):
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=side):
+                    step(b)
+                graphs.append(gr)
+        torch.cuda.current_stream().wait_stream(side)
+        for b in range(nb):
+            graphs[b].replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            graphs[i % nb].replay()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ms_per_step = (t1 - t0) * 1e3 / args.steps
+        kernel_ms = probe_ms[dominant]
+        sampled = []
+    else:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            if i % every == 0:
+                ops.profile_kernel(dominant, kev[i][0], kev[i][1])
+            elif i % every == 1:
+                ops.profile_kernel(0)
+            step(i)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ops.profile_kernel(0)
+        ms_per_step = (t1 - t0) * 1e3 / args.steps
+        kernel_ms = sum(kev[i][0].elapsed_time(kev[i][1]) for i in sampled) / len(sampled)
 
     for i in range(args.steps):
         step(i, ev[i])
@@ -247,7 +275,8 @@ def run_gpu(args):
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.mode, dominant)),
                 "kernel_us": round(kernel_ms * 1e3, 2),
-                "launches_timed": "%d of the %d in the timed region" % (len(sampled), args.steps),
+                "launches_timed": ("%d of the %d in the timed region" % (len(sampled), args.steps)
+                                   if sampled else "3 eager steps before the timed region"),
                 "timing": "HIP events recorded on the launch stream right before and after the "
                           "launch: the kernel plus about 3 us of dispatch latency",
                 "bytes_per_launch": int(kernel_bytes[dominant]),
@@ -577,7 +606,9 @@ def main():
         "config": {"workload": wl.describe(), "combine_mode": args.mode,
                    "optimizer": "sparse Adagrad lr=0.01 eps=1e-10",
                    "schedule": "sort of the step's ids on a side stream, concurrent with its fetch"
-                   if args.schedule == "overlap" else "one stream"},
+                   if args.schedule == "overlap" else
+                   "one stream, every step replayed from a HIP graph captured once per batch"
+                   if args.schedule == "graph" else "one stream"},
         "roofline": roofline,
     }
     line.update(extra)

@@ -766,6 +766,70 @@ def test_full_size_local_aggregation_and_accumulator_round_trip(lib):
     assert acc.flush()[0].numel() == 0                      # the table is empty again
 
 
+def test_step_replayed_from_a_hip_graph_matches_eager(lib):
+    """The library allocates nothing, synchronises nothing and clears memory with kernels only, so
+    a whole step can be captured once and replayed.  Every replay - with fresh inputs copied into
+    the captured buffers and eager work of the same library in between - must give exactly what
+    the eager step gives from the same state."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad
+    rng = np.random.default_rng(77)
+    N, D, H, n = 50_000, 64, 5_000, 20_000
+    table0 = torch.from_numpy((rng.standard_normal((N, D)) * 0.01).astype(np.float32)).cuda()
+    hot_ids = torch.from_numpy(np.sort(rng.choice(N, H, replace=False)).astype(np.int64)).cuda()
+    batches = [(dev(zipfish(rng, n, N)), dev((rng.standard_normal((n, D)) * 1e-3).astype(np.float32)))
+               for _ in range(4)]
+
+    def make():
+        opt = SparseAdagrad(table0.clone(), hot_ids, lr=0.01, eps=1e-10)
+        bufs = dict(rows=torch.empty((n, D), device="cuda"),
+                    comb=(torch.empty(n, dtype=torch.int64, device="cuda"),
+                          torch.empty((n, D), device="cuda"),
+                          torch.empty(n, dtype=torch.int64, device="cuda"),
+                          torch.empty(1, dtype=torch.int64, device="cuda")))
+        return opt, bufs
+
+    def step(opt, bufs, q, g):
+        ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_set, out=bufs["rows"])
+        plan = ops.combine_plan(q, D, id_bound=N, workspace=opt._ws,
+                                out=(bufs["comb"][0], bufs["comb"][3]))
+        uids, sums, cnts, nu = ops.combine_apply(plan, g, ops.COMBINE_FAST,
+                                                 out=(bufs["comb"][1], bufs["comb"][2]))
+        opt.update(uids, sums, nu)
+
+    eager, ebufs = make()
+    graphed, gbufs = make()
+    q_in, g_in = batches[0][0].clone(), batches[0][1].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(graphed, gbufs, q_in, g_in)           # warm-up on the capture stream: workspaces exist
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step(graphed, gbufs, q_in, g_in)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    # the warm-up changed the graphed optimizer once with batch 0: bring the eager one level
+    step(eager, ebufs, *batches[0])
+    for i in range(6):
+        q, g = batches[i % 4]
+        step(eager, ebufs, q, g)
+        q_in.copy_(q); g_in.copy_(g)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(gbufs["rows"], ebufs["rows"])
+        u = int(ebufs["comb"][3].item())
+        assert int(gbufs["comb"][3].item()) == u
+        for k in range(3):
+            assert torch.equal(gbufs["comb"][k][:u], ebufs["comb"][k][:u])
+        for name in ("cold_w", "cold_s", "hot_w", "hot_s"):
+            assert torch.equal(getattr(graphed, name), getattr(eager, name)), (i, name)
+        # eager work of the same library between replays
+        ops.lookup(q, graphed.hot_set)
+        ops.combine(q[:1000], g[:1000], id_bound=N)
+
+
 def test_combine_plan_then_apply_and_side_stream_schedule(lib):
     """The two halves of combine give what the whole gives; a plan made on a side stream while the
     main stream fetches gives the same optimizer step as the one-stream order."""
