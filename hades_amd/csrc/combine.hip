@@ -13,7 +13,9 @@
 //      through LDS and writes them out.
 //   2. run boundaries -> uids, seg_start, seg_of (index of the run every sorted position is in).
 //   3. segmented sum of the gradient rows:
-//        EXACT: one lane group per distinct id walks its rows left to right.
+//        EXACT: one lane group per distinct id walks its rows left to right; a run of 64 rows or
+//               more is staged through LDS by 1024-thread blocks, one per 32-float column slice,
+//               and added in the same order by one thread per column.
 //        FAST : the sorted sequence is cut into fixed chunks of 32 positions per lane group; a
 //               block stages the sort permutation of its groups in LDS, every group sums its
 //               runs left to right with 16 row loads in flight, runs that cross group borders
@@ -22,6 +24,8 @@
 //               order.  Work per group is uniform whatever the id skew; the shape of the sum
 //               depends only on (n, dim), so results are reproducible run to run.
 #include "internal.h"
+
+#include <atomic>
 
 namespace hades {
 namespace {
@@ -958,13 +962,16 @@ int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bo
     const dim3 lgrid(static_cast<unsigned>(ceil_div(n, kLongRun)),
                      static_cast<unsigned>(ceil_div(dim, kLongSlice)));
     if (p.vec == 4) {
-      // 128 KB of dynamic LDS: above the default limit, which has to be raised once
+      // 128 KB of dynamic LDS: above the default limit, which has to be raised once per device
       constexpr int kLongLds = kLongThreads * kLongRows * sizeof(f32x4);  // a batch of row slices
-      static bool raised = false;
-      if (!raised) {
+      static std::atomic<uint64_t> raised{0};  // bit d: done on device d
+      int device = 0;
+      HADES_HIP_TRY(hipGetDevice(&device));
+      const uint64_t bit = uint64_t(1) << (device & 63);
+      if (!(raised.load(std::memory_order_acquire) & bit)) {
         HADES_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&seg_exact_long_kernel<4>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLongLds));
-        raised = true;
+        raised.fetch_or(bit, std::memory_order_release);
       }
       HADES_LAUNCH((seg_exact_kernel<4>), dim3((unsigned)blocks), dim3(kThreads), 0, st, a);
       HADES_LAUNCH((seg_exact_long_kernel<4>), lgrid, dim3(kLongThreads), kLongLds, st, a);
