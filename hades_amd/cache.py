@@ -7,7 +7,7 @@ rows (88.8 MB instead of 888 MB at 111 M rows), and with the lookup fused into t
 """
 import torch
 
-from . import ops
+from . import EmbCacheLib, ops
 
 
 def select_hot_ids(hotness, num_hot, candidate_ids=None):
@@ -44,12 +44,18 @@ class EmbCache:
         self.hot_ids = hot_ids.to(self.device)
         self.hot_set = ops.HotSet(self.hot_ids)
         self.hot = []
-        cpu_ids = hot_ids.cpu()
         for t in self.cold:
             if t.is_cuda:
                 self.hot.append(t[self.hot_ids].contiguous())
             else:
-                self.hot.append(t[cpu_ids].to(self.device))
+                # a pinned host table is read zero-copy by the gather kernel, not indexed on the CPU
+                hot = torch.empty((self.hot_ids.numel(),) + tuple(t.shape[1:]), dtype=t.dtype,
+                                  device=self.device)
+                if t.dtype in (torch.float32, torch.float64):
+                    EmbCacheLib.cudaFetch2(t, self.hot_ids, hot)
+                else:
+                    hot.copy_(t[hot_ids.cpu()])
+                self.hot.append(hot)
         self.num_rows = self.cold[0].size(0)
         self._count_hit = count_hit
         self._hit_num = 0
@@ -95,5 +101,8 @@ class EmbCache:
         for cold, hot in zip(self.cold, self.hot):
             if cold.is_cuda:
                 cold[self.hot_ids] = hot
+            elif cold.dtype in (torch.float32, torch.float64):
+                EmbCacheLib.cudaSet(hot, cold, self.hot_ids)     # scatter into the pinned table
+                torch.cuda.current_stream().synchronize()        # the host may read it next
             else:
                 cold[self.hot_ids.cpu()] = hot.cpu()

@@ -766,6 +766,48 @@ def test_full_size_local_aggregation_and_accumulator_round_trip(lib):
     assert acc.flush()[0].numel() == 0                      # the table is empty again
 
 
+@pytest.mark.parametrize("pinned", [False, True])
+def test_emb_cache_state_tables(lib, pinned):
+    """EmbCache over the three tables of the reference's state cache (step [N], mem [N, D],
+    power [N, D]; python/EmbCache/cache.py:66-131): budgeted hotness placement, getitem / setitem
+    against plain indexing of a merged reference copy, hit rate, write-back."""
+    from hades_amd.cache import EmbCache
+    rng = np.random.default_rng(9)
+    N, D = 20_000, 32
+    mk = (lambda *s: torch.zeros(*s, pin_memory=True)) if pinned else (lambda *s: torch.zeros(*s, device="cuda"))
+    tables = [mk(N), mk(N, D), mk(N, D)]
+    for t in tables:
+        t.copy_(torch.from_numpy(rng.standard_normal(tuple(t.shape)).astype(np.float32)))
+    ref = [t.clone().cpu().numpy() for t in tables]
+    hotness = torch.from_numpy(rng.random(N).astype(np.float32))
+    item = 4 + 4 * D + 4 * D + 8
+    cache = EmbCache.create_cache(tables, hotness, alloca_mem_size=3000 * item + 5, count_hit=True)
+    want_hot = O.select_hot_ids(hotness, 3000)
+    assert np.array_equal(cache.hot_ids.cpu().numpy(), want_hot)
+    for step in range(3):
+        q = rng.integers(0, N, 4000).astype(np.int64)
+        got = cache[dev(q)]
+        for k in range(3):
+            assert np.array_equal(got[k].cpu().numpy(), ref[k][q])
+        u = np.unique(rng.integers(0, N, 3000)).astype(np.int64)
+        vals = [rng.standard_normal((u.size,) + r.shape[1:]).astype(np.float32) for r in ref]
+        cache[dev(u)] = tuple(dev(v) for v in vals)
+        for k in range(3):
+            ref[k][u] = vals[k]
+    hits = sum(int(np.isin(q_, want_hot).sum()) for q_ in [q])      # last batch, as a sanity bound
+    assert 0.0 < cache.get_hit_rate() < 1.0 and hits > 0
+    # cached rows live in the hot copy only until written back
+    torch.cuda.synchronize()
+    hot_changed = np.isin(u, want_hot)
+    if hot_changed.any():
+        k0 = u[hot_changed][0]
+        assert not np.array_equal(tables[1][k0].cpu().numpy(), ref[1][k0])
+    cache.write_back()
+    torch.cuda.synchronize()
+    for k in range(3):
+        assert np.array_equal(tables[k].cpu().numpy(), ref[k])
+
+
 def test_step_replayed_from_a_hip_graph_matches_eager(lib):
     """The library allocates nothing, synchronises nothing and clears memory with kernels only, so
     a whole step can be captured once and replayed.  Every replay - with fresh inputs copied into
