@@ -165,3 +165,17 @@ class SparseAdam(_SparseRowOptimizer):
         ops.adam_update_(uids, grad, (self.hot_w, self.hot_step, self.hot_m, self.hot_v),
                          (self.cold_w, self.cold_step, self.cold_m, self.cold_v), self.hot_set,
                          self.lr, self.betas[0], self.betas[1], self.eps, num_unique)
+
+    def update_like_reference(self, idx, grad, cnt=None, is_unique=False, mode=ops.COMBINE_FAST):
+        """The reference's SparseAdam.update(idx, grad, emb, cnt, is_unique)
+        (python/EmbCache/sparse_optim.py:590-685) on this optimizer's table: duplicate ids get
+        the MEAN of their gradient rows (unique_grads, :613; with `cnt` the divisor is one plus
+        the summed counts, :145-148), already-unique input is divided by `cnt` if given (:607-611);
+        then one Adam step on every distinct row.  Returns the distinct ids."""
+        if is_unique:
+            uids = idx
+            vals = grad if cnt is None else grad / cnt.unsqueeze(1)
+        else:
+            uids, vals = unique_grads(idx, grad, cnt, id_bound=self.num_rows, mode=mode)
+        self.update(uids, vals.contiguous())
+        return uids

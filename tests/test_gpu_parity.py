@@ -637,6 +637,50 @@ def test_adam_update(lib):
             assert np.allclose(got, want, rtol=1e-6, atol=1e-12)
 
 
+@pytest.mark.parametrize("variant", ["duplicates", "duplicates_cnt", "unique_cnt"])
+def test_sparse_adam_like_reference(lib, variant):
+    """SparseAdam.update_like_reference against the reference's update restated by the oracle:
+    unique_grads (mean over duplicates, the count quirk with cnt) or the is_unique branch, then
+    adam_rows on the gathered rows (python/EmbCache/sparse_optim.py:590-685)."""
+    from hades_amd.sparse_optim import SparseAdam
+    rng = np.random.default_rng(17)
+    n_rows, h, dim = 6000, 800, 32
+    w = (rng.standard_normal((n_rows, dim)) * 0.01).astype(np.float32)
+    st = np.zeros(n_rows, np.float32); m = np.zeros_like(w); v = np.zeros_like(w)
+    hot_ids = np.sort(rng.choice(n_rows, h, replace=False)).astype(np.int64)
+    opt = SparseAdam(dev(w), dev(hot_ids), lr=0.01, betas=(0.9, 0.999), eps=1e-8)
+    for _ in range(3):
+        idx = zipfish(rng, 2500, n_rows)
+        if variant == "unique_cnt":
+            idx = np.unique(idx)
+        g = (rng.standard_normal((idx.size, dim)) * 1e-2).astype(np.float32)
+        cnt = None if variant == "duplicates" else rng.integers(1, 6, idx.size).astype(np.int64)
+        if variant == "unique_cnt":
+            u, vals = idx, g / cnt[:, None].astype(np.float32)                  # :607-611
+        else:
+            tu, tv = O.unique_grads(idx, g, cnt)                                # :613
+            u, vals = tu.numpy(), tv.numpy()
+        w[u], st[u], m[u], v[u] = O.adam_rows(w[u], st[u], m[u], v[u], vals, 0.01, 0.9, 0.999, 1e-8)
+        got_u = opt.update_like_reference(dev(idx), dev(g), None if cnt is None else dev(cnt),
+                                          is_unique=(variant == "unique_cnt"), mode=ops_exact(lib))
+        assert np.array_equal(got_u.cpu().numpy(), u)
+    torch.cuda.synchronize()
+    for k, (cold, hot, want) in enumerate(((opt.cold_w, opt.hot_w, w), (opt.cold_step, opt.hot_step, st),
+                                           (opt.cold_m, opt.hot_m, m), (opt.cold_v, opt.hot_v, v))):
+        got = cold.cpu().numpy().copy()
+        got[hot_ids] = hot.cpu().numpy()
+        if k == 0:
+            assert np.abs(got - want).max() <= 1e-4 * 0.01      # as in test_adam_update
+        elif k == 1:
+            assert np.array_equal(got, want)
+        else:
+            assert np.allclose(got, want, rtol=1e-6, atol=1e-12)
+
+
+def ops_exact(lib):
+    return lib[1].COMBINE_EXACT
+
+
 # ---- cold-gradient accumulator ------------------------------------------------------------------
 @pytest.mark.parametrize("dim", [128, 5])
 def test_hash_accumulator(lib, dim):
