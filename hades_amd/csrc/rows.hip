@@ -17,7 +17,8 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kRowsPerBlock = 128;
+constexpr int kRowsPerBlock = 64;   // measured: 64 rows 34.7 us, 128 rows 37.1 us, 32 rows 35.6 us
+                                    // for 200 K rows of 512 bytes
 constexpr int kThreads = 256;
 constexpr int kUnroll = 8;
 
