@@ -23,12 +23,26 @@ How each function is pinned (tests/test_oracle.py):
                                         forms (all ids distinct, all ids equal), sum(cnt) == n
   adagrad                             : torch.optim.Adagrad on the gathered rows; g == 0 leaves w
                                         unchanged; first-step closed form
-  adam                                : torch.optim.Adam (same mathematics, different rounding) at
-                                        1e-6 relative; the reference has no test of its own
+  adam                                : PARTLY PINNED.  torch.optim.Adam (same mathematics) agrees to
+                                        2e-4 of one update on w and to rounding on m and v; the
+                                        reference forms 1 - beta^t in float32
+                                        (python/EmbCache/sparse_optim.py:652-655), a 6e-5 relative
+                                        error no library routine reproduces, and holds no test or
+                                        vector for it: below that level the weight update is
+                                        parity unpinned
   hash accumulator                    : a Python dict model; flush(accumulate(batches)) equals
                                         combine(concat(batches))
   hot placement                       : the reference's own argsort recipe, cache.py:165-171
-The C restatement of the native functions (hades_oracle.c) is checked against this module.
+  bucket_by_owner                     : torch.sort(stable=True) + bincount over the reference's
+                                        owner formula; brute-force bucket membership in input order
+  SACacheIndexModel                   : a sequence worked by hand from src/cache/cache_line.h, and
+                                        the reference's own cache_line class compiled into
+                                        oracle/_ref (ref_sacache_driver.cpp) on random sequences
+  ColdCacheServerModel                : per-id bookkeeping (pending sum, count, iteration counter,
+                                        threshold) without evictions; a worked case for the dense
+                                        local part
+The C restatement of the native functions (hades_oracle.c) is checked against this module; the
+committed vectors of tests/golden/ (made without this module) are checked in tests/test_golden.py.
 """
 import numpy as np
 import torch
