@@ -23,7 +23,10 @@ How each function is pinned (tests/test_oracle.py):
                                         forms (all ids distinct, all ids equal), sum(cnt) == n
   adagrad                             : torch.optim.Adagrad on the gathered rows; g == 0 leaves w
                                         unchanged; first-step closed form
-  adam                                : PARTLY PINNED.  torch.optim.Adam (same mathematics) agrees to
+  adam                                : PARTLY PINNED.  Closed forms: from zero state, and again with
+                                        the same gradient, every step is -lr * sign(g), m and v
+                                        follow (1 - beta^t) g and (1 - beta^t) g^2; g = 0 moves
+                                        nothing.  torch.optim.Adam (same mathematics) agrees to
                                         2e-4 of one update on w and to rounding on m and v; the
                                         reference forms 1 - beta^t in float32
                                         (python/EmbCache/sparse_optim.py:652-655), a 6e-5 relative

@@ -335,6 +335,25 @@ def test_adam_matches_torch_optim_adam():
     assert (step == 4).all()
 
 
+def test_adam_closed_forms():
+    # first step from zero state: m = (1-b1) g, v = (1-b2) g^2, both bias corrections cancel,
+    # so dw = -lr * g / (|g| + eps) = -lr * sign(g) up to rounding - a dropped correction, a
+    # dropped sqrt or a wrong sign all fail this
+    g = np.array([[3.0, -0.5, 1e-3, -2e-2]], np.float32)
+    w0 = np.array([[1.0, 2.0, -3.0, 0.5]], np.float32)
+    z1, z = np.zeros(1, np.float32), np.zeros_like(g)
+    w1, step, m1, v1 = O.adam_rows(w0, z1, z, z, g, 0.01, 0.9, 0.999, 1e-12)
+    assert np.allclose(w1 - w0, -0.01 * np.sign(g), rtol=1e-5) and step[0] == 1
+    assert np.allclose(m1, 0.1 * g, rtol=1e-6) and np.allclose(v1, 0.001 * g * g, rtol=1e-5)
+    # g = 0 from zero state: nothing moves but the step counter (0 / (0 + eps))
+    w2, step2, m2, v2 = O.adam_rows(w0, z1, z, z, z, 0.01, 0.9, 0.999, 1e-8)
+    assert np.array_equal(w2, w0) and step2[0] == 1 and not m2.any() and not v2.any()
+    # second step with the same gradient: m and v follow the geometric sums, dw is again -lr*sign(g)
+    w3, step3, m3, v3 = O.adam_rows(w1, step, m1, v1, g, 0.01, 0.9, 0.999, 1e-12)
+    assert np.allclose(m3, (1 - 0.9 ** 2) * g, rtol=1e-6) and np.allclose(v3, (1 - 0.999 ** 2) * g * g, rtol=1e-5)
+    assert np.allclose(w3 - w1, -0.01 * np.sign(g), rtol=2e-4) and step3[0] == 2
+
+
 # ---- accumulator ----------------------------------------------------------------------------
 def test_accumulator_flush_equals_combine_of_all_batches():
     rng = np.random.default_rng(12)
