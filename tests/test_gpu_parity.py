@@ -288,6 +288,41 @@ def test_index_cache_large_vs_reference_cache_line(lib, sacache_ref, cache_size,
         _same_cache_state(ic, r)
 
 
+def test_index_cache_reference_recipes_at_their_sizes(lib, sacache_ref):
+    """The reference's own scripts at their sizes, with assertions where they print:
+    test/test_lookup.py (a 4 M-entry cache, ten adds of 2 M random ids, then ten 400 K-id lookups whose
+    host and device results must agree, :8-35) and test/test_single_cache.py (ten rounds of add 200 K /
+    lookup 200 K / reset 20 K, then get_valid_entries_num and getall, :13-40)."""
+    import hades_amd.EmbCacheLib as E
+    g = torch.Generator().manual_seed(42)
+    size = 4_000_000
+    ic, r = E.IndexCache(size, "test_cache", True), sacache_ref(size)
+    assert ic.get_valid_entries_num() == 0
+    for i in range(10):                                                   # test_lookup.py:12-14
+        index = torch.randint(0, size, (2_000_000,), generator=g)
+        assert np.array_equal(ic.add(index.cuda()).cpu().numpy(), r.add(index.numpy()))
+    for i in range(10):                                                   # test_lookup.py:17-35
+        index = torch.randint(0, size, (400_000,), generator=g)
+        out1 = ic.lookup(index.cuda())
+        out2 = ic.cudalookup(index.cuda())
+        assert torch.equal(out1, out2)                                    # :34
+        assert np.array_equal(out1.cpu().numpy(), r.lookup(index.numpy()))
+    ic, r = E.IndexCache(size, "test_cache", True), sacache_ref(size)
+    for i in range(10):                                                   # test_single_cache.py:13-34
+        index = torch.randint(0, size, (200_000,), generator=g)
+        assert np.array_equal(ic.add(index.cuda()).cpu().numpy(), r.add(index.numpy()))
+        index = torch.randint(0, size, (200_000,), generator=g)
+        assert np.array_equal(ic.lookup(index.cuda()).cpu().numpy(), r.lookup(index.numpy()))
+        index = torch.unique(torch.randint(0, size, (20_000,), generator=g))
+        ic.reset(index.cuda()); r.reset(index.numpy())
+    assert ic.get_valid_entries_num() == r.get_valid_entries_num() > 0    # :36
+    a, b = ic.getall(size)                                                # :37-39
+    want_a, want_b = r.getall(size)
+    k = want_a.size
+    assert np.array_equal(a[:k].cpu().numpy(), want_a) and np.array_equal(b[:k].cpu().numpy(), want_b)
+    assert int((b[k:] != -1).sum()) == 0 and int(a[k:].abs().sum()) == 0
+
+
 # ---- cold-data cache: the server's gradient path with its staleness rule -------------------
 def _cold_state_equal(c, m):
     assert np.array_equal(c.emb_cache_buff.cpu().numpy(), m.emb.numpy())
