@@ -7,10 +7,12 @@
 //   1. stable LSD radix sort of (key = id, value = occurrence position), 8 bits per pass, only
 //      over the key bits that id_bound leaves significant.  Stability keeps the positions of
 //      equal ids ascending, which is what makes a sequential in-segment sum reproduce CPU
-//      index_add_.  Per pass two kernels: per-tile digit counts [tile][digit], then a scatter in
-//      which every block derives its own global digit offsets from those counts (column sums over
-//      all tiles and over the tiles before it - no separate scan kernel), ranks its keys stably
-//      through LDS and writes them out.
+//      index_add_.  Per pass two kernels: digit counts per tile of 1024 keys and per group of four
+//      tiles, then a scatter in which every block derives its own global digit offsets from those
+//      counts (column sums over the group rows and the tile rows before it), ranks its keys
+//      stably through LDS and writes them out.  From 64 groups on (batches above 256 K ids) a
+//      third, tiny kernel turns the group counts into prefixes first, so that a scatter block
+//      reads five count rows whatever the batch size.
 //   2. run boundaries -> uids, seg_start, seg_of (index of the run every sorted position is in).
 //   3. segmented sum of the gradient rows:
 //        EXACT: one lane group per distinct id walks its rows left to right; a run of 64 rows or
@@ -36,6 +38,8 @@ constexpr int kRadixBits = 8;
 constexpr int kBins = 1 << kRadixBits;
 constexpr int kMaxPasses = 8;
 constexpr int kGroup = 4;  // tiles counted by one block of the count kernel
+constexpr int kIpt = 4;    // keys per thread in a radix tile: tiles of 1024 keys
+constexpr int kScanFrom = 64;  // groups of tiles from which the group counts get their own scan
 
 // ---- key transforms ---------------------------------------------------------
 template <typename KeyT>
@@ -117,6 +121,31 @@ __global__ __launch_bounds__(kGroup * kThreads) void radix_count_kernel(
   }
 }
 
+// ---- prefix of the group counts (large batches only) -------------------------------------------
+// gcnt[g][d] becomes the number of keys with digit d in the groups before g, and row `ngroups`
+// receives the column totals, so that a scatter block reads two rows of gcnt instead of one per
+// group.  One wave per digit column: lanes take 64 consecutive groups, scan them in registers and
+// carry the running total to the next 64.
+__global__ __launch_bounds__(kThreads) void radix_group_scan_kernel(uint32_t* __restrict__ gcnt,
+                                                                   int64_t ngroups) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int d = blockIdx.x * kWaves + threadIdx.x / kWave;   // grid = kBins / kWaves blocks
+  uint32_t carry = 0;
+  for (int64_t g0 = 0; g0 < ngroups; g0 += kWave) {
+    const int64_t g = g0 + lane;
+    const uint32_t v = g < ngroups ? gcnt[g * kBins + d] : 0u;
+    uint32_t incl = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const uint32_t t = __shfl_up(incl, off);
+      if (lane >= off) incl += t;
+    }
+    if (g < ngroups) gcnt[g * kBins + d] = carry + incl - v;
+    carry += __shfl(incl, kWave - 1);
+  }
+  if (lane == 0) gcnt[ngroups * kBins + d] = carry;
+}
+
 // ---- one radix pass ---------------------------------------------------------------------
 // Tile order: wave w of the block owns tile positions [w*IPT*64, (w+1)*IPT*64), round r of that
 // wave the 64 positions from r*64 on.  Ranks are handed out in exactly that order.
@@ -124,7 +153,7 @@ template <typename KeyT, bool FIRST, int IPT>
 __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
     const void* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, int64_t n, int shift,
     uint32_t mask, int bits, const uint32_t* __restrict__ cnt_cur,
-    const uint32_t* __restrict__ gcnt, int64_t ngroups, KeyT* __restrict__ keys_out,
+    const uint32_t* __restrict__ gcnt, int64_t ngroups, int scanned, KeyT* __restrict__ keys_out,
     uint32_t* __restrict__ vals_out) {
   __shared__ uint32_t s_cnt[kWaves][kBins];
   __shared__ uint32_t s_glob[kBins];
@@ -147,31 +176,37 @@ __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
 
   // global offset of (digit, this tile): all keys with a smaller digit, plus the keys with this
   // digit in the tiles before this one.  Thread d owns digit d (kThreads == kBins).
-  // Rows to add up: one per group of tiles (all of them for the totals, those before this tile's
-  // group for the prefix), then the tile rows of this group before this tile.  The sums are
-  // latency-bound: wave w takes the rows v = w (mod kWaves), lane l the four digits 4l..4l+3 of a
-  // row as one 16-byte load, sixteen rows in flight.
+  // Rows to add up, unscanned counts: one per group of tiles (all of them for the totals, those
+  // before this tile's group for the prefix), then the tile rows of this group before this tile.
+  // Scanned counts (large batches, radix_group_scan_kernel has run): the totals row, the prefix
+  // row of this tile's group, then the same tile rows - at most five rows whatever the batch.
+  // The sums are latency-bound: wave w takes the rows v = w (mod kWaves), lane l the four digits
+  // 4l..4l+3 of a row as one 16-byte load, sixteen rows in flight.
   {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     constexpr int kInFlight = 16;
     const int64_t me = blockIdx.x;
     const int64_t my_group = me / kGroup;
-    const int64_t nrows = ngroups + (me - my_group * kGroup);
+    const int64_t nhead = scanned ? 2 : ngroups;   // rows that come from gcnt
+    const int64_t nrows = nhead + (me - my_group * kGroup);
     u32x4 tot4 = {0, 0, 0, 0}, pre4 = {0, 0, 0, 0};
     for (int64_t v0 = wave; v0 < nrows; v0 += kWaves * kInFlight) {
       u32x4 h[kInFlight];
 #pragma unroll
       for (int k = 0; k < kInFlight; ++k) {
         const int64_t v = v0 + static_cast<int64_t>(k) * kWaves;
-        const uint32_t* row = v < ngroups ? gcnt + v * kBins
-                                          : cnt_cur + (my_group * kGroup + (v - ngroups)) * kBins;
+        const int64_t head_row = scanned ? (v == 0 ? ngroups : my_group) : v;
+        const uint32_t* row = v < nhead ? gcnt + head_row * kBins
+                                        : cnt_cur + (my_group * kGroup + (v - nhead)) * kBins;
         h[k] = v < nrows ? reinterpret_cast<const u32x4*>(row)[lane] : u32x4{0, 0, 0, 0};
       }
 #pragma unroll
       for (int k = 0; k < kInFlight; ++k) {
         const int64_t v = v0 + static_cast<int64_t>(k) * kWaves;
-        if (v < ngroups) tot4 += h[k];
-        if (v < my_group || v >= ngroups) pre4 += h[k];
+        const bool to_tot = scanned ? v == 0 : v < ngroups;
+        const bool to_pre = scanned ? v >= 1 : (v < my_group || v >= ngroups);
+        if (to_tot) tot4 += h[k];
+        if (to_pre) pre4 += h[k];
       }
     }
     // s_cnt doubles as scratch here: rows 0..3 hold the per-wave totals; the per-wave prefixes
@@ -708,7 +743,7 @@ struct Plan {
   bool key64;
   int key_bits;
   int passes;
-  int ipt;        // keys per thread in a radix tile: 4, 8 or 16
+  bool scan;      // group counts are prefix-scanned by a kernel of their own
   int vec;        // 4 or 1
   int group;
   int col_tiles;
@@ -729,10 +764,10 @@ Plan make_plan(int64_t n, int64_t dim, int64_t id_bound, bool grad_aligned) {
   }
   if (p.key_bits < 1) p.key_bits = 1;
   p.passes = (p.key_bits + kRadixBits - 1) / kRadixBits;
-  // every pass reads all per-tile counts in every block: keep the number of tiles moderate
-  p.ipt = 4;
-  while (p.ipt < 16 && ceil_div(nn, kThreads * p.ipt) > 512) p.ipt *= 2;
-  p.ntiles = ceil_div(nn, kThreads * p.ipt);
+  p.ntiles = ceil_div(nn, kThreads * kIpt);
+  // past kScanFrom groups of tiles the group counts are turned into prefixes by a kernel of their
+  // own (3-4 us), and a scatter block reads five count rows instead of one per group
+  p.scan = ceil_div(p.ntiles, kGroup) > kScanFrom;
   p.vec = (dim % 4 == 0 && grad_aligned) ? 4 : 1;
   const int64_t lanes = (dim + p.vec - 1) / p.vec;
   int g = kMinGroup;
@@ -762,7 +797,7 @@ void carve_sort(Carver& c, int64_t n, SortWs* w) {
   for (int i = 0; i < 2; ++i) w->vals[i] = c.take<uint32_t>(nn);
   w->cnt_len = make_plan(nn, 1, 0, true).ntiles * kBins;  // the tile count depends on n only
   w->cnt = c.take<uint32_t>(w->cnt_len);
-  w->gcnt = c.take<uint32_t>(ceil_div(w->cnt_len / kBins, kGroup) * kBins);
+  w->gcnt = c.take<uint32_t>((ceil_div(w->cnt_len / kBins, kGroup) + 1) * kBins);  // + totals row
   w->bytes = c.total();
 }
 
@@ -789,12 +824,15 @@ Ws carve(void* ws, int64_t n, int64_t dim) {
   return w;
 }
 
-template <typename KeyT, int IPT>
-int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
+template <typename KeyT>
+int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
                  hipStream_t st, const void** keys_out, const uint32_t** perm_out) {
   const int64_t ngroups = ceil_div(p.ntiles, kGroup);
+  HADES_REQUIRE(p.ntiles * kBins <= w.cnt_len, "internal: radix count buffer too small");
+  constexpr int IPT = kIpt;
   const dim3 grid(static_cast<unsigned>(p.ntiles)), cgrid(static_cast<unsigned>(ngroups)),
-      block(kThreads), cblock(kGroup * kThreads);
+      block(kThreads), cblock(kGroup * kThreads), sgrid(kBins / kWaves);
+  const int scanned = p.scan ? 1 : 0;
   const int base = p.key_bits / p.passes, extra = p.key_bits % p.passes;
   int bits_of[kMaxPasses], shift_of[kMaxPasses + 1];
   shift_of[0] = 0;
@@ -812,15 +850,17 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
     if (pass == 0) {
       HADES_LAUNCH((radix_count_kernel<KeyT, true, IPT>), cgrid, cblock, 0, st, kin, n,
                    shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.status);
+      if (scanned) HADES_LAUNCH(radix_group_scan_kernel, sgrid, block, 0, st, w.gcnt, ngroups);
       HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, true, IPT>), grid,
                          block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
-                         w.gcnt, ngroups, kout, vout);
+                         w.gcnt, ngroups, scanned, kout, vout);
     } else {
       HADES_LAUNCH((radix_count_kernel<KeyT, false, IPT>), cgrid, cblock, 0, st, kin, n,
                    shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.status);
+      if (scanned) HADES_LAUNCH(radix_group_scan_kernel, sgrid, block, 0, st, w.gcnt, ngroups);
       HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, false, IPT>), grid,
                          block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
-                         w.gcnt, ngroups, kout, vout);
+                         w.gcnt, ngroups, scanned, kout, vout);
     }
     kin = kout;
     vin = vout;
@@ -829,18 +869,6 @@ int run_sort_ipt(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
   *keys_out = kin;
   *perm_out = vin;
   return HADES_OK;
-}
-
-template <typename KeyT>
-int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
-             hipStream_t st, const void** keys_out, const uint32_t** perm_out) {
-  HADES_REQUIRE(p.ntiles * kBins <= w.cnt_len,
-                "internal: radix count buffer too small");
-  switch (p.ipt) {
-    case 4: return run_sort_ipt<KeyT, 4>(idx, n, id_bound, p, w, st, keys_out, perm_out);
-    case 8: return run_sort_ipt<KeyT, 8>(idx, n, id_bound, p, w, st, keys_out, perm_out);
-    default: return run_sort_ipt<KeyT, 16>(idx, n, id_bound, p, w, st, keys_out, perm_out);
-  }
 }
 
 template <typename KeyT>
