@@ -43,6 +43,34 @@ def test_dropin_rejects_host_tensors_without_gpu():
         E.cudaSplit(i, torch.zeros(4, dtype=torch.int8))
 
 
+def test_dropin_exposes_index_cache_and_later_operators_without_gpu():
+    # resolved lazily (src/pybind.cc:17-45); host tensors are refused before any launch
+    import hades_amd.EmbCacheLib as E
+    from hades_amd import ops
+    from hades_amd.index_cache import IndexCache, LocalCache
+    assert E.IndexCache is IndexCache
+    for name in ("get_size", "get_valid_entries_num", "get_capacity", "get_space", "add", "lookup",
+                 "reset", "getall", "cudalookup"):
+        assert callable(getattr(IndexCache, name)), name
+    for name in ("lookup", "cudalookup", "add", "get_num_entries", "reset"):   # cache.py:18-31
+        assert callable(getattr(LocalCache, name)), name
+    i = torch.zeros(4, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="device tensor"):
+        ops.bucket_by_owner(i, None, None, None, 4, 4)
+    with pytest.raises(RuntimeError, match="int64"):
+        ops.bucket_by_owner(i.to(torch.int32), None, None, None, 4, 4)
+    with pytest.raises(AttributeError):
+        E.no_such_function
+
+
+def test_staleness_threshold_is_the_reference_formula():
+    # python/EmbCache/server.py:87-88
+    from hades_amd.cold_cache import staleness_threshold
+    h = torch.tensor([0.0, 0.0005, 0.009, 0.099, 0.5, 1.0, 10.0])
+    assert staleness_threshold(h).tolist() == [100, 100, 100, 10, 2, 1, 1]
+    assert staleness_threshold(h).dtype == torch.int32
+
+
 def test_select_hot_ids_matches_oracle_and_reference_recipe():
     g = torch.Generator().manual_seed(0)
     hotness = torch.rand(5000, generator=g)
