@@ -521,6 +521,12 @@ CASES = [  # (n, dim, id space, kind)
     (5000, 100, 300, "zipf"), (20_000, 128, 2_400_000, "zipf"), (70_001, 260, 5000, "zipf"),
     (65_536, 64, 1_000_000, "zipf"),
     (3000, 7, 3, "zipf"), (2500, 1, 2, "zipf"), (40_000, 128, 40, "zipf"),   # very long runs
+    # sizes either side of the sort's tile (1024), group of tiles (4096), the segmented sum's block
+    # span (256) and the point where the group counts get their own scan (64 groups = 262 144 ids)
+    (255, 8, 90, "zipf"), (256, 8, 90, "zipf"), (257, 8, 90, "zipf"),
+    (1023, 4, 700, "zipf"), (1024, 4, 700, "zipf"), (1025, 4, 700, "zipf"),
+    (4095, 4, 100_000, "zipf"), (4097, 4, 100_000, "zipf"),
+    (262_144, 4, 3_000_000, "zipf"), (262_145, 4, 3_000_000, "zipf"), (530_000, 8, 50_000_000, "zipf"),
 ]
 
 
