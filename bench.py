@@ -48,6 +48,10 @@ def parse_args():
                          "fetch; graph: every step is the replay of a HIP graph captured once per "
                          "batch (no kernel inside a replay can be bracketed with events, so the "
                          "roofline time is taken from eager steps before the timed region)")
+    ap.add_argument("--flush-rule", default="every8", choices=["every8", "staleness"],
+                    help="cfg4 only: write the accumulated cold gradients back every 8 steps (hash "
+                         "accumulator), or per row by the cache server's staleness rule (cold-data "
+                         "cache)")
     ap.add_argument("--batches", type=int, default=4, help="distinct pre-generated id batches")
     ap.add_argument("--event-every", type=int, default=4,
                     help="bracket every n-th launch of the dominant kernel with HIP events inside "
@@ -432,6 +436,114 @@ def run_cfg4(args):
     print(json.dumps(line))
 
 
+def run_cfg4_staleness(args):
+    """cfg4 with the reference's own rule instead of "every 8 steps": the cold-data cache of the
+    cache server (set-associative index over 4 M slots, per-row staleness thresholds from the
+    hotness, count threshold 16) in front of the pinned-host table.  Per step: combine the batch;
+    gradients of cached ids accumulate in their slots; the other ids are applied to the host
+    table at once and their rows enter the cache; rows that are due leave the cache and are
+    applied.  One host synchronisation per step (the number of uncached ids sizes the row fetch).
+    Prints its own JSON line."""
+    import torch
+    import hades_amd.EmbCacheLib as E
+    from hades_amd import ops, synth
+    from hades_amd.cold_cache import ColdDataCache
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = synth.CONFIGS["cfg4"]
+    N, D, H, n, slots = cfg["num_rows"], cfg["dim"], cfg["num_hot"], cfg["batch"], cfg["num_slots"]
+    seed = 1234 + 4
+    warm = max(args.warmup, 8)
+    # a fresh batch of ids for every step of the warm-up and of both measured passes: a cache sees
+    # the stream's long tail only if the ids do not come round again; the gradient rows (268 MB a
+    # batch) are reused
+    nb, ng = warm + 2 * args.steps, 4
+    log("allocating the %d x %d pinned host table (%.1f GB)" % (N, D, N * D * 4 / 1e9))
+    cold_w = torch.empty((N, D), dtype=torch.float32, pin_memory=True)
+    log("filling it")
+    synth.fill_normal_(cold_w, 0.01, seed, progress=log)
+    cold_s = torch.zeros((N, D), dtype=torch.float32, device=dev)
+    log("sampling %d batches of %d cold ids" % (nb, n))
+    sampler = synth.ZipfSampler(N - H, cfg["zipf_s"], dev)
+    ids = [synth.make_ids(sampler, N, n, seed * 1000 + b, rank_offset=H) for b in range(nb)]
+    grads = [synth.make_grads(n, D, seed * 2000 + b, dev) for b in range(ng)]
+    # hotness of an id = its expected number of occurrences per step: popular cold rows may wait
+    # one iteration, the long tail up to 100 (threshold = ceil(1 / (0.001 + hotness)), capped)
+    ranks = torch.arange(1, N - H + 1, dtype=torch.float64, device=dev)
+    p = ranks.pow_(-cfg["zipf_s"])
+    p.div_(p.sum())
+    hotness = torch.zeros(N, dtype=torch.float32, device=dev)
+    hotness[synth.rank_to_id(torch.arange(H + 1, N + 1, dtype=torch.int64, device=dev), N)] = \
+        (p * n).float()
+    del ranks, p, sampler
+    cache = ColdDataCache(slots, D, hotness, cnt_threshold=16, device=dev)
+    del hotness
+    ws = ops.Workspace(dev)
+    comb_out = (torch.empty(n, dtype=torch.int64, device=dev),
+                torch.empty((n, D), dtype=torch.float32, device=dev),
+                torch.empty(n, dtype=torch.int64, device=dev),
+                torch.empty(1, dtype=torch.int64, device=dev))
+    fetched = torch.empty((n, D), dtype=torch.float32, device=dev)
+    log("workload ready")
+    stats = {"miss": 0, "hit": 0, "flushed": 0}
+
+    def step(i, count=False):
+        q, g = ids[i], grads[i % ng]
+        uids, sums, cnts, nu = ops.combine_padded(q, g, id_bound=N, workspace=ws, out=comb_out)
+        u = int(nu.item())
+        uids, sums = uids[:u], sums[:u]
+        locs = cache.accumulate_gradients_cold_remote(uids, sums)          # cached ids: delayed
+        _, hit_pos, miss_pos = ops.split(locs)
+        if miss_pos.numel():
+            m_ids = uids[miss_pos]
+            m_sums = sums[miss_pos]
+            ops.adagrad_update_(m_ids, m_sums, None, None, cold_w, cold_s, None, 0.01, 1e-10)
+            rows = fetched[:m_ids.numel()]
+            E.cudaFetch2(cold_w, m_ids, rows)                              # the rows a trainer pulled
+            cache.update_cache(m_ids, rows)
+        f_ids, f_grads, f_cnts, f_num = cache.staled_gradients_remote_padded(slots)
+        ops.adagrad_update_(f_ids, f_grads, None, None, cold_w, cold_s, None, 0.01, 1e-10,
+                            num_unique=f_num)
+        if count:
+            stats["miss"] += int(miss_pos.numel()); stats["hit"] += int(hit_pos.numel())
+            stats["flushed"] += int(f_num.item())
+
+    for i in range(warm):
+        step(i)
+    torch.cuda.synchronize()
+    log("warm-up done, %d entries cached" % cache.index.get_valid_entries_num())
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(warm + i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    for i in range(args.steps):                     # as many steps again, counted (more host syncs)
+        step(warm + args.steps + i, count=True)
+    K = args.steps
+    miss, hit, flushed = (stats[k] / K for k in ("miss", "hit", "flushed"))
+    # rows over the host link: uncached ids are read, written and fetched once more for the cache;
+    # flushed rows are read and written
+    host_rows = miss * 3 + flushed * 2
+    line = {
+        "metric": "cold gradient rows/s (combine + cold-data cache with the staleness rule + write-back)",
+        "value": round(n / (ms_per_step * 1e-3), 1), "unit": "rows/s", "n_gpus": 1, "steps": K,
+        "warmup": warm, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cfg4 with the cache server's rule: %d cold ids/step zipf s=%.2f, "
+                               "%d-slot set-associative cold-data cache in HBM, per-row staleness "
+                               "threshold from the hotness, count threshold 16, %d x %d pinned-host "
+                               "table" % (n, cfg["zipf_s"], slots, N, D)},
+        "distinct_per_step": round((miss + hit), 1), "cached_hits_per_step": round(hit, 1),
+        "uncached_per_step": round(miss, 1), "flushed_rows_per_step": round(flushed, 1),
+        "cache_entries": cache.index.get_valid_entries_num(),
+        "host_link_rows_per_step": round(host_rows, 1),
+        "host_link_GB/s_both_ways": round(host_rows * 4 * D / (ms_per_step * 1e-3) / 1e9, 2),
+    }
+    print(json.dumps(line))
+
+
 def run_neighbours(args):
     """The operators either side of the step, each timed on its own over `steps` calls after
     `warmup` (wall clock around a synchronised loop, so launch overheads count): the pre-exchange
@@ -582,7 +694,10 @@ def main():
               "gradient exchange is out of scope); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     if args.workload == "cfg4":
-        run_cfg4(args)
+        if args.flush_rule == "staleness":
+            run_cfg4_staleness(args)
+        else:
+            run_cfg4(args)
         return
     if args.workload == "neighbours":
         run_neighbours(args)
