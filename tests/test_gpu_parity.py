@@ -288,6 +288,35 @@ def test_index_cache_large_vs_reference_cache_line(lib, sacache_ref, cache_size,
         _same_cache_state(ic, r)
 
 
+def test_index_cache_generated_programs_vs_model(lib):
+    """Generated operation sequences (hypothesis) on tiny caches, where lines fill up, evict and
+    are reset all the time: locs, line contents and ages after every operation."""
+    from hypothesis import HealthCheck, given, settings, strategies as st
+    import hades_amd.EmbCacheLib as E
+    program = st.lists(st.tuples(st.sampled_from(["add", "lookup", "reset", "cudalookup"]),
+                                 st.lists(st.integers(-2, 70), min_size=0, max_size=25)),
+                       min_size=1, max_size=20)
+
+    @settings(max_examples=40, deadline=None, suppress_health_check=list(HealthCheck))
+    @given(st.integers(1, 40), program)
+    def run(cache_size, prog):
+        ic, m = E.IndexCache(cache_size, "unused", True), O.SACacheIndexModel(cache_size)
+        for op, ids in prog:
+            ids = np.array(ids, dtype=np.int64)
+            ok = ids[ids >= 0]                      # the model, like the reference, takes ids >= 0
+            if op == "reset":
+                ic.reset(dev(ids)); m.reset(ok)
+            else:
+                got = getattr(ic, op)(dev(ids)).cpu().numpy()
+                want = np.full(ids.shape, -1, np.int64)
+                want[ids >= 0] = getattr(m, op)(ok)
+                assert np.array_equal(got, want), (op, ids.tolist())
+            assert np.array_equal(ic.line_ids.cpu().numpy().reshape(-1, 8), m.ids)
+            assert np.array_equal(ic.line_age.cpu().numpy().reshape(-1, 8), m.age)
+
+    run()
+
+
 def test_index_cache_reference_recipes_at_their_sizes(lib, sacache_ref):
     """The reference's own scripts at their sizes, with assertions where they print:
     test/test_lookup.py (a 4 M-entry cache, ten adds of 2 M random ids, then ten 400 K-id lookups whose
@@ -574,6 +603,35 @@ def test_combine(lib, n, dim, space, kind, bounded):
         # runs that fit inside one chunk are summed left to right: bit-equal to the exact mode
         short = wc <= 1
         assert np.array_equal(got[short], ws[short])
+
+
+def test_combine_generated_batches(lib):
+    """Generated small batches (hypothesis): any ids - negative, wide, heavily repeated -, any
+    row width, with and without an id bound."""
+    from hypothesis import HealthCheck, given, settings, strategies as st
+    _, ops = lib
+    wide = st.one_of(st.integers(0, 12), st.integers(0, 12), st.integers(-(2 ** 62), 2 ** 62))
+
+    @settings(max_examples=50, deadline=None, suppress_health_check=list(HealthCheck))
+    @given(st.lists(wide, min_size=0, max_size=300), st.integers(1, 9), st.booleans())
+    def run(ids, dim, bounded):
+        idx = np.array(ids, dtype=np.int64)
+        if bounded:
+            idx = np.abs(idx) % 1000
+        rng = np.random.default_rng(idx.size * 31 + dim)
+        grad = rng.standard_normal((idx.size, dim)).astype(np.float32)
+        wu, ws, wc = O.combine_sequential(idx, grad)
+        _, w64, _ = O.combine_float64(idx, grad)
+        bound = 1000 if bounded else 0
+        uids, sums, cnts = ops.combine(dev(idx), dev(grad), bound, ops.COMBINE_EXACT)
+        assert np.array_equal(uids.cpu().numpy(), wu) and np.array_equal(cnts.cpu().numpy(), wc)
+        assert np.array_equal(sums.cpu().numpy(), ws)
+        uids, sums, cnts = ops.combine(dev(idx), dev(grad), bound, ops.COMBINE_FAST)
+        assert np.array_equal(uids.cpu().numpy(), wu) and np.array_equal(cnts.cpu().numpy(), wc)
+        if idx.size:
+            assert combine_tol_ok(sums.cpu().numpy(), w64, max(np.abs(w64).max(), 1e-30))
+
+    run()
 
 
 def test_unique_grads_dropin(lib):
