@@ -605,6 +605,41 @@ def test_combine(lib, n, dim, space, kind, bounded):
         assert np.array_equal(got[short], ws[short])
 
 
+def test_rows_and_update_generated_shapes(lib):
+    """Generated shapes (hypothesis) for the row kernels: any row width (vector and scalar paths,
+    rows that are not a multiple of 16 bytes), any batch size, any hot fraction; fetch, set and
+    the Adagrad update against the oracle, bit for bit."""
+    from hypothesis import HealthCheck, given, settings, strategies as st
+    _, ops = lib
+
+    @settings(max_examples=40, deadline=None, suppress_health_check=list(HealthCheck))
+    @given(st.integers(1, 300), st.integers(0, 400), st.integers(0, 60), st.integers(0, 10 ** 6))
+    def run(dim, n, n_hot, seed):
+        rng = np.random.default_rng(seed)
+        n_rows = 500
+        cold = rng.standard_normal((n_rows, dim)).astype(np.float32)
+        hot_ids = np.sort(rng.choice(n_rows, n_hot, replace=False)).astype(np.int64)
+        hot = rng.standard_normal((n_hot, dim)).astype(np.float32)
+        q = rng.integers(0, n_rows, n).astype(np.int64)
+        t_cold, t_hot, t_ids = dev(cold), dev(hot), dev(hot_ids)
+        got = ops.cached_fetch(t_cold, t_hot, dev(q), t_ids)
+        assert np.array_equal(got.cpu().numpy(), O.cached_fetch(cold, hot, q, hot_ids))
+        u = np.unique(q)
+        rows = rng.standard_normal((u.size, dim)).astype(np.float32)
+        ops.cached_set(dev(rows), t_cold, t_hot, dev(u), t_ids)
+        O.cached_set(rows, cold, hot, u, hot_ids)
+        assert np.array_equal(t_cold.cpu().numpy(), cold) and np.array_equal(t_hot.cpu().numpy(), hot)
+        cs, hs = np.abs(cold) * 0.1, np.abs(hot) * 0.1
+        t_cs, t_hs = dev(cs), dev(hs)
+        g = (rng.standard_normal((u.size, dim)) * 1e-2).astype(np.float32)
+        ops.adagrad_update_(dev(u), dev(g), t_hot, t_hs, t_cold, t_cs, t_ids, 0.01, 1e-10)
+        O.sparse_adagrad_step(cold, cs, hot, hs, hot_ids, u, g, 0.01, 1e-10)
+        for a, b in ((t_cold, cold), (t_cs, cs), (t_hot, hot), (t_hs, hs)):
+            assert np.array_equal(a.cpu().numpy(), b)
+
+    run()
+
+
 def test_combine_generated_batches(lib):
     """Generated small batches (hypothesis): any ids - negative, wide, heavily repeated -, any
     row width, with and without an id bound."""
