@@ -31,11 +31,19 @@ __global__ __launch_bounds__(kThreads) void owner_of_kernel(const int64_t* __res
 
 // sizes[g] = number of sorted owners equal to g (difference of two upper bounds, which is what
 // the reference takes from cudaBinarySearch2 over arange(num_owners))
+// An owner outside [0, num_owners) leaves the owners unsorted: every size is then reported as -1.
 __global__ __launch_bounds__(kThreads) void bucket_sizes_kernel(const uint32_t* __restrict__ sorted,
                                                                int64_t n, int64_t num_owners,
-                                                               int64_t* __restrict__ sizes) {
+                                                               int64_t* __restrict__ sizes,
+                                                               const int32_t* __restrict__ bad,
+                                                               int64_t nbad) {
+  const int violated = any_flag_set(bad, nbad);
   const int64_t g = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (g >= num_owners) return;
+  if (violated) {
+    sizes[g] = -1;
+    return;
+  }
   const int64_t hi = upper_bound_dev<uint32_t>(sorted, n, static_cast<uint32_t>(g));
   const int64_t lo = g > 0 ? upper_bound_dev<uint32_t>(sorted, n, static_cast<uint32_t>(g - 1)) : 0;
   sizes[g] = hi - lo;
@@ -106,15 +114,15 @@ int hades_bucket_by_owner(const int64_t* ids, int64_t n, const int64_t* range_pa
 
   HADES_LAUNCH(owner_of_kernel, grid, block, 0, st, ids, n, range_partition, num_part,
                local_num_gpus, owner);
-  // owners outside [0, num_owners) (negative ids, ids beyond the last range) set bit 0 of the
-  // first workspace word, as ids beyond id_bound do in the combine
+  // owners outside [0, num_owners) (negative ids, ids beyond the last range) are flagged by the
+  // sort's first pass, as ids beyond id_bound are in the combine; the sizes kernel reports them
   SortResult sr;
   const int rc = sort_ids(owner, n, num_owners, workspace, sort_bytes, st, &sr);
   if (rc != HADES_OK) return rc;
   HADES_REQUIRE(!sr.key64, "internal: owner keys must be 32-bit");
   HADES_LAUNCH(bucket_sizes_kernel, dim3(static_cast<unsigned>(ceil_div(num_owners, kThreads))),
                block, 0, st, static_cast<const uint32_t*>(sr.sorted_keys), n, num_owners,
-               split_sizes);
+               split_sizes, sr.bad, sr.nbad);
   HADES_LAUNCH(bucket_gather_kernel, grid, block, 0, st, sr.perm, n, ids, cnt, ids_out, cnt_out,
                perm_out);
   if (grad != nullptr)  // rows: dst[j, :] = src[perm[j], :] (positions are below 2^30: int32 index)

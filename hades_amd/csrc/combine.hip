@@ -89,7 +89,7 @@ template <typename KeyT, bool FIRST, int IPT>
 __global__ __launch_bounds__(kGroup * kThreads) void radix_count_kernel(
     const void* __restrict__ keys_in, int64_t n, int shift, uint32_t mask,
     uint32_t* __restrict__ cnt, uint32_t* __restrict__ gcnt, int64_t ntiles, int64_t id_bound,
-    int32_t* __restrict__ status) {
+    int32_t* __restrict__ bad_blk) {
   __shared__ uint32_t s_hist[kGroup][kBins];
   const int g = threadIdx.x / kThreads;  // the tile of the group this thread counts
   const int t = threadIdx.x % kThreads;  // kThreads == kBins: also the digit it writes out
@@ -110,8 +110,10 @@ __global__ __launch_bounds__(kGroup * kThreads) void radix_count_kernel(
       atomicAdd(&s_hist[g][static_cast<uint32_t>(k >> shift) & mask], 1u);
     }
   }
-  if (FIRST && bad) atomicOr(status, 1);
-  __syncthreads();
+  // the first pass also checks the promise 0 <= id < id_bound: one flag per block, written by
+  // every block on every call, so the flags need no clearing and are never stale
+  const int any_bad = __syncthreads_or(FIRST && bad ? 1 : 0);
+  if (FIRST && threadIdx.x == 0) bad_blk[blockIdx.x] = any_bad;
   if (tile < ntiles) cnt[tile * kBins + t] = s_hist[g][t];
   if (g == 0) {
     uint32_t sum = 0;
@@ -303,8 +305,16 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
     const KeyT* __restrict__ keys, const uint32_t* __restrict__ perm, int64_t n,
     const uint32_t* __restrict__ blk_cnt, int64_t* __restrict__ uids,
     uint32_t* __restrict__ seg_start, uint32_t* __restrict__ seg_of,
-    int64_t* __restrict__ num_unique, int32_t* __restrict__ inverse) {
+    int64_t* __restrict__ num_unique, int32_t* __restrict__ inverse,
+    const int32_t* __restrict__ bad_blk, int64_t nbad) {
   __shared__ uint32_t smem[kWaves + 1];
+  // the block that writes num_unique first learns whether the first count pass saw an id outside
+  // [0, id_bound): it then reports -1 distinct ids, which every consumer treats as "no live rows"
+  int violated = 0;
+  if (blockIdx.x == gridDim.x - 1) {
+    for (int64_t b = threadIdx.x; b < nbad; b += kThreads) violated |= bad_blk[b];
+    violated = __syncthreads_or(violated);
+  }
   // runs that begin in the tiles before this one
   uint32_t before = 0;
   for (int64_t b = threadIdx.x; b < static_cast<int64_t>(blockIdx.x); b += kThreads)
@@ -348,7 +358,7 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
         }
         if (j == n - 1) {
           seg_start[u] = static_cast<uint32_t>(n);
-          num_unique[0] = static_cast<int64_t>(u);
+          num_unique[0] = violated ? int64_t(-1) : static_cast<int64_t>(u);
         }
       }
     }
@@ -781,7 +791,9 @@ Plan make_plan(int64_t n, int64_t dim, int64_t id_bound, bool grad_aligned) {
 
 // workspace of the sort alone
 struct SortWs {
-  int32_t* status;
+  int32_t* bad;         // [ceil(ntiles / kGroup)]: 1 where a block of the first count pass saw an id
+                        // outside [0, id_bound); rewritten in full by every sort
+  int64_t nbad;
   void* keys[2];
   uint32_t* vals[2];
   uint32_t* cnt;        // [ntiles][kBins], rewritten by every pass
@@ -792,10 +804,11 @@ struct SortWs {
 
 void carve_sort(Carver& c, int64_t n, SortWs* w) {
   const int64_t nn = n > 0 ? n : 1;
-  w->status = c.take<int32_t>(64);
   for (int i = 0; i < 2; ++i) w->keys[i] = c.take<uint64_t>(nn);  // sized for 64-bit keys
   for (int i = 0; i < 2; ++i) w->vals[i] = c.take<uint32_t>(nn);
   w->cnt_len = make_plan(nn, 1, 0, true).ntiles * kBins;  // the tile count depends on n only
+  w->nbad = ceil_div(w->cnt_len / kBins, kGroup);
+  w->bad = c.take<int32_t>(w->nbad);
   w->cnt = c.take<uint32_t>(w->cnt_len);
   w->gcnt = c.take<uint32_t>((ceil_div(w->cnt_len / kBins, kGroup) + 1) * kBins);  // + totals row
   w->bytes = c.total();
@@ -849,14 +862,14 @@ int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, con
     uint32_t* vout = w.vals[cur];
     if (pass == 0) {
       HADES_LAUNCH((radix_count_kernel<KeyT, true, IPT>), cgrid, cblock, 0, st, kin, n,
-                   shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.status);
+                   shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.bad);
       if (scanned) HADES_LAUNCH(radix_group_scan_kernel, sgrid, block, 0, st, w.gcnt, ngroups);
       HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, true, IPT>), grid,
                          block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
                          w.gcnt, ngroups, scanned, kout, vout);
     } else {
       HADES_LAUNCH((radix_count_kernel<KeyT, false, IPT>), cgrid, cblock, 0, st, kin, n,
-                   shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.status);
+                   shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.bad);
       if (scanned) HADES_LAUNCH(radix_group_scan_kernel, sgrid, block, 0, st, w.gcnt, ngroups);
       HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, false, IPT>), grid,
                          block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
@@ -879,7 +892,7 @@ int run_runs(const void* sorted_keys, const uint32_t* perm, int64_t n, const Pla
   HADES_LAUNCH((run_count_kernel<KeyT>), rgrid, block, 0, st, keys, n, w.run_cnt);
   HADES_LAUNCH_CHECK();
   HADES_LAUNCH((run_emit_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt, uids,
-                     w.seg_start, w.seg_of, num_unique, inverse);
+                     w.seg_start, w.seg_of, num_unique, inverse, w.sort.bad, w.sort.nbad);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }
@@ -904,6 +917,8 @@ int sort_ids(const int64_t* ids, int64_t n, int64_t id_bound, void* workspace,
     return set_error(HADES_ERR_WORKSPACE, "sort workspace too small: need %zu bytes, got %zu",
                      w.bytes, workspace_bytes);
   out->key64 = p.key64;
+  out->bad = w.bad;
+  out->nbad = w.nbad;
   return p.key64 ? run_sort<uint64_t>(ids, n, id_bound, p, w, st, &out->sorted_keys, &out->perm)
                  : run_sort<uint32_t>(ids, n, id_bound, p, w, st, &out->sorted_keys, &out->perm);
 }

@@ -65,8 +65,9 @@ __global__ __launch_bounds__(kThreads) void hash_accumulate_kernel(AccArgs a) {
     const int64_t id = a.ids[row0 + r];
     uint64_t h = mix64(static_cast<uint64_t>(id)) & mask;
     int64_t slot = -1;
+    // a negative id is never stored (-1 marks an empty slot): its row is dropped, status bit 3
     // bounded probe: every wave leaves the loop after at most num_slots steps
-    for (int64_t probe = 0; probe < a.num_slots; ++probe) {
+    for (int64_t probe = 0; id >= 0 && probe < a.num_slots; ++probe) {
       unsigned long long* kp = reinterpret_cast<unsigned long long*>(a.keys + h);
       int64_t k = static_cast<int64_t>(__hip_atomic_load(kp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
       if (k == kEmpty) {
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(kThreads) void hash_accumulate_kernel(AccArgs a) {
       h = (h + 1) & mask;
     }
     if (slot < 0) {
-      atomicOr(a.status, 1);
+      atomicOr(a.status, id < 0 ? 8 : 1);
     } else {
       a.cnt[slot] += a.in_cnt ? a.in_cnt[row0 + r] : 1;
     }
@@ -133,6 +134,7 @@ struct FlushArgs {
   int64_t* keys; float* accum; int64_t* cnt; int64_t dim;
   const int64_t* live_pos; const uint32_t* perm; const int64_t* num_out;
   int64_t* out_ids; float* out_sums; int64_t* out_cnts; int64_t cap;
+  const int32_t* bad; int64_t nbad; int32_t* status;
 };
 
 // out row j <- the live slot with the j-th smallest id; the slot is emptied
@@ -140,6 +142,12 @@ template <int VEC>
 __global__ __launch_bounds__(kThreads) void flush_emit_kernel(FlushArgs a) {
   typedef typename Vf<VEC>::type V;
   __shared__ int64_t s_slot[kRows];
+  // a stored id outside [0, id_bound] left the ids unsorted: the rows still leave, status bit 2
+  // says that their order is not ascending
+  if (blockIdx.x == 0) {
+    const int violated = any_flag_set(a.bad, a.nbad);
+    if (violated && threadIdx.x == 0) atomicOr(a.status, 4);
+  }
   const int64_t L = a.num_out[0];
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRows;
   const int64_t left = (L < a.cap ? L : a.cap) - row0;
@@ -282,7 +290,8 @@ int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slot
   SortResult sr;
   rc = sort_ids(w.ids, cap, id_bound > 0 ? id_bound + 1 : 0, w.sort_ws, w.sort_bytes, st, &sr);
   if (rc != HADES_OK) return rc;
-  FlushArgs a{keys, accum, cnt, dim, w.live_pos, sr.perm, num_out, out_ids, out_sums, out_cnts, cap};
+  FlushArgs a{keys, accum, cnt, dim, w.live_pos, sr.perm, num_out, out_ids, out_sums, out_cnts, cap,
+              sr.bad, sr.nbad, status};
   const dim3 grid(static_cast<unsigned>(ceil_div(cap, kRows))), block(kThreads);
   const bool vec4 = dim % 4 == 0 && (align_of_ptr(accum) % 16) == 0 && (align_of_ptr(out_sums) % 16) == 0;
   if (vec4)

@@ -34,7 +34,9 @@ def _dcode(t):
 
 
 class Workspace:
-    """A reusable, 256-byte aligned device scratch buffer that grows on demand."""
+    """A reusable, 256-byte aligned device scratch buffer that grows on demand.  One workspace
+    serves one stream at a time: work queued on another stream must be ordered after the work
+    that used it before (the module's default workspaces are kept per stream for that reason)."""
 
     def __init__(self, device="cuda"):
         self.device = torch.device(device)
@@ -42,8 +44,15 @@ class Workspace:
 
     def get(self, nbytes):
         if self.buf is None or self.buf.numel() < nbytes:
-            # zero-filled: the sort keeps a sticky status word at the start of its workspace
+            # zero-filled: the cold-data cache's flush keeps a sticky status word at the start
             self.buf = torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=self.device)
+        else:
+            # the caching allocator hands a freed block back to the stream it was allocated on:
+            # tell it when the buffer is used on another one
+            cur = torch.cuda.current_stream(self.device)
+            if cur != getattr(self, "_stream", cur):
+                self.buf.record_stream(cur)
+        self._stream = torch.cuda.current_stream(self.device)
         return self.buf
 
 
@@ -51,10 +60,17 @@ _default_ws = {}
 
 
 def _ws(device, kind):
-    key = (str(device), kind)
+    """The module's own workspace for (device, kind of operator, current stream): two streams
+    never share scratch memory by default."""
+    key = (str(device), kind, torch.cuda.current_stream(device).cuda_stream)
     if key not in _default_ws:
         _default_ws[key] = Workspace(device)
     return _default_ws[key]
+
+
+def _bound_error():
+    return RuntimeError("combine: an id lies outside [0, id_bound) (num_unique came back as -1); "
+                        "pass id_bound=0 for ids without a known bound")
 
 
 # ---- kernel timing -------------------------------------------------------------
@@ -261,10 +277,22 @@ class CombinePlan:
     """The id-only half of a combine: sort permutation and run boundaries (kept in `workspace`),
     the distinct ids and their number.  Made by combine_plan, consumed by combine_apply."""
 
-    def __init__(self, n, dim, id_bound, uids, num_unique, inverse, workspace):
+    def __init__(self, n, dim, id_bound, uids, num_unique, inverse, workspace, buf):
         self.n, self.dim, self.id_bound = n, dim, id_bound
         self.uids, self.num_unique, self.inverse = uids, num_unique, inverse
         self.workspace = workspace
+        # the buffer the plan was written into: a workspace that grew or was given to a later
+        # plan no longer holds it
+        self._buf_ptr, self._buf_len = buf.data_ptr(), buf.numel()
+        workspace._plan = self
+
+    def check_live(self):
+        buf = self.workspace.buf
+        if (buf is None or buf.data_ptr() != self._buf_ptr or buf.numel() != self._buf_len
+                or getattr(self.workspace, "_plan", None) is not self):
+            raise RuntimeError("combine plan invalidated: its workspace was reallocated or reused "
+                               "by a later plan before combine_apply consumed it")
+        return buf
 
 
 def combine_plan(idx, dim, id_bound=0, return_inverse=False, workspace=None, out=None):
@@ -284,7 +312,7 @@ def combine_plan(idx, dim, id_bound=0, return_inverse=False, workspace=None, out
     ws = workspace.get(_lib.query("hades_combine_workspace_bytes", n, int(dim)))
     _lib.call("hades_combine_plan", _ptr(idx), n, int(dim), int(id_bound), _ptr(uids),
               _ptr(num_unique), _opt(inverse), _ptr(ws), ws.numel(), _stream())
-    return CombinePlan(n, int(dim), int(id_bound), uids, num_unique, inverse, workspace)
+    return CombinePlan(n, int(dim), int(id_bound), uids, num_unique, inverse, workspace, ws)
 
 
 def combine_apply(plan, grad, mode=COMBINE_FAST, out=None):
@@ -299,16 +327,19 @@ def combine_apply(plan, grad, mode=COMBINE_FAST, out=None):
         cnts = torch.empty(plan.n, dtype=torch.int64, device=dev)
     else:
         sums, cnts = out
-    ws = plan.workspace.get(_lib.query("hades_combine_workspace_bytes", plan.n, plan.dim))
+    ws = plan.check_live()
     _lib.call("hades_combine_apply", _ptr(grad), plan.n, plan.dim, plan.id_bound, int(mode),
               _ptr(sums), _ptr(cnts), _ptr(plan.num_unique), _ptr(ws), ws.numel(), _stream())
     return plan.uids, sums, cnts, plan.num_unique
 
 
 def combine(idx, grad, id_bound=0, mode=COMBINE_FAST, workspace=None):
-    """As combine_padded, trimmed to the number of distinct ids (one host synchronisation)."""
+    """As combine_padded, trimmed to the number of distinct ids (one host synchronisation).
+    Raises if an id violated id_bound."""
     uids, sums, cnts, num_unique = combine_padded(idx, grad, id_bound, mode, workspace=workspace)
     u = int(num_unique.item())
+    if u < 0:
+        raise _bound_error()
     return uids[:u], sums[:u], cnts[:u]
 
 

@@ -38,9 +38,13 @@ def unique_grads(idx, grad, cnt=None, id_bound=0, mode=ops.COMBINE_FAST):
         uids, sums, cnts, nu = ops.combine_padded(idx, grad, id_bound, mode)
         ops.rows_div_count_(sums, cnts, nu)
         u = int(nu.item())
+        if u < 0:
+            raise ops._bound_error()
         return uids[:u], sums[:u]
     uids, sums, _, nu, inverse = ops.combine_padded(idx, grad, id_bound, mode, return_inverse=True)
     u = int(nu.item())
+    if u < 0:
+        raise ops._bound_error()
     grad_cnt = torch.ones(u, dtype=cnt.dtype, device=cnt.device)
     grad_cnt.index_add_(0, inverse.long(), cnt)
     sums = sums[:u] / grad_cnt.unsqueeze(1)

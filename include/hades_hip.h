@@ -225,8 +225,9 @@ int hades_cached_set(const void* src, void* cold_dst, void* hot_dst, const int64
  * (fewer sort passes); id_bound == 0 sorts all 64 bits as signed integers.
  * mode: HADES_COMBINE_FAST or HADES_COMBINE_EXACT.  n must be < 2^30.
  * Optional output (may be NULL): inverse[i] = index of idx[i] in uids (int32[n]).
- * The first int32 of the workspace is a sticky status word: bit 0 is set when an id violated
- * id_bound (the result is then unspecified).  Zero-fill the workspace once before first use. */
+ * If an id violates id_bound, num_unique[0] is set to -1 and the other outputs are unspecified;
+ * every operator of this library that takes num_unique treats a negative value as "no live rows",
+ * so nothing is read or written out of range downstream.  The workspace needs no initialisation. */
 size_t hades_combine_workspace_bytes(int64_t n, int64_t dim);
 int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim, int64_t id_bound,
                   int mode, int64_t* uids, float* sums, int64_t* cnts, int64_t* num_unique,
@@ -281,8 +282,12 @@ int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num
  * EmbCacheServer._accumulate_gradients_cold_remote (python/EmbCache/server.py:546-562): per unique
  * incoming id  buf[slot] += g; cnt[slot] += c; key[slot] = id.
  * num_slots must be a power of two.  keys: int64[num_slots] (empty = -1), accum: float[num_slots,dim],
- * cnt: int64[num_slots].  ids within one call must be duplicate-free (combine first).
- * status[0] (int32, device) is set non-zero if the table is full. */
+ * cnt: int64[num_slots].  Precondition: the ids of one call are duplicate-free (combine first);
+ * duplicates inside a call race on the count and the row.
+ * status[0] (int32, device, sticky, cleared by the caller) collects error bits: 1 the table was
+ * full and a row was dropped; 2 more live entries than the flush capacity (nothing emitted);
+ * 4 a stored id was outside [0, id_bound] at flush time (rows emitted, but not in ascending
+ * order); 8 a negative id was offered to accumulate (its row was dropped: -1 marks an empty slot). */
 int hades_hash_clear(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots, int64_t dim,
                      void* stream);
 int hades_hash_accumulate(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots,
@@ -292,7 +297,7 @@ int hades_hash_accumulate(int64_t* keys, float* accum, int64_t* cnt, int64_t num
 /* Flush: emit every live slot as (id, sum row, count) in ascending id order, then clear the table
  * (evident intent of python/EmbCache/server.py:413-419; see the note on :414 in the oracle).
  *   out_ids int64[cap], out_sums float[cap, dim], out_cnts int64[cap], num_out int64[1] (device)
- * cap bounds the number of live slots emitted (status[0] set non-zero if exceeded). */
+ * cap bounds the number of live slots emitted (status bit 2 and num_out[0] = 0 if exceeded). */
 size_t hades_hash_flush_workspace_bytes(int64_t num_slots, int64_t cap);
 int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots, int64_t dim,
                      int64_t id_bound, int64_t* out_ids, float* out_sums, int64_t* out_cnts,
@@ -308,8 +313,9 @@ int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slot
  *   split_sizes[g] = number of rows owned by g, g in [0, num_owners) (:48-52, int64 on the device)
  *   perm_out[j] (optional) = input position of output row j.
  * grad (dim columns of dtype) and cnt are optional, each together with its output.
- * Rows keep their input order inside a bucket.  An owner outside [0, num_owners) sets bit 0 of the
- * first workspace word and makes the result unspecified. */
+ * Rows keep their input order inside a bucket.  If an owner falls outside [0, num_owners) (a
+ * negative id, an id beyond the last range), every entry of split_sizes is -1 and the other
+ * outputs are unspecified. */
 size_t hades_bucket_workspace_bytes(int64_t n);
 int hades_bucket_by_owner(const int64_t* ids, int64_t n, const int64_t* range_partition,
                           int64_t num_part, int64_t local_num_gpus, int64_t num_owners,
