@@ -16,6 +16,7 @@ LIB_PATH = os.environ.get("HADES_LIB_PATH") or os.path.join(_HERE, "csrc", "libh
 F32, F64 = 0, 1
 I32, I64, I16, I8, U8 = 0, 1, 2, 3, 4
 COMBINE_FAST, COMBINE_EXACT = 0, 1
+COMBINE_STATIC_SCRATCH_BYTES = 16 << 20
 
 _P = c_void_p
 _L = c_int64
@@ -52,6 +53,7 @@ _SIGNATURES = {
     "hades_cached_fetch_loc": [_P, _P, _P, _P, _L, _P, _L, c_int, _P],
     "hades_cached_set": [_P, _P, _P, _P, _L, _P, _L, _P, _L, c_int, _P],
     "hades_combine": [_P, _P, _L, _L, _L, c_int, _P, _P, _P, _P, _P, _P, c_size_t, _P],
+    "hades_combine_static": [_P, _P, _L, _L, _L, c_int, _P, _P, _P, _P, _P, _P],
     "hades_combine_plan": [_P, _L, _L, _L, _P, _P, _P, _P, c_size_t, _P],
     "hades_combine_apply": [_P, _L, _L, _L, c_int, _P, _P, _P, _P, c_size_t, _P],
     "hades_rows_div_count": [_P, _P, _P, _L, _L, c_int, _P],

@@ -28,6 +28,12 @@
 #include "internal.h"
 
 #include <atomic>
+#include <mutex>
+
+// Scratch memory of hades_combine_static: one copy per GPU, held from the moment the code object
+// is loaded on that GPU until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress; the address kernels are given is the one that call returns.
+static __device__ __align__(256) unsigned char g_static_scratch[HADES_COMBINE_STATIC_SCRATCH_BYTES];
 
 namespace hades {
 namespace {
@@ -1057,6 +1063,38 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
   if (rc != HADES_OK) return rc;
   return hades_combine_apply(grad, n, dim, id_bound, mode, sums, cnts, num_unique, workspace,
                              workspace_bytes, stream);
+}
+
+int hades_combine_static(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
+                         int64_t id_bound, int mode, int64_t* uids, float* sums, int64_t* cnts,
+                         int64_t* num_unique, int32_t* inverse, void* stream) {
+  HADES_REQUIRE(n >= 0 && dim >= 1, "n must be >= 0 and dim >= 1");
+  const size_t need = hades_combine_workspace_bytes(n, dim);
+  HADES_REQUIRE(need <= size_t(HADES_COMBINE_STATIC_SCRATCH_BYTES),
+                "hades_combine_static: n=%lld rows of dim=%lld need %zu bytes of scratch, the "
+                "library holds %zu; use hades_combine with a workspace of your own",
+                (long long)n, (long long)dim, need, size_t(HADES_COMBINE_STATIC_SCRATCH_BYTES));
+  // device address of this GPU's copy of the scratch array, looked up once per device
+  static std::mutex mu;
+  static void* scratch_of[64] = {};
+  int device = 0;
+  HADES_HIP_TRY(hipGetDevice(&device));
+  HADES_REQUIRE(device >= 0 && device < 64, "device ordinal %d out of range", device);
+  void* scratch = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (scratch_of[device] == nullptr) {
+      void* p = nullptr;
+      HADES_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_scratch)));
+      HADES_REQUIRE(p != nullptr, "hipGetSymbolAddress returned a null scratch address");
+      scratch_of[device] = p;
+    }
+    scratch = scratch_of[device];
+  }
+  // Nothing in the scratch has to start at zero: every word a kernel reads was written earlier in
+  // the same call (count rows, bound flags, run tables and partial rows are rewritten in full).
+  return hades_combine(idx, grad, n, dim, id_bound, mode, uids, sums, cnts, num_unique, inverse,
+                       scratch, size_t(HADES_COMBINE_STATIC_SCRATCH_BYTES), stream);
 }
 
 int hades_rows_div_count(float* sums, const int64_t* cnts, const int64_t* num_unique,

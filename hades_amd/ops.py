@@ -343,6 +343,26 @@ def combine(idx, grad, id_bound=0, mode=COMBINE_FAST, workspace=None):
     return uids[:u], sums[:u], cnts[:u]
 
 
+def combine_static(idx, grad, id_bound=0, mode=COMBINE_FAST, out=None):
+    """combine_padded on the library's own fixed scratch array (no workspace, nothing allocated by
+    the library): for callers that cannot allocate.  Batches whose scratch need exceeds
+    COMBINE_STATIC_SCRATCH_BYTES are refused.  Calls that overlap on one GPU race on the array."""
+    _i64(idx, "idx"); _dev(grad, "grad")
+    _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
+    n, dim = idx.numel(), grad.size(1)
+    _check(grad.size(0) == n, "grad must have one row per id")
+    dev = idx.device
+    if out is None:
+        out = (torch.empty(n, dtype=torch.int64, device=dev),
+               torch.empty((n, dim), dtype=torch.float32, device=dev),
+               torch.empty(n, dtype=torch.int64, device=dev),
+               torch.empty(1, dtype=torch.int64, device=dev))
+    uids, sums, cnts, num_unique = out
+    _lib.call("hades_combine_static", _ptr(idx), _ptr(grad), n, dim, int(id_bound), int(mode),
+              _ptr(uids), _ptr(sums), _ptr(cnts), _ptr(num_unique), _NULL, _stream())
+    return uids, sums, cnts, num_unique
+
+
 def rows_div_count_(sums, cnts, num_unique=None, one_plus=False):
     """In place: sums[u] /= (cnts[u] + one_plus) for the live rows."""
     _dev(sums, "sums"); _i64(cnts, "cnts")

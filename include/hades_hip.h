@@ -246,6 +246,22 @@ int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bo
                         float* sums, int64_t* cnts, const int64_t* num_unique, void* workspace,
                         size_t workspace_bytes, void* stream);
 
+/* hades_combine with the scratch memory inside the library.  No counterpart in the reference.  It
+ * is for callers that cannot allocate device memory or hand over a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The call allocates and frees
+ * nothing; its scratch is a fixed array of HADES_COMBINE_STATIC_SCRATCH_BYTES that every GPU the
+ * library runs on holds until the process ends.  Same arguments and results as hades_combine
+ * without the workspace pair.  A batch whose hades_combine_workspace_bytes(n, dim) exceeds the
+ * array is refused with HADES_ERR_ARG (the limit admits e.g. 262 144 ids of dim 128).  All calls
+ * on one GPU share that GPU's array: two calls that overlap in time on one GPU (different streams
+ * or threads) race, and the array must not be relied on between calls.  The first call on a
+ * device looks up the array's device address (hipGetSymbolAddress); make that call outside any
+ * graph capture. */
+#define HADES_COMBINE_STATIC_SCRATCH_BYTES (16u << 20)
+int hades_combine_static(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
+                         int64_t id_bound, int mode, int64_t* uids, float* sums, int64_t* cnts,
+                         int64_t* num_unique, int32_t* inverse, void* stream);
+
 /* unique_grads (python/EmbCache/sparse_optim.py:142-157): in-place division of the first
  * num_unique[0] rows of sums by cnts (plus `one_plus` added to the divisor: the reference starts
  * the count from ones when a cnt vector is supplied, :145-148). */
