@@ -1,19 +1,26 @@
 """Benchmark of the embedding-cache hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5] [--mode fast|exact]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]      the headline workload (cfg3) + cfg2 nested
+    python bench.py --workload cfg2|cfg3|cfg5 [--mode fast|exact] [--schedule serial|split|overlap|graph]
     python bench.py --workload cfg4          cold-gradient accumulator with delayed write-back
     python bench.py --workload cfg4 --flush-rule staleness    the cache server's own per-row rule
     python bench.py --workload neighbours    pre-exchange bucketing, index cache, cold-data cache
 
 One step = lookup + cached_fetch of the query rows, combine of the per-query gradients, and the
 sparse Adagrad update of every distinct row, on one batch of synthetic Zipf ids that is already
-resident in HBM.  Prints ONE JSON line: whole-step throughput in query rows/s, the roofline of the
-dominant kernel (algorithmic bytes / HIP-event time of its launches inside the timed region) and
-the same step timed on the host cores with the CPU oracle.
+resident in HBM.  The headline workload keeps 10 % of a 111 M x 128 table in HBM and the rest in
+pinned host memory; its step runs on the split schedule: lookup + stable hot/cold partition, then
+the hot rows through kernels that only touch HBM and the cold rows through kernels that only touch
+the host table, on two streams.  Prints ONE JSON line: whole-step throughput in query rows/s
+(mean, median, p10/p90 over the timed steps), the HBM roofline of every row kernel (algorithmic
+bytes / HIP-event time of its launches inside the timed region), the host-link roofline of the
+cold-row kernels against the nominal 64 GB/s and against pinned hipMemcpyAsync rates measured in
+the same run, and the same step timed on the host cores with the CPU oracle.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -24,16 +31,21 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 PCIE_PEAK_GBS = 64.0
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by what the
-# same counters read for a plain 256 MiB copy: reads x2.000, writes x1.000), per workload and
-# kernel id (1 cached_fetch mover, 2 segmented sum, 3 Adagrad).  Hardware counters cannot be read
-# from inside this script, so the figures of the profiled run are recorded here; a workload or
-# kernel that was not profiled reports null.
-MEASURED_TRAFFIC_BYTES = {
-    ("cfg2", "fast", 1): 185.4e6,
-    ("cfg2", "fast", 2): 142.3e6,
-    ("cfg2", "fast", 3): 194.5e6,
-}
+
+def measured_traffic(workload, mode):
+    """HBM bytes per launch from the committed rocprofv3 counter summary of this workload
+    (profiles/<workload>_step_hbm_traffic.txt, lines `TRAFFIC kernel=<key> bytes=<n>`), or {} if
+    there is none: hardware counters cannot be read from inside this script."""
+    path = os.path.join(ROOT, "profiles", "%s_step_hbm_traffic.txt" % workload)
+    out = {}
+    if mode != "fast" or not os.path.exists(path):
+        return out
+    with open(path) as f:
+        for line in f:
+            m = re.match(r"\s*TRAFFIC\s+kernel=(\S+)\s+bytes=([0-9.eE+]+)", line)
+            if m:
+                out[m.group(1)] = float(m.group(2))
+    return out
 
 
 def parse_args():
@@ -41,23 +53,25 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
-    ap.add_argument("--schedule", default="serial", choices=["serial", "overlap", "graph"],
-                    help="serial: every kernel of the step on one stream (the default: measured "
-                         "faster); overlap: the sort of the ids runs on a side stream next to the "
-                         "fetch; graph: every step is the replay of a HIP graph captured once per "
-                         "batch (no kernel inside a replay can be bracketed with events, so the "
-                         "roofline time is taken from eager steps before the timed region)")
+    ap.add_argument("--schedule", default=None, choices=["serial", "split", "overlap", "graph"],
+                    help="serial: every kernel of the step on one stream, hot and cold rows in the "
+                         "same kernels (default when the whole table is in HBM); split: lookup + "
+                         "hot/cold partition, hot rows on one stream, cold rows on another (default "
+                         "when the cold table is in host memory); overlap: serial with the sort of "
+                         "the ids on a side stream next to the fetch; graph: serial, every step the "
+                         "replay of a HIP graph captured once per batch")
     ap.add_argument("--flush-rule", default="every8", choices=["every8", "staleness"],
                     help="cfg4 only: write the accumulated cold gradients back every 8 steps (hash "
                          "accumulator), or per row by the cache server's staleness rule (cold-data "
                          "cache)")
     ap.add_argument("--batches", type=int, default=4, help="distinct pre-generated id batches")
     ap.add_argument("--event-every", type=int, default=4,
-                    help="bracket every n-th launch of the dominant kernel with HIP events inside "
-                         "the timed region (1 = every launch)")
+                    help="bracket the row kernels with HIP events in every n-th timed step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="headline run only: skip the nested cfg2 measurement")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three plain 256 MiB device copies before the timed region "
@@ -71,6 +85,17 @@ def log(msg):
 
 
 _T0 = time.perf_counter()
+
+
+def pct(xs, p):
+    """p-th percentile (linear interpolation) of a list."""
+    xs = sorted(xs)
+    if not xs:
+        return float("nan")
+    k = (len(xs) - 1) * p / 100.0
+    lo = int(k)
+    hi = min(lo + 1, len(xs) - 1)
+    return xs[lo] + (xs[hi] - xs[lo]) * (k - lo)
 
 
 class Workload:
@@ -99,9 +124,10 @@ class Workload:
         synth.fill_normal_(table, 0.01, seed, progress=log if N > 50_000_000 else None)
         hot_ids = synth.hot_ids(N, H, device) if H else torch.empty(0, dtype=torch.int64, device=device)
         log("hot copies and optimizer state")
-        # cfg3: the cold weights are the pinned host table; the cold Adagrad state stays in HBM
-        # (a second 57 GB page-locked allocation is refused on the benchmark box, and 288 GB of
-        # HBM have the room)
+        # cfg3: the cold weights are the pinned host table; the cold Adagrad state stays in HBM.
+        # The benchmark box refuses a page-locked allocation that would hold weights and state
+        # together (113.7 GB in one piece: hipHostMalloc says out of memory; 56.8 GB is granted),
+        # and 288 GB of HBM have the room.
         self.opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=device,
                                  state_on_device=self.host_cold)
         log("sampling %d batches of %d ids" % (nbatches, self.n))
@@ -123,23 +149,130 @@ class Workload:
     def describe(self):
         return ("%s: %d x %d fp32 table (%s), hot %d rows in HBM, %d ids/step zipf s=%.2f%s" %
                 (self.name, self.N, self.D,
-                 "cold weights in pinned host memory read zero-copy, cold Adagrad state in HBM"
-                 if self.host_cold
+                 "cold weights in pinned host memory read and written zero-copy; deviation: cold "
+                 "Adagrad state in HBM, the box refuses the 113.7 GB page-locked allocation that "
+                 "would hold weights and state" if self.host_cold
                  else "all in HBM", self.H, self.n, self.cfg["zipf_s"],
                  ", %d trainer batches concatenated" % self.trainers if self.trainers > 1 else ""))
 
 
-def run_gpu(args):
+def link_probe(dev, nbytes=256 << 20, reps=4):
+    """Pinned hipMemcpyAsync rates of this box, GB/s: host to device, device to host, and each
+    direction while the other runs on a second stream."""
+    import torch
+    h1 = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+    h2 = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+    d1 = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    d2 = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+
+    def h2d():
+        with torch.cuda.stream(s1):
+            d1.copy_(h1, non_blocking=True)
+
+    def d2h():
+        with torch.cuda.stream(s2):
+            h2.copy_(d2, non_blocking=True)
+
+    def rate(fns):
+        for f in fns:
+            f()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            for f in fns:
+                f()
+        torch.cuda.synchronize()
+        return nbytes * reps / (time.perf_counter() - t0) / 1e9
+
+    out = {"h2d_GB/s": round(rate([h2d]), 2), "d2h_GB/s": round(rate([d2h]), 2),
+           "both_ways_each_GB/s": round(rate([h2d, d2h]), 2),
+           "note": "pinned hipMemcpyAsync of %d MiB, %d repetitions" % (nbytes >> 20, reps)}
+    del h1, h2, d1, d2
+    return out
+
+
+def parity_gate(wl, step_fn, rows=20_000):
+    """One untimed step in the deterministic-order mode on the first `rows` ids of batch 0,
+    through the same schedule as the timed steps, checked against torch's own device operators:
+    slots and fetched rows bit-exact, distinct ids and counts exact, summed gradients and the
+    updated weight / state rows within 1e-5 relative per row.  Raises on a mismatch."""
+    import torch
+    from hades_amd import ops
+    opt = wl.opt
+    m = min(rows, wl.n)
+    q = wl.ids[0][:m].contiguous()
+    g = wl.grads[0][:m].contiguous()
+    hot = opt.hot_ids
+
+    def table_rows(cold, hot_t, ids):
+        """rows of (cold, hot_t) named by ids, gathered with torch indexing only"""
+        pos = torch.searchsorted(hot, ids, right=True)
+        hit = (pos > 0) & (hot[(pos - 1).clamp_(min=0)] == ids) if hot.numel() else torch.zeros_like(ids, dtype=torch.bool)
+        loc = torch.where(hit, pos - 1, torch.full_like(pos, -1))
+        out = torch.empty((ids.numel(), wl.D), dtype=torch.float32, device=ids.device)
+        if hot.numel():
+            out[hit] = hot_t[loc[hit]]
+        miss = ~hit
+        if cold.is_cuda:
+            out[miss] = cold[ids[miss]]
+        else:
+            out[miss] = cold[ids[miss].cpu()].to(ids.device)
+        return out, loc
+
+    want_rows, want_loc = table_rows(opt.cold_w, opt.hot_w, q)
+    got_loc = ops.lookup(q, opt.hot_set)
+    assert torch.equal(got_loc, want_loc), "parity gate: lookup slots differ"
+    uniq, inv, cnt = torch.unique(q, sorted=True, return_inverse=True, return_counts=True)
+    sums64 = torch.zeros((uniq.numel(), wl.D), dtype=torch.float64, device=q.device)
+    sums64.index_add_(0, inv, g.double())
+    w0, _ = table_rows(opt.cold_w, opt.hot_w, uniq)
+    s0, _ = table_rows(opt.cold_s, opt.hot_s, uniq)
+
+    rows_out, (uids, sums, cnts, nu) = step_fn(q, g, ops.COMBINE_EXACT)
+    torch.cuda.synchronize()
+    assert torch.equal(rows_out[:m], want_rows), "parity gate: fetched rows differ"
+    u = int(nu.item())
+    assert u == uniq.numel() and torch.equal(uids[:u], uniq), "parity gate: distinct ids differ"
+    assert torch.equal(cnts[:u], cnt), "parity gate: counts differ"
+
+    def close(a, b, what):
+        err = (a.double() - b.double()).abs().amax(dim=1)
+        scale = b.double().abs().amax(dim=1).clamp_(min=1e-30)
+        worst = float((err / scale).max())
+        assert worst <= 1e-5, "parity gate: %s off by %.3g relative" % (what, worst)
+        return worst
+
+    e_sum = close(sums[:u], sums64, "summed gradients")
+    gs = sums[:u]
+    s1 = s0 + gs * gs
+    w1 = w0 - (0.01 * gs) / (s1.sqrt() + 1e-10)
+    w_got, _ = table_rows(opt.cold_w, opt.hot_w, uniq)
+    s_got, _ = table_rows(opt.cold_s, opt.hot_s, uniq)
+    e_w = close(w_got, w1, "updated weights")
+    e_s = close(s_got, s1, "updated Adagrad state")
+    return {"rows": m, "distinct": u, "mode": "exact",
+            "bit_exact": ["lookup slots", "fetched rows", "distinct ids", "counts"],
+            "max_rel_err": {"sums": e_sum, "weights": e_w, "state": e_s}, "tolerance": 1e-5,
+            "against": "torch device ops (searchsorted, indexing, unique + float64 index_add_, "
+                       "Adagrad closed form)"}
+
+
+def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
     import torch
     from hades_amd import ops
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    wl = Workload(args.workload, args.batches, dev)
+    wl = Workload(workload, args.batches, dev)
     opt = wl.opt
     mode = ops.COMBINE_FAST if args.mode == "fast" else ops.COMBINE_EXACT
-    ws = ops.Workspace(dev)
     nb = len(wl.ids)
-    phases = ("fetch", "combine", "update")
+    n, D, N = wl.n, wl.D, wl.N
+    K = args.steps
+    if schedule is None:
+        schedule = "split" if wl.host_cold else "serial"
+    split = schedule == "split"
+    overlap = schedule == "overlap"
 
     def new_events(count):
         evs = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
@@ -147,38 +280,58 @@ def run_gpu(args):
             e.record()          # torch creates the HIP event on first use
         return evs
 
-    ev = [new_events(4) for _ in range(args.steps)]
-    kev = [new_events(2) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-
     uids_o, sums_o, cnts_o, nu_o = wl.comb_out
-    overlap = args.schedule == "overlap"
 
-    def step(i, events=None):
-        """fetch -> combine -> update of batch i.  With the overlapped schedule the id-only half
-        of the combine (sort + run boundaries) is issued on a side stream before the fetch, as a
-        trainer that knows the ids at forward time would do; everything that touches rows stays
-        on the main stream in program order."""
-        q, g = wl.ids[i % nb], wl.grads[i % nb]
-        if overlap:
-            plan = opt.prepare(q, out=(uids_o, nu_o))
+    def run_step(q, g, cmode, events=None, timing=None):
+        """fetch -> combine -> update of one batch.
+
+        serial: one stream; hot and cold rows share the fetch kernel and the update kernel.
+        overlap: serial, but the id-only half of the combine (sort + run boundaries) is issued on
+        a side stream before the fetch, as a trainer that knows the ids at forward time would do.
+        split: lookup + hot/cold partition; the hot gather on the main stream and the cold gather
+        on the cold stream; the id-only half of the combine runs on the main stream meanwhile
+        (it needs the ids only); join: the fetched rows are complete, which is where a trainer's
+        forward and backward would sit; segmented sum of the gradients; lookup + partition of the
+        distinct ids; hot update on the main stream and cold update on the cold stream; join."""
+        sizes = q.numel()
+        rows = wl.rows_out[:sizes]
+        out_ids = (uids_o[:sizes], nu_o)
+        out_sum = (sums_o[:sizes], cnts_o[:sizes])
         if events: events[0].record()
-        ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_set, out=wl.rows_out)
-        if events: events[1].record()
-        if overlap:
-            torch.cuda.current_stream().wait_event(plan.ready)
+        if split:
+            opt.fetch_split(q, out=rows, join=False, timing=timing)
+            plan = ops.combine_plan(q, D, id_bound=N, workspace=opt._ws, out=out_ids)
+            opt.join()
+            if events: events[1].record()
+            res = ops.combine_apply(plan, g, cmode, out=out_sum)
+            if events: events[2].record()
+            opt.update_split(res[0], res[1], res[3], join=True, timing=timing)
         else:
-            plan = ops.combine_plan(q, wl.D, id_bound=wl.N, workspace=opt._ws, out=(uids_o, nu_o))
-        uids, sums, cnts, nu = ops.combine_apply(plan, g, mode, out=(sums_o, cnts_o))
-        if events: events[2].record()
-        opt.update(uids, sums, nu)
+            if overlap:
+                plan = opt.prepare(q, out=out_ids)
+            ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_set, out=rows)
+            if events: events[1].record()
+            if overlap:
+                torch.cuda.current_stream().wait_event(plan.ready)
+            else:
+                plan = ops.combine_plan(q, D, id_bound=N, workspace=opt._ws, out=out_ids)
+            res = ops.combine_apply(plan, g, cmode, out=out_sum)
+            if events: events[2].record()
+            opt.update(res[0], res[1], res[3])
         if events: events[3].record()
+        return rows, res
 
-    # the three row-moving kernels of a step; the dominant one is found on a few untimed steps
-    kernels = {ops.KERNEL_CACHED_FETCH: "row_move_kernel<AddrFetchSorted> (hades_cached_fetch)",
-               ops.KERNEL_SEG_SUM: "seg_chunk_kernel (hades_combine)" if args.mode == "fast"
-               else "seg_exact_kernel (hades_combine)",
-               ops.KERNEL_ADAGRAD: "adagrad_kernel (hades_adagrad_update)"}
+    def step(i, events=None, timing=None):
+        run_step(wl.ids[i % nb], wl.grads[i % nb], mode, events, timing)
+
+    gate = None
+    if with_gate:
+        gate = parity_gate(wl, lambda q, g, m: run_step(q, g, m))
+        log("parity gate passed: %s" % json.dumps(gate["max_rel_err"]))
+    link = link_probe(dev) if (with_link and wl.host_cold) else None
+    if link:
+        log("host link: %s" % json.dumps(link))
+
     for i in range(args.warmup):
         step(i)
     if args.copy_probe:
@@ -188,28 +341,46 @@ def run_gpu(args):
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
-    probe_ms = {}
-    for kid in kernels:
-        acc = 0.0
-        for i in range(3):
-            ops.profile_kernel(kid, kev[i][0], kev[i][1])
-            step(i)
-        torch.cuda.synchronize()
-        for i in range(3):
-            acc += kev[i][0].elapsed_time(kev[i][1])
-        probe_ms[kid] = acc / 3
-    ops.profile_kernel(0)
-    dominant = max(kernels, key=lambda k: probe_ms[k])
+    torch.cuda.synchronize()
 
-    # Timed region: exactly K steps.  An event record is a packet of its own on the queue (3-4 us
-    # of GPU time each), so only every `event_every`-th launch of the dominant kernel is bracketed
-    # here and the per-phase events are taken in a second, untimed pass over the same steps.
+    # ---- the row kernels and how each is bracketed ----
+    # split: the four listed kernels by event pairs recorded from Python on their own stream, the
+    # segmented sum by the library's hook; serial: all three by the hook, one kernel per sampled
+    # step in rotation (the hook brackets one kernel at a time).
     every = max(1, args.event_every)
-    sampled = [i for i in range(args.steps) if i % every == 0]
-    if args.schedule == "graph":
+    sampled = [i for i in range(K) if i % every == 0]
+    seg_name = "seg_chunk_kernel" if args.mode == "fast" else "seg_exact_kernel + seg_exact_long_kernel"
+    if split:
+        knames = {"hot_fetch": "row_move_listed_kernel<gather> over the hot class (hades_fetch_listed)",
+                  "cold_fetch": "row_move_listed_kernel<gather> over the cold class (hades_fetch_listed)",
+                  "seg_sum": seg_name + " (hades_combine_apply)",
+                  "hot_update": "adagrad_listed_kernel over the hot class (hades_adagrad_update_listed)",
+                  "cold_update": "adagrad_listed_kernel over the cold class (hades_adagrad_update_listed)"}
+        hook_of = {"seg_sum": ops.KERNEL_SEG_SUM}
+    else:
+        knames = {"fetch": "row_move_kernel<AddrFetchSorted> (hades_cached_fetch)",
+                  "seg_sum": seg_name + " (hades_combine_apply)",
+                  "update": "adagrad_kernel (hades_adagrad_update)"}
+        hook_of = {"fetch": ops.KERNEL_CACHED_FETCH, "seg_sum": ops.KERNEL_SEG_SUM,
+                   "update": ops.KERNEL_ADAGRAD}
+    kev = {i: {k: new_events(2) for k in knames} for i in sampled}
+    step_ev = new_events(K + 1)
+    phase_ev = [new_events(4) for _ in range(K)]
+    torch.cuda.synchronize()
+    hooks = sorted(hook_of)
+    armed = {}
+
+    kernel_ms = {k: [] for k in knames}
+    if schedule == "graph":
         # one captured graph per pre-generated batch (the library allocates nothing and clears
         # memory with kernels only, so a step captures as it is); launches inside a replay cannot
-        # be bracketed, so the dominant kernel's time is that of the eager probe steps above
+        # be bracketed, so the kernels are timed on eager steps before the timed region
+        for j, i in enumerate(sampled):
+            hk = hooks[j % len(hooks)]
+            ops.profile_kernel(hook_of[hk], kev[i][hk][0], kev[i][hk][1])
+            step(i)
+            armed[i] = [hk]
+        ops.profile_kernel(0)
         graphs = []
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -224,92 +395,170 @@ def run_gpu(args):
             graphs[b].replay()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(args.steps):
+        step_ev[0].record()
+        for i in range(K):
             graphs[i % nb].replay()
+            step_ev[i + 1].record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-        ms_per_step = (t1 - t0) * 1e3 / args.steps
-        kernel_ms = probe_ms[dominant]
-        sampled = []
     else:
-        torch.cuda.synchronize()
+        # Timed region: exactly K steps.  One event record per step marks the step boundary
+        # (3-4 us of GPU time each, inside the measured time); the kernel brackets are taken in
+        # every `event_every`-th step only.
         t0 = time.perf_counter()
-        for i in range(args.steps):
+        step_ev[0].record()
+        for j_i, i in enumerate(range(K)):
+            tim = None
             if i % every == 0:
-                ops.profile_kernel(dominant, kev[i][0], kev[i][1])
+                j = i // every
+                if split:
+                    tim = {k: kev[i][k] for k in knames if k not in hook_of}
+                    hk = "seg_sum"
+                    armed[i] = list(knames)
+                else:
+                    hk = hooks[j % len(hooks)]
+                    armed[i] = [hk]
+                ops.profile_kernel(hook_of[hk], kev[i][hk][0], kev[i][hk][1])
             elif i % every == 1:
                 ops.profile_kernel(0)
-            step(i)
+            step(i, timing=tim)
+            step_ev[i + 1].record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         ops.profile_kernel(0)
-        ms_per_step = (t1 - t0) * 1e3 / args.steps
-        kernel_ms = sum(kev[i][0].elapsed_time(kev[i][1]) for i in sampled) / len(sampled)
+    ms_per_step = (t1 - t0) * 1e3 / K
+    for i, names in armed.items():
+        for k in names:
+            kernel_ms[k].append(kev[i][k][0].elapsed_time(kev[i][k][1]))
+    step_ms = [step_ev[i].elapsed_time(step_ev[i + 1]) for i in range(K)]
 
-    for i in range(args.steps):
-        step(i, ev[i])
+    # phases: a second, untimed pass with four event records per step on the main stream
+    for i in range(K):
+        step(i, events=phase_ev[i])
     torch.cuda.synchronize()
-    phase_ms = {p: sum(ev[i][k].elapsed_time(ev[i][k + 1]) for i in range(args.steps)) / args.steps
+    phases = ("fetch", "combine", "update")
+    phase_ms = {p: sum(phase_ev[i][k].elapsed_time(phase_ev[i][k + 1]) for i in range(K)) / K
                 for k, p in enumerate(phases)}
+
     # distinct ids per step and hot-hit statistics of the batches actually used
-    uniq, hot_hit, uniq_hot = [], [], []
+    uniq, hot_q, uniq_hot = [], [], []
     for q in wl.ids:
         u = torch.unique(q)
         uniq.append(u.numel())
         if wl.H:
-            hot_hit.append(float((ops.lookup(q, opt.hot_ids) >= 0).float().mean()))
+            hot_q.append(int((ops.lookup(q, opt.hot_ids) >= 0).sum()))
             uniq_hot.append(int((ops.lookup(u, opt.hot_ids) >= 0).sum()))
         else:
-            hot_hit.append(0.0)
+            hot_q.append(0)
             uniq_hot.append(0)
     U = sum(uniq) / len(uniq)
     U_hot = sum(uniq_hot) / len(uniq_hot)
-    hit = sum(hot_hit) / len(hot_hit)
-    n, D = wl.n, wl.D
-    # algorithmic bytes per launch (fp32).  Phases: fetch 16 + 8D per query row; combine
-    # n(8+4D) read + U(16+4D) written; Adagrad 8 + 20D per distinct row.  Kernels: the fetch and
-    # Adagrad kernels are their whole phase; the segmented-sum kernel reads n rows plus 8 bytes of
-    # sort output per row and writes U rows.
-    alg_bytes = {"fetch": n * (16 + 8 * D), "combine": n * (8 + 4 * D) + U * (16 + 4 * D),
-                 "update": U * (8 + 20 * D)}
-    kernel_bytes = {ops.KERNEL_CACHED_FETCH: alg_bytes["fetch"],
-                    ops.KERNEL_SEG_SUM: n * (8 + 4 * D) + U * 4 * D,
-                    ops.KERNEL_ADAGRAD: alg_bytes["update"]}
-    achieved = kernel_bytes[dominant] / (kernel_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": kernels[dominant], "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.mode, dominant)),
-                "kernel_us": round(kernel_ms * 1e3, 2),
-                "launches_timed": ("%d of the %d in the timed region" % (len(sampled), args.steps)
-                                   if sampled else "3 eager steps before the timed region"),
+    n_hot = sum(hot_q) / len(hot_q)
+    n_cold, U_cold = n - n_hot, U - U_hot
+    # Algorithmic bytes per launch (fp32; one launch covers the whole batch or its class).
+    # fetch 16 + 8D per query row; segmented sum n(8+4D) read + U*4D written; Adagrad 8 + 20D per
+    # distinct row.  A cold row moves 4D bytes over the host link in the fetch and 4D each way in
+    # the update (weights; the cold Adagrad state sits in HBM).
+    row_f, row_u = 16 + 8 * D, 8 + 20 * D
+    alg_bytes = {"fetch": n * row_f, "combine": n * (8 + 4 * D) + U * (16 + 4 * D), "update": U * row_u}
+    kbytes = {"fetch": n * row_f, "update": U * row_u, "seg_sum": n * (8 + 4 * D) + U * 4 * D,
+              "hot_fetch": n_hot * row_f, "cold_fetch": n_cold * row_f,
+              "hot_update": U_hot * row_u, "cold_update": U_cold * row_u}
+    traffic = measured_traffic(workload, args.mode)
+    kernels = {}
+    for k, name in knames.items():
+        if not kernel_ms[k]:
+            continue
+        ms = sum(kernel_ms[k]) / len(kernel_ms[k])
+        gbs = kbytes[k] / (ms * 1e-3) / 1e9
+        entry = {"kernel": name, "us": round(ms * 1e3, 2), "launches_timed": len(kernel_ms[k]),
+                 "bytes_per_launch": int(kbytes[k]), "GB/s": round(gbs, 1)}
+        if k.startswith("cold_") and wl.host_cold:
+            entry["bound"] = "pcie"
+        else:
+            entry["bound"] = "hbm"
+            entry["frac"] = round(gbs / HBM_PEAK_GBS, 4)
+            tb = traffic.get(k)
+            entry["traffic"] = tb
+            if tb:
+                entry["traffic_GB/s"] = round(tb / (ms * 1e-3) / 1e9, 1)
+                entry["traffic_frac"] = round(tb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        kernels[k] = entry
+    # the headline roofline: the HBM-bound row kernel that moves the most bytes (hot traffic)
+    hbm_keys = [k for k in kernels if kernels[k]["bound"] == "hbm"]
+    main_k = "hot_fetch" if "hot_fetch" in kernels else max(hbm_keys, key=lambda k: kbytes[k])
+    mk = kernels[main_k]
+    roofline = {"bound": "hbm", "kernel": mk["kernel"], "achieved": mk["GB/s"], "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": mk["frac"], "traffic": mk.get("traffic"),
+                "traffic_source": ("profiles/%s_step_hbm_traffic.txt (rocprofv3 FETCH_SIZE + "
+                                   "WRITE_SIZE of an earlier run of this command)" % workload)
+                if mk.get("traffic") else None,
+                "kernel_us": mk["us"], "launches_timed": "%d of the %d in the timed region" %
+                (mk["launches_timed"], K) if schedule != "graph" else "eager steps before the timed region",
                 "timing": "HIP events recorded on the launch stream right before and after the "
                           "launch: the kernel plus about 3 us of dispatch latency",
-                "bytes_per_launch": int(kernel_bytes[dominant]),
-                "other_kernels_us": {kernels[k]: round(probe_ms[k] * 1e3, 2) for k in kernels
-                                     if k != dominant}}
+                "bytes_per_launch": mk["bytes_per_launch"]}
+    if split:
+        hot_b = sum(kbytes[k] for k in ("hot_fetch", "seg_sum", "hot_update"))
+        hot_ms = sum(kernels[k]["us"] for k in ("hot_fetch", "seg_sum", "hot_update")) / 1e3
+        roofline["hot_traffic_all_row_kernels"] = {
+            "GB/s": round(hot_b / (hot_ms * 1e-3) / 1e9, 1),
+            "frac": round(hot_b / (hot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "note": "hot gather + segmented sum + hot update: algorithmic bytes over the sum of "
+                    "their kernel times"}
     per_phase = {p: {"ms": round(phase_ms[p], 4),
                      "GB/s": round(alg_bytes[p] / (phase_ms[p] * 1e-3) / 1e9, 1),
                      "frac_hbm": round(alg_bytes[p] / (phase_ms[p] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
                  for p in phases}
     total_bytes = sum(alg_bytes.values())
-    extra = {"phases": per_phase,
-             "phases_note": "from a second, untimed pass with four event records per step "
-                            "(each adds 3-4 us to its phase)",
-             "step_alg_GB": round(total_bytes / 1e9, 4),
-             "step_GB/s": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
-             "step_frac_hbm": round(total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-             "unique_per_step": round(U, 1), "unique_hot_per_step": round(U_hot, 1),
-             "hot_hit": round(hit, 4)}
+    res = {"workload": wl.describe(), "schedule": schedule, "n": n,
+           "ms_per_step": ms_per_step,
+           "step_us": {"mean": round(ms_per_step * 1e3, 1), "median": round(pct(step_ms, 50) * 1e3, 1),
+                       "p10": round(pct(step_ms, 10) * 1e3, 1), "p90": round(pct(step_ms, 90) * 1e3, 1),
+                       "note": "mean: wall clock over the K timed steps; median/p10/p90: the same "
+                               "steps by HIP events at the step boundaries"},
+           "roofline": roofline, "kernels": kernels,
+           "phases": per_phase,
+           "phases_note": "from a second, untimed pass with four event records per step (each adds "
+                          "3-4 us to its phase)" +
+                          ("; fetch = both gathers and the id sort that runs beside the cold one"
+                           if split else ""),
+           "step_alg_GB": round(total_bytes / 1e9, 4),
+           "step_GB/s": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+           "step_frac_hbm": round(total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+           "unique_per_step": round(U, 1), "unique_hot_per_step": round(U_hot, 1),
+           "hot_hit": round(n_hot / n, 4), "parity_gate": gate}
     if wl.host_cold:
-        cold_q = n * (1 - hit)
-        cold_u = U - U_hot
-        extra["pcie"] = {
-            "fetch_GB/s": round(cold_q * 4 * D / (phase_ms["fetch"] * 1e-3) / 1e9, 2),
-            "update_read_GB/s": round(cold_u * 4 * D / (phase_ms["update"] * 1e-3) / 1e9, 2),
-            "update_write_GB/s": round(cold_u * 4 * D / (phase_ms["update"] * 1e-3) / 1e9, 2),
-            "cold_query_rows": round(cold_q, 1), "cold_unique_rows": round(cold_u, 1),
-            "peak_per_direction": PCIE_PEAK_GBS}
-    return wl, ms_per_step, roofline, extra
+        def link_entry(rows, ms):
+            gbs = rows * 4 * D / (ms * 1e-3) / 1e9
+            e = {"MB": round(rows * 4 * D / 1e6, 2), "GB/s": round(gbs, 2),
+                 "frac_nominal": round(gbs / PCIE_PEAK_GBS, 4)}
+            return e, gbs
+        pcie = {"bound": "pcie", "peak": PCIE_PEAK_GBS, "unit": "GB/s per direction",
+                "cold_query_rows": round(n_cold, 1), "cold_unique_rows": round(U_cold, 1),
+                "memcpy": link}
+        if split:
+            f, f_gbs = link_entry(n_cold, kernels["cold_fetch"]["us"] / 1e3)
+            u, u_gbs = link_entry(U_cold, kernels["cold_update"]["us"] / 1e3)
+            timing_note = "cold-class kernels bracketed by HIP events on the cold stream"
+        else:
+            f, f_gbs = link_entry(n_cold, kernels["fetch"]["us"] / 1e3)
+            u, u_gbs = link_entry(U_cold, kernels["update"]["us"] / 1e3)
+            timing_note = "hot and cold rows share the kernels: kernel time of the whole fetch / update"
+        if link:
+            f["frac_memcpy_h2d"] = round(f_gbs / link["h2d_GB/s"], 4)
+            u["frac_memcpy_h2d"] = round(u_gbs / link["h2d_GB/s"], 4)
+            u["frac_memcpy_both_ways"] = round(u_gbs / link["both_ways_each_GB/s"], 4)
+        pcie["fetch_host_to_device"] = f
+        pcie["update_each_way_at_once"] = u
+        pcie["achieved"] = round(min(f_gbs, u_gbs), 2)
+        pcie["frac"] = round(min(f_gbs, u_gbs) / PCIE_PEAK_GBS, 4)
+        pcie["note"] = ("%s; the update reads and writes the cold weight rows (4D bytes each way "
+                        "per distinct cold row); achieved/frac = the lower of the two" % timing_note)
+        res["pcie"] = pcie
+    del wl, opt
+    torch.cuda.empty_cache()
+    return res
 
 
 def run_cfg4(args):
@@ -703,8 +952,10 @@ def main():
     if args.workload == "neighbours":
         run_neighbours(args)
         return
-    wl, ms_per_step, roofline, extra = run_gpu(args)
-    n = wl.n
+    res = run_gpu(args, args.workload, args.schedule)
+    ms_per_step = res.pop("ms_per_step")
+    n = res.pop("n")
+    schedule = res.pop("schedule")
     line = {
         "metric": "embedding rows/s (fetch+combine+update)",
         "value": round(n / (ms_per_step * 1e-3), 1),
@@ -713,22 +964,30 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
-        "step_us": round(ms_per_step * 1e3, 1),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": wl.describe(), "combine_mode": args.mode,
+        "config": {"workload": res.pop("workload"), "combine_mode": args.mode,
                    "optimizer": "sparse Adagrad lr=0.01 eps=1e-10",
-                   "schedule": "sort of the step's ids on a side stream, concurrent with its fetch"
-                   if args.schedule == "overlap" else
-                   "one stream, every step replayed from a HIP graph captured once per batch"
-                   if args.schedule == "graph" else "one stream"},
-        "roofline": roofline,
+                   "schedule": {"serial": "one stream, hot and cold rows in the same kernels",
+                                "split": "lookup + hot/cold partition; hot rows on the main stream, "
+                                         "cold rows on a second stream of the same priority",
+                                "overlap": "one stream + the sort of the step's ids on a side stream, "
+                                           "concurrent with its fetch",
+                                "graph": "one stream, every step replayed from a HIP graph captured "
+                                         "once per batch"}[schedule]},
     }
-    line.update(extra)
-    del wl
+    line.update(res)
+    if args.workload == "cfg3" and not args.no_secondary:
+        log("secondary workload cfg2 (whole table in HBM)")
+        sec = run_gpu(args, "cfg2", None, with_gate=False, with_link=False)
+        line["secondary"] = {"cfg2": {
+            "workload": sec["workload"], "schedule": sec["schedule"],
+            "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
+            "step_us": sec["step_us"], "step_frac_hbm": sec["step_frac_hbm"],
+            "roofline": sec["roofline"], "kernels": sec["kernels"], "phases": sec["phases"]}}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = run_cpu_baseline(args.workload, args.cpu_seconds)
     print(json.dumps(line))

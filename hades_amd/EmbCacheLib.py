@@ -57,8 +57,9 @@ def _dev(t, name):
     _check(t.is_contiguous(), "%s must be contiguous" % name)
 
 
-def _dev_or_pinned(t, name):
-    _check(t.is_contiguous(), "%s must be contiguous" % name)
+def _dev_or_pinned(t, name, contiguous=True):
+    if contiguous:
+        _check(t.is_contiguous(), "%s must be contiguous" % name)
     if not t.is_cuda:
         _check(t.is_pinned() or t.untyped_storage().data_ptr() in _registered,
                "%s is pageable host memory: pin it (cudaPin / pin_memory=True) before a kernel "
@@ -90,6 +91,40 @@ def _row_dim(ref, others):
 def pinned_empty(shape, dtype=torch.float32):
     """A page-locked, device-mapped host tensor (what the cold table should live in)."""
     return torch.empty(shape, dtype=dtype, pin_memory=True)
+
+
+_host_allocs = {}   # data_ptr -> (raw pointer, bytes) of tensors made by host_alloc
+
+
+def host_alloc(shape, dtype=torch.float32, coherent=True):
+    """A host tensor in memory from hades_host_alloc (page-locked and mapped into the device's
+    address space: kernels read and write it zero-copy).  coherent=False asks for coarse-grained
+    memory (see HADES_HOST_NONCOHERENT in the header).  Free it with host_free(tensor) once no
+    kernel uses it any more; the tensor and its views must not be touched afterwards."""
+    shape = tuple(int(x) for x in (shape if hasattr(shape, "__len__") else (shape,)))
+    numel = 1
+    for x in shape:
+        numel *= x
+    nbytes = numel * torch.empty((), dtype=dtype).element_size()
+    if nbytes == 0:
+        return torch.empty(shape, dtype=dtype)
+    raw = ctypes.c_void_p()
+    _lib.call("hades_host_alloc_flags", ctypes.byref(raw), nbytes,
+              0 if coherent else _lib.HOST_NONCOHERENT)
+    buf = (ctypes.c_char * nbytes).from_address(raw.value)
+    t = torch.frombuffer(buf, dtype=dtype).view(shape)
+    _host_allocs[t.data_ptr()] = (raw.value, nbytes)
+    _registered.add(t.untyped_storage().data_ptr())
+    return t
+
+
+def host_free(tensor):
+    """Gives the memory of a host_alloc tensor back (hades_host_free)."""
+    ptr = tensor.data_ptr()
+    _check(ptr in _host_allocs, "host_free: not a tensor made by host_alloc")
+    raw, _ = _host_allocs.pop(ptr)
+    _registered.discard(tensor.untyped_storage().data_ptr())
+    _lib.call("hades_host_free", ctypes.c_void_p(raw))
 
 
 # ---- pinning (src/cuda/pin_memory.cu:9-26) ----------------------------------

@@ -19,7 +19,14 @@ __version__ = "0.1.0"
 
 def install_as_embcachelib():
     """Registers hades_amd.EmbCacheLib under the name `EmbCacheLib`, so that unmodified reference
-    code (`import EmbCacheLib`, python/EmbCache/cache.py:2) binds to this implementation."""
+    code (`import EmbCacheLib`, python/EmbCache/cache.py:2) binds to this implementation.
+
+    What differs from the reference's module for such code: launches go to torch's current stream;
+    failures raise RuntimeError instead of ending the process; tensors must be contiguous; host
+    tensors given to a kernel must be page-locked already (cudaPin on pageable memory raises where
+    the platform refuses hipHostRegister: allocate with pin_memory=True or EmbCacheLib.host_alloc);
+    IndexCache lives in device memory, ignores its shared-memory arguments, accepts CPU or device
+    id tensors (CPU in, CPU out) and returns device tensors from getall."""
     from . import EmbCacheLib
     sys.modules["EmbCacheLib"] = EmbCacheLib
     return EmbCacheLib

@@ -16,6 +16,7 @@ LIB_PATH = os.environ.get("HADES_LIB_PATH") or os.path.join(_HERE, "csrc", "libh
 F32, F64 = 0, 1
 I32, I64, I16, I8, U8 = 0, 1, 2, 3, 4
 COMBINE_FAST, COMBINE_EXACT = 0, 1
+HOST_NONCOHERENT = 1
 COMBINE_STATIC_SCRATCH_BYTES = 16 << 20
 
 _P = c_void_p
@@ -30,6 +31,7 @@ _SIGNATURES = {
     "hades_pin": [_P, c_size_t],
     "hades_unpin": [_P],
     "hades_host_alloc": [ctypes.POINTER(c_void_p), c_size_t],
+    "hades_host_alloc_flags": [ctypes.POINTER(c_void_p), c_size_t, ctypes.c_uint],
     "hades_host_free": [_P],
     "hades_shm_create": [c_char_p, _L, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int64)],
     "hades_shm_open": [c_char_p, _L, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int64)],
@@ -49,6 +51,10 @@ _SIGNATURES = {
     "hades_hot_index_build": [_P, _L, _P, c_size_t, _P],
     "hades_split_compact": [_P, _L, _P, _P, _P, _P, _P, c_size_t, _P],
     "hades_split3_compact": [_P, c_int, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t, _P],
+    "hades_lookup_split": [_P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, c_size_t, _P],
+    "hades_fetch_listed": [_P, _L, _P, _P, _P, _L, _P, _L, c_int, _P],
+    "hades_set_listed": [_P, _P, _L, _P, _P, _P, _L, _L, c_int, _P],
+    "hades_adagrad_update_listed": [_P, _P, _P, _P, _L, _L, _P, _P, _L, c_float, c_float, _P],
     "hades_cached_fetch": [_P, _P, _P, _L, _P, _L, _P, _P, _P, _L, c_int, _P],
     "hades_cached_fetch_loc": [_P, _P, _P, _P, _L, _P, _L, c_int, _P],
     "hades_cached_set": [_P, _P, _P, _P, _L, _P, _L, _P, _L, c_int, _P],

@@ -67,6 +67,11 @@ inline int ilog2_ceil(uint64_t x) {  // smallest b with 2^b >= x
 }
 inline uintptr_t align_of_ptr(const void* p) { return reinterpret_cast<uintptr_t>(p); }
 
+// true if `p` is host memory that kernels reach over the host link (hipHostMalloc / registered)
+bool is_host_memory(const void* p);
+// blocks to launch for a kernel whose table rows cross the host link (see core.hip)
+int64_t host_link_blocks(bool read_and_write);
+
 // Carve aligned sub-buffers out of a caller-provided workspace.
 struct Carver {
   char* base;
@@ -138,11 +143,12 @@ struct HotSet {
   }
 };
 
-// wave64 inclusive prefix sum of a 32-bit value over the lanes of a wavefront
-__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t v) {
+// wave64 inclusive prefix sum over the lanes of a wavefront (lane 63 ends up with the wave total)
+template <typename T>
+__device__ __forceinline__ T wave_inclusive_sum(T v) {
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
-    uint32_t t = __shfl_up(v, d, kWave);
+    T t = __shfl_up(v, d, kWave);
     if (lane_id() >= d) v += t;
   }
   return v;
@@ -169,12 +175,7 @@ __device__ __forceinline__ T block_exclusive_sum(T v, T* smem, T* total) {
   constexpr int kWaves = kBlock / kWave;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  T inc = v;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    T t = __shfl_up(inc, d, kWave);
-    if (lane >= d) inc += t;
-  }
+  const T inc = wave_inclusive_sum<T>(v);
   if (lane == kWave - 1) smem[wave] = inc;
   __syncthreads();
   if (threadIdx.x == 0) {

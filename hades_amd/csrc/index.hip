@@ -104,58 +104,56 @@ __global__ __launch_bounds__(kThreads) void split_masks_kernel(const I* __restri
 }
 
 // ---- stable compaction ------------------------------------------------------
-// A tile is kTile consecutive elements; thread t of the block owns elements [8t, 8t+8) of the
-// tile so that the order of positions inside every class list is ascending.
-constexpr int kItems = 8;
-constexpr int kTile = kThreads * kItems;
-constexpr uint32_t kNone = 3;  // class code of an element that belongs to no list
+// A tile is kTile consecutive elements, taken in kRounds rounds of one element per thread
+// (element tile0 + r*kThreads + t in round r: coalesced).  Ranks inside a wave come from a ballot
+// of the class predicate and a count of the set bits below the lane (mbcnt); the (round, wave)
+// counts of a tile are prefixed in LDS, and the tiles before it are summed from the per-tile
+// counts of the first kernel.  Positions inside every class list are ascending.
+constexpr int kRounds = 8;
+constexpr int kTile = kThreads * kRounds;
+constexpr int kWaves = kThreads / kWave;
+constexpr uint32_t kNone = 3;           // class code of an element that belongs to no list
+constexpr int64_t kSumTilesInKernel = 4096;  // above this many tiles a scan kernel prefixes them
 
-__device__ __forceinline__ uint64_t pack_counts(uint64_t cls8, int valid) {
-  // per-class counts of the (up to 8) class bytes, 21 bits per class
-  uint64_t packed = 0;
-#pragma unroll
-  for (int k = 0; k < kItems; ++k) {
-    const uint32_t c = static_cast<uint32_t>(cls8 >> (8 * k)) & 0xffu;
-    if (k < valid && c < kNone) packed += uint64_t(1) << (21 * c);
-  }
-  return packed;
-}
-
-// classify + per-block counts.  Classifier returns the class code (0..2, or kNone) of element i.
+// classify + per-tile counts.  Classifier returns the class code (0..2, or kNone) of element i;
+// it is called exactly once per element and may write per-element results of its own.
 template <typename Classifier>
 __global__ __launch_bounds__(kThreads) void classify_count_kernel(Classifier cf, int64_t n,
                                                                  uint8_t* __restrict__ cls,
                                                                  uint32_t* __restrict__ blk_cnt,
                                                                  int64_t nblocks) {
-  __shared__ uint64_t smem[kThreads / kWave + 1];
-  const int64_t i0 = static_cast<int64_t>(blockIdx.x) * kTile + threadIdx.x * kItems;
-  uint64_t cls8 = 0;
-  int valid = 0;
+  __shared__ uint32_t s_cnt[kWaves][3];
+  const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  uint32_t cnt[3] = {0, 0, 0};   // wave-uniform
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
+  for (int r = 0; r < kRounds; ++r) {
+    const int64_t i = tile0 + r * kThreads + threadIdx.x;
     uint32_t c = kNone;
-    if (i0 + k < n) {
-      c = cf(i0 + k);
-      valid = k + 1;
+    if (i < n) {
+      c = cf(i);
+      cls[i] = static_cast<uint8_t>(c);
     }
-    cls8 |= static_cast<uint64_t>(c) << (8 * k);
-  }
-  // cls workspace is padded to a whole number of tiles: the full 8-byte store is always in range
-  *reinterpret_cast<uint64_t*>(cls + i0) = cls8;
-  uint64_t total;
-  (void)block_exclusive_sum<uint64_t, kThreads>(pack_counts(cls8, valid), smem, &total);
-  if (threadIdx.x == 0) {
 #pragma unroll
-    for (int c = 0; c < 3; ++c)
-      blk_cnt[c * nblocks + blockIdx.x] = static_cast<uint32_t>(total >> (21 * c)) & 0x1fffffu;
+    for (int k = 0; k < 3; ++k) cnt[k] += __popcll(__ballot(c == static_cast<uint32_t>(k)));
+  }
+  if (lane_id() == 0) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) s_cnt[threadIdx.x / kWave][k] = cnt[k];
+  }
+  __syncthreads();
+  if (threadIdx.x < 3) {
+    uint32_t sum = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sum += s_cnt[w][threadIdx.x];
+    blk_cnt[threadIdx.x * nblocks + blockIdx.x] = sum;
   }
 }
 
-// single block: per-class exclusive prefix over the blocks, and the class totals
+// single block: per-class exclusive prefix over the tiles (only for inputs of more than
+// kSumTilesInKernel tiles; below that every compaction block sums the tiles before it itself)
 __global__ __launch_bounds__(kThreads) void block_prefix_kernel(const uint32_t* __restrict__ blk_cnt,
                                                                int64_t* __restrict__ blk_off,
-                                                               int64_t nblocks, int num_classes,
-                                                               int64_t* __restrict__ totals) {
+                                                               int64_t nblocks, int num_classes) {
   __shared__ int64_t smem[kThreads / kWave + 1];
   for (int c = 0; c < num_classes; ++c) {
     int64_t carry = 0;
@@ -167,7 +165,6 @@ __global__ __launch_bounds__(kThreads) void block_prefix_kernel(const uint32_t* 
       if (b < nblocks) blk_off[c * nblocks + b] = carry + ex;
       carry += total;
     }
-    if (threadIdx.x == 0) totals[c] = carry;
   }
 }
 
@@ -177,50 +174,92 @@ struct CompactOut {
 };
 
 __global__ __launch_bounds__(kThreads) void compact_kernel(const uint8_t* __restrict__ cls,
+                                                          const uint32_t* __restrict__ blk_cnt,
                                                           const int64_t* __restrict__ blk_off,
                                                           int64_t nblocks, int64_t n,
-                                                          int num_classes, CompactOut out) {
-  __shared__ uint64_t smem[kThreads / kWave + 1];
-  const int64_t i0 = static_cast<int64_t>(blockIdx.x) * kTile + threadIdx.x * kItems;
-  const uint64_t cls8 = *reinterpret_cast<const uint64_t*>(cls + i0);
-  const int64_t left = n - i0;
-  const int valid = left >= kItems ? kItems : (left > 0 ? static_cast<int>(left) : 0);
-  uint64_t total;
-  const uint64_t ex = block_exclusive_sum<uint64_t, kThreads>(pack_counts(cls8, valid), smem, &total);
+                                                          int num_classes, CompactOut out,
+                                                          int64_t* __restrict__ totals) {
+  __shared__ int64_t s_wsum[kWaves][3];
+  __shared__ int64_t s_base[3];
+  __shared__ uint32_t s_cnt[kRounds][kWaves][3];   // counts, then exclusive offsets inside the tile
+  const int lane = lane_id();
+  const int wave = threadIdx.x / kWave;
+  const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kTile;
 
-  int64_t run[3];
+  // the tile's class codes first, so that their latency overlaps the sum over earlier tiles
+  uint32_t c[kRounds];
 #pragma unroll
-  for (int c = 0; c < 3; ++c)
-    run[c] = c < num_classes
-                 ? blk_off[c * nblocks + blockIdx.x] + static_cast<int64_t>((ex >> (21 * c)) & 0x1fffffu)
-                 : 0;
+  for (int r = 0; r < kRounds; ++r) {
+    const int64_t i = tile0 + r * kThreads + threadIdx.x;
+    c[r] = i < n ? cls[i] : kNone;
+  }
+
+  // elements of each class in the tiles before this one
+  if (blk_off != nullptr) {
+    if (threadIdx.x < 3)
+      s_base[threadIdx.x] = static_cast<int>(threadIdx.x) < num_classes
+                                ? blk_off[threadIdx.x * nblocks + blockIdx.x] : 0;
+  } else {
+    int64_t part[3] = {0, 0, 0};
+    for (int64_t b = threadIdx.x; b < static_cast<int64_t>(blockIdx.x); b += kThreads) {
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
-    if (k < valid) {
-      const uint32_t c = static_cast<uint32_t>(cls8 >> (8 * k)) & 0xffu;
+      for (int k = 0; k < 3; ++k)
+        if (k < num_classes) part[k] += blk_cnt[k * nblocks + b];
+    }
 #pragma unroll
-      for (int cc = 0; cc < 3; ++cc) {
-        if (cc < num_classes && c == cc) {
-          if (out.pos[cc]) out.pos[cc][run[cc]] = i0 + k;
-          ++run[cc];
-        }
-      }
+    for (int k = 0; k < 3; ++k) {
+      const int64_t w = wave_inclusive_sum<int64_t>(part[k]);
+      if (lane == kWave - 1) s_wsum[wave][k] = w;
+    }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+      int64_t sum = 0;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) sum += s_wsum[w][threadIdx.x];
+      s_base[threadIdx.x] = sum;
     }
   }
+
 #pragma unroll
-  for (int cc = 0; cc < 3; ++cc) {
-    uint8_t* m = out.mask[cc];
-    if (m == nullptr) continue;
-    uint64_t bits = 0;
+  for (int r = 0; r < kRounds; ++r) {
 #pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-      const uint32_t c = static_cast<uint32_t>(cls8 >> (8 * k)) & 0xffu;
-      bits |= static_cast<uint64_t>(c == cc ? 1u : 0u) << (8 * k);
+    for (int k = 0; k < 3; ++k) {
+      const uint32_t cnt = __popcll(__ballot(c[r] == static_cast<uint32_t>(k)));
+      if (lane == 0) s_cnt[r][wave][k] = cnt;
     }
-    if (valid == kItems && (reinterpret_cast<uintptr_t>(m + i0) & 7u) == 0) {
-      *reinterpret_cast<uint64_t*>(m + i0) = bits;
-    } else {
-      for (int k = 0; k < valid; ++k) m[i0 + k] = static_cast<uint8_t>(bits >> (8 * k)) & 1u;
+  }
+  __syncthreads();
+  if (threadIdx.x < 3) {
+    uint32_t run = 0;
+    for (int r = 0; r < kRounds; ++r) {
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const uint32_t t = s_cnt[r][w][threadIdx.x];
+        s_cnt[r][w][threadIdx.x] = run;
+        run += t;
+      }
+    }
+    if (blockIdx.x == gridDim.x - 1 && static_cast<int>(threadIdx.x) < num_classes)
+      totals[threadIdx.x] = s_base[threadIdx.x] + run;
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const int64_t i = tile0 + r * kThreads + threadIdx.x;
+    const uint32_t cc = c[r];
+    uint64_t mine = 0;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const uint64_t bal = __ballot(cc == static_cast<uint32_t>(k));
+      if (cc == static_cast<uint32_t>(k)) mine = bal;
+    }
+    if (i < n) {
+      if (static_cast<int>(cc) < num_classes && out.pos[cc] != nullptr)
+        out.pos[cc][s_base[cc] + s_cnt[r][wave][cc] + ballot_rank(mine)] = i;
+#pragma unroll
+      for (int k = 0; k < 3; ++k)
+        if (out.mask[k] != nullptr) out.mask[k][i] = cc == static_cast<uint32_t>(k) ? 1 : 0;
     }
   }
 }
@@ -236,6 +275,20 @@ struct ClassifyTable {
   __device__ __forceinline__ uint32_t operator()(int64_t i) const {
     const int8_t v = table[static_cast<int64_t>(ids[i])];
     return (v >= 0 && v <= 2) ? static_cast<uint32_t>(v) : kNone;
+  }
+};
+
+// lookup fused into the classification: the slot of every query is written on the way
+struct ClassifyLookup {
+  const int64_t* q;
+  HotSet hs;
+  int64_t* loc;
+  const int64_t* num_live;   // optional: only the first num_live[0] queries count
+  __device__ __forceinline__ uint32_t operator()(int64_t i) const {
+    if (num_live != nullptr && i >= num_live[0]) return kNone;
+    const int64_t l = hs.slot(q[i]);
+    loc[i] = l;
+    return l >= 0 ? 0u : 1u;
   }
 };
 
@@ -256,9 +309,9 @@ CompactWs carve_compact(void* ws, int64_t n) {
   const int64_t nblocks = ceil_div(n > 0 ? n : 1, kTile);
   Carver c(ws);
   CompactWs w;
-  w.cls = c.take<uint8_t>(nblocks * kTile);
+  w.cls = c.take<uint8_t>(n > 0 ? n : 1);
   w.blk_cnt = c.take<uint32_t>(3 * nblocks);
-  w.blk_off = c.take<int64_t>(3 * nblocks);
+  w.blk_off = c.take<int64_t>(nblocks > kSumTilesInKernel ? 3 * nblocks : 1);
   w.bytes = c.total();
   return w;
 }
@@ -277,13 +330,14 @@ int run_compact(const Classifier& cf, int64_t n, int num_classes, const CompactO
   HADES_REQUIRE(nblocks < (int64_t(1) << 31), "n too large");
   HADES_LAUNCH((classify_count_kernel<Classifier>), dim3((unsigned)nblocks), dim3(kThreads), 0,
                      st, cf, n, w.cls, w.blk_cnt, nblocks);
-  HADES_LAUNCH_CHECK();
-  HADES_LAUNCH(block_prefix_kernel, dim3(1), dim3(kThreads), 0, st, w.blk_cnt, w.blk_off,
-                     nblocks, num_classes, counts);
-  HADES_LAUNCH_CHECK();
-  HADES_LAUNCH(compact_kernel, dim3((unsigned)nblocks), dim3(kThreads), 0, st, w.cls,
-                     w.blk_off, nblocks, n, num_classes, out);
-  HADES_LAUNCH_CHECK();
+  const int64_t* blk_off = nullptr;
+  if (nblocks > kSumTilesInKernel) {
+    HADES_LAUNCH(block_prefix_kernel, dim3(1), dim3(kThreads), 0, st, w.blk_cnt, w.blk_off,
+                       nblocks, num_classes);
+    blk_off = w.blk_off;
+  }
+  HADES_LAUNCH(compact_kernel, dim3((unsigned)nblocks), dim3(kThreads), 0, st, w.cls, w.blk_cnt,
+                     blk_off, nblocks, n, num_classes, out, counts);
   return HADES_OK;
 }
 
@@ -445,6 +499,21 @@ int hades_split_compact(const int64_t* loc, int64_t n, uint8_t* hot_mask, int64_
   HADES_REQUIRE(n == 0 || loc, "null pointer argument");
   CompactOut out{{hot_mask, nullptr, nullptr}, {hot_pos, cold_pos, nullptr}};
   return run_compact(ClassifyLoc{loc}, n, 2, out, counts, workspace, workspace_bytes,
+                     static_cast<hipStream_t>(stream));
+}
+
+int hades_lookup_split(const int64_t* q, const int64_t* num_live, int64_t n,
+                       const int64_t* sorted_hot, int64_t num_hot,
+                       const void* hot_index, int64_t* loc, uint8_t* hot_mask, int64_t* hot_pos,
+                       int64_t* cold_pos, int64_t* counts, void* workspace, size_t workspace_bytes,
+                       void* stream) {
+  HADES_REQUIRE(n >= 0 && num_hot >= 0, "n and num_hot must be >= 0");
+  HADES_REQUIRE(n == 0 || (q && loc), "null pointer argument");
+  HADES_REQUIRE(num_hot == 0 || sorted_hot, "sorted_hot is null but num_hot > 0");
+  CompactOut out{{hot_mask, nullptr, nullptr}, {hot_pos, cold_pos, nullptr}};
+  ClassifyLookup cf{q, HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}, loc,
+                    num_live};
+  return run_compact(cf, n, 2, out, counts, workspace, workspace_bytes,
                      static_cast<hipStream_t>(stream));
 }
 

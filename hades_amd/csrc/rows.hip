@@ -151,6 +151,96 @@ __global__ __launch_bounds__(kThreads) void row_move_kernel(Addr addr, int64_t n
   }
 }
 
+// ---- the listed mover ---------------------------------------------------------
+// Rows named by a position list whose length lives in device memory (the two halves of a hot/cold
+// split): for j < count[0], p = list[j] is a batch position and index[p] a table row.
+//   GATHER : batch[p, :] = table[index[p], :]        SCATTER: table[index[p], :] = batch[p, :]
+// Blocks stride over the list in steps of kRowsPerBlock rows, so the grid need not match the count.
+struct ListedArgs {
+  const char* table_ro;        // GATHER source
+  char* table_rw;              // SCATTER destination
+  int64_t table_stride_bytes;  // bytes between consecutive table rows (>= row bytes)
+  const int64_t* index;        // [positions]
+  const int64_t* list;         // [max_count]
+  const int64_t* count;        // [1]
+  int64_t max_count;
+  const char* batch_ro;        // SCATTER source
+  char* batch_rw;              // GATHER destination
+  int64_t row_bytes;
+};
+
+template <typename Vec, bool GATHER>
+__global__ __launch_bounds__(kThreads) void row_move_listed_kernel(ListedArgs a, int chunks_per_row,
+                                                                  int shift) {
+  __shared__ const char* s_src[kRowsPerBlock];
+  __shared__ char* s_dst[kRowsPerBlock];
+  int64_t cnt = a.count[0];
+  cnt = cnt < a.max_count ? cnt : a.max_count;
+  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock; row0 < cnt;
+       row0 += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
+    const int64_t left = cnt - row0;
+    const int rows_here = left < kRowsPerBlock ? static_cast<int>(left) : kRowsPerBlock;
+    for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+      const int64_t p = a.list[row0 + r];
+      const int64_t t = a.index[p] * a.table_stride_bytes;
+      if (GATHER) {
+        s_src[r] = a.table_ro + t;
+        s_dst[r] = a.batch_rw + p * a.row_bytes;
+      } else {
+        s_src[r] = a.batch_ro + p * a.row_bytes;
+        s_dst[r] = a.table_rw + t;
+      }
+    }
+    __syncthreads();
+    const int total = rows_here * chunks_per_row;
+    for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
+      Vec v[kUnroll];
+      Vec* d[kUnroll];
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        const int c = base + k * kThreads;
+        if (c < total) {
+          const int r = shift >= 0 ? (c >> shift) : (c / chunks_per_row);
+          const int ch = c - r * chunks_per_row;
+          v[k] = reinterpret_cast<const Vec*>(s_src[r])[ch];
+          d[k] = reinterpret_cast<Vec*>(s_dst[r]) + ch;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        const int c = base + k * kThreads;
+        if (c < total) *d[k] = v[k];
+      }
+    }
+    __syncthreads();   // the row pointers are rewritten by the next round
+  }
+}
+
+constexpr int64_t kMaxListedBlocks = 16384;
+
+template <bool GATHER>
+int launch_listed(const ListedArgs& a, int vec, hipStream_t stream) {
+  const int64_t cpr64 = a.row_bytes / vec;
+  HADES_REQUIRE(cpr64 * kRowsPerBlock < (int64_t(1) << 30), "row of %lld bytes is too large",
+                (long long)a.row_bytes);
+  const int cpr = static_cast<int>(cpr64);
+  const int shift = is_pow2(cpr) ? ilog2_ceil(cpr) : -1;
+  int64_t blocks = ceil_div(a.max_count, kRowsPerBlock);
+  if (blocks > kMaxListedBlocks) blocks = kMaxListedBlocks;
+  // rows that cross the host link: a narrow grid that strides over the list
+  const void* table = GATHER ? static_cast<const void*>(a.table_ro) : a.table_rw;
+  if (is_host_memory(table) && blocks > host_link_blocks(false)) blocks = host_link_blocks(false);
+  dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+  if (vec == 16) {
+    HADES_LAUNCH((row_move_listed_kernel<u32x4, GATHER>), grid, block, 0, stream, a, cpr, shift);
+  } else if (vec == 8) {
+    HADES_LAUNCH((row_move_listed_kernel<u32x2, GATHER>), grid, block, 0, stream, a, cpr, shift);
+  } else {
+    HADES_LAUNCH((row_move_listed_kernel<uint32_t, GATHER>), grid, block, 0, stream, a, cpr, shift);
+  }
+  return HADES_OK;
+}
+
 int pick_vec(int64_t row_bytes, std::initializer_list<const void*> bases) {
   int v = 16;
   while (v > 4) {
@@ -319,6 +409,40 @@ int hades_cached_fetch_loc(const void* cold_src, const void* hot_src, const int6
   const int vec = pick_vec(row_bytes, {cold_src, hot_src, dst});
   AddrFetchLoc a{(const char*)cold_src, (const char*)hot_src, q, loc, (char*)dst, row_bytes};
   return launch_mover(a, n, row_bytes, vec, static_cast<hipStream_t>(stream));
+}
+
+int hades_fetch_listed(const void* src, int64_t src_stride, const int64_t* src_index,
+                       const int64_t* list, const int64_t* count, int64_t max_count, void* dst,
+                       int64_t dim, int dtype, void* stream) {
+  HADES_REQUIRE(max_count >= 0 && dim >= 1, "max_count must be >= 0 and dim >= 1");
+  HADES_REQUIRE(elem_size(dtype) != 0, "Type can only be float or double (code %d)", dtype);
+  HADES_REQUIRE(src_stride == 0 || src_stride >= dim, "src_stride must be 0 or >= dim");
+  if (max_count == 0) return HADES_OK;
+  HADES_REQUIRE(src && src_index && list && count && dst, "null pointer argument");
+  const int64_t row_bytes = dim * elem_size(dtype);
+  const int64_t stride_bytes = (src_stride ? src_stride : dim) * elem_size(dtype);
+  int vec = pick_vec(row_bytes, {src, dst});
+  while (vec > 4 && stride_bytes % vec != 0) vec >>= 1;
+  ListedArgs a{(const char*)src, nullptr, stride_bytes, src_index, list, count, max_count,
+               nullptr, (char*)dst, row_bytes};
+  return launch_listed<true>(a, vec, static_cast<hipStream_t>(stream));
+}
+
+int hades_set_listed(const void* src, void* dst, int64_t dst_stride, const int64_t* dst_index,
+                     const int64_t* list, const int64_t* count, int64_t max_count, int64_t dim,
+                     int dtype, void* stream) {
+  HADES_REQUIRE(max_count >= 0 && dim >= 1, "max_count must be >= 0 and dim >= 1");
+  HADES_REQUIRE(elem_size(dtype) != 0, "Type can only be float or double (code %d)", dtype);
+  HADES_REQUIRE(dst_stride == 0 || dst_stride >= dim, "dst_stride must be 0 or >= dim");
+  if (max_count == 0) return HADES_OK;
+  HADES_REQUIRE(src && dst_index && list && count && dst, "null pointer argument");
+  const int64_t row_bytes = dim * elem_size(dtype);
+  const int64_t stride_bytes = (dst_stride ? dst_stride : dim) * elem_size(dtype);
+  int vec = pick_vec(row_bytes, {src, dst});
+  while (vec > 4 && stride_bytes % vec != 0) vec >>= 1;
+  ListedArgs a{nullptr, (char*)dst, stride_bytes, dst_index, list, count, max_count,
+               (const char*)src, nullptr, row_bytes};
+  return launch_listed<false>(a, vec, static_cast<hipStream_t>(stream));
 }
 
 int hades_cached_set(const void* src, void* cold_dst, void* hot_dst, const int64_t* q, int64_t n,

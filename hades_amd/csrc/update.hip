@@ -124,6 +124,75 @@ __global__ __launch_bounds__(kThreads) void adagrad_kernel(AdagradArgs a) {
   }
 }
 
+// Adagrad over the rows named by a position list whose length lives in device memory (one half of
+// a hot/cold split): for j < count[0], p = list[j]; the gradient is row p of grad, the weight and
+// state rows are row row_index[p] of w and s, whose rows lie `stride` floats apart (w and s of a
+// row may sit next to each other in one table: s = w + dim, stride = 2 * dim).
+struct AdagradListedArgs {
+  const int64_t* row_index;
+  const float* grad;
+  const int64_t* list;
+  const int64_t* count;
+  int64_t max_count;
+  int64_t dim;
+  float* w;
+  float* s;
+  int64_t stride;
+  float lr, eps;
+};
+
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedArgs a) {
+  typedef typename Vf<VEC>::type V;
+  __shared__ int64_t s_row[kRows];    // element offset of the row in w and s
+  __shared__ int64_t s_grad[kRows];   // element offset of the row in grad
+  int64_t cnt = a.count[0];
+  cnt = cnt < a.max_count ? cnt : a.max_count;
+  const int cpr = static_cast<int>(a.dim / VEC);
+  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRows; row0 < cnt;
+       row0 += static_cast<int64_t>(gridDim.x) * kRows) {
+    const int64_t left = cnt - row0;
+    const int rows_here = left < kRows ? static_cast<int>(left) : kRows;
+    for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+      const int64_t p = a.list[row0 + r];
+      s_row[r] = a.row_index[p] * a.stride;
+      s_grad[r] = p * a.dim;
+    }
+    __syncthreads();
+    const int total = rows_here * cpr;
+    for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
+      V g[kUnroll], s[kUnroll], w[kUnroll];
+      V* sp[kUnroll];
+      V* wp[kUnroll];
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        const int c = base + k * kThreads;
+        if (c < total) {
+          const int r = c / cpr;
+          const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
+          sp[k] = reinterpret_cast<V*>(a.s + s_row[r] + col);
+          wp[k] = reinterpret_cast<V*>(a.w + s_row[r] + col);
+          g[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(a.grad + s_grad[r] + col));
+          s[k] = *sp[k];
+          w[k] = *wp[k];
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        const int c = base + k * kThreads;
+        if (c < total) {
+          const V s1 = s[k] + g[k] * g[k];
+          const V std_ = vsqrt(s1) + a.eps;
+          const V w1 = w[k] - vdiv(a.lr * g[k], std_);
+          *sp[k] = s1;
+          *wp[k] = w1;
+        }
+      }
+    }
+    __syncthreads();   // the row offsets are rewritten by the next round
+  }
+}
+
 template <int VEC>
 __global__ __launch_bounds__(kThreads) void adam_kernel(AdamArgs a) {
   typedef typename Vf<VEC>::type V;
@@ -229,6 +298,30 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
   else
     HADES_LAUNCH_TIMED(HADES_KERNEL_ADAGRAD, st, (adagrad_kernel<1>), grid, block, 0, st, a);
   HADES_LAUNCH_CHECK();
+  return HADES_OK;
+}
+
+int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,
+                                const int64_t* count, int64_t max_count, int64_t dim, float* w,
+                                float* s, int64_t stride, float lr, float eps, void* stream) {
+  HADES_REQUIRE(max_count >= 0 && dim >= 1, "max_count must be >= 0 and dim >= 1");
+  HADES_REQUIRE(stride == 0 || stride >= dim, "stride must be 0 or >= dim");
+  HADES_REQUIRE(dim * kRows < (int64_t(1) << 30), "dim too large");
+  if (max_count == 0) return HADES_OK;
+  HADES_REQUIRE(row_index && grad && list && count && w && s, "null pointer argument");
+  if (stride == 0) stride = dim;
+  AdagradListedArgs a{row_index, grad, list, count, max_count, dim, w, s, stride, lr, eps};
+  int64_t blocks = ceil_div(max_count, kRows);
+  if (blocks > 16384) blocks = 16384;
+  // rows that cross the host link: a narrow grid that strides over the list
+  if ((is_host_memory(w) || is_host_memory(s)) && blocks > host_link_blocks(true))
+    blocks = host_link_blocks(true);
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dim % 4 == 0 && stride % 4 == 0 && aligned16({grad, w, s}))
+    HADES_LAUNCH((adagrad_listed_kernel<4>), grid, block, 0, st, a);
+  else
+    HADES_LAUNCH((adagrad_listed_kernel<1>), grid, block, 0, st, a);
   return HADES_OK;
 }
 

@@ -4,9 +4,12 @@
 (src/pybind.cc:17-36 over SACacheIndex, src/cache/cache.h) and `LocalCache` those of its Python
 wrapper (python/EmbCache/cache.py:6-31).  The reference holds the structure in host shared memory,
 takes and returns CPU tensors for add / lookup / reset / getall and device tensors only for
-cudalookup; here the structure lives in HBM and every method takes and returns device tensors, so
-that the lookup of a batch needs no round trip through the host
-(python/EmbCache/dist_emb.py:183-185).
+cudalookup; here the structure lives in HBM and the fast path is device tensors in, device
+tensors out, so that the lookup of a batch needs no round trip through the host
+(python/EmbCache/dist_emb.py:183-185).  For unmodified reference code, add / lookup / reset /
+cudalookup also accept a CPU int64 tensor: it is copied to the device and the locs come back as a
+CPU tensor (the reference's `lookup(ids.cpu()).cuda()` keeps working, at the price of the copies
+the reference pays too).  getall returns device tensors.
 
 Batches are handled in input order line by line: the result of the reference with one OpenMP
 thread.  Ids must be int64; negative ids are never cached (loc -1).
@@ -54,7 +57,19 @@ class IndexCache:
         return int(num_valid.item())
 
     # ---- operations ----
+    def _in(self, ids):
+        """(ids on the device, whether the caller's tensor lives on the host)"""
+        _check(ids.dtype == torch.int64, "ids must be int64")
+        if ids.is_cuda:
+            return ids, False
+        return ids.contiguous().to(self.device), True
+
     def _ordered(self, entry, ids):
+        ids, from_host = self._in(ids)
+        locs = self._ordered_dev(entry, ids)
+        return locs.cpu() if from_host else locs
+
+    def _ordered_dev(self, entry, ids):
         _i64(ids, "ids")
         locs = torch.empty_like(ids)
         n = ids.numel()
@@ -75,14 +90,16 @@ class IndexCache:
 
     def cudalookup(self, ids):
         """loc or -1 per id; the cache is left as it is (src/cache/lookup.cu:15-45)."""
+        ids, from_host = self._in(ids)
         _i64(ids, "ids")
         locs = torch.empty_like(ids)
         _lib.call("hades_sacache_lookup", _ptr(self.line_ids), self.lines, _ptr(ids), ids.numel(),
                   _ptr(locs), _stream())
-        return locs
+        return locs.cpu() if from_host else locs
 
     def reset(self, ids):
         """Frees the entries of the ids that are present (cache.h:109-121)."""
+        ids, _ = self._in(ids)
         _i64(ids, "ids")
         _lib.call("hades_sacache_reset", _ptr(self.line_ids), _ptr(self.line_age), self.lines,
                   _ptr(ids), ids.numel(), _stream())

@@ -162,6 +162,78 @@ def split(loc, workspace=None):
     return hot_mask, hot_pos[:nh], cold_pos[:nc]
 
 
+def lookup_split(ids, sorted_hot, num_live=None, workspace=None, out=None):
+    """Lookup and hot/cold split in one call, no host synchronisation.
+
+    Returns (loc int64[n], hot_pos int64[n], cold_pos int64[n], counts int64[2]): the slot of every
+    id in the hot set (or -1), the ascending positions of the hot and of the cold ids (the first
+    counts[0] / counts[1] entries are live) and the two counts.  `num_live` (int64[1] on the device)
+    limits the batch to its first num_live[0] entries, e.g. the padded output of combine_padded.
+    `out` may bring the four tensors."""
+    _i64(ids, "ids")
+    hp, hn, hi = _hot_args(sorted_hot)
+    n, dev = ids.numel(), ids.device
+    if out is None:
+        out = (torch.empty(n, dtype=torch.int64, device=dev), torch.empty(n, dtype=torch.int64, device=dev),
+               torch.empty(n, dtype=torch.int64, device=dev), torch.empty(2, dtype=torch.int64, device=dev))
+    loc, hot_pos, cold_pos, counts = out
+    _check(loc.numel() >= n and hot_pos.numel() >= n and cold_pos.numel() >= n and counts.numel() >= 2,
+           "lookup_split outputs too small")
+    nbytes = _lib.query("hades_split_compact_workspace_bytes", n)
+    ws = (workspace or _ws(dev, "split")).get(nbytes)
+    _lib.call("hades_lookup_split", _ptr(ids), _opt(num_live), n, hp, hn, hi, _ptr(loc), _NULL, _ptr(hot_pos),
+              _ptr(cold_pos), _ptr(counts), _ptr(ws), ws.numel(), _stream())
+    return loc, hot_pos, cold_pos, counts
+
+
+def _stride_of(table, dim):
+    """Row stride in elements of a 2-D (or 1-D) table whose rows are contiguous."""
+    if table.dim() == 1:
+        _check(table.is_contiguous(), "1-D tables must be contiguous")
+        return 1
+    _check(table.stride(1) == 1 and table.stride(0) >= dim, "table rows must be contiguous")
+    return table.stride(0)
+
+
+def fetch_listed(table, index, pos_list, count, out):
+    """out[p] = table[index[p]] for the first count[0] positions p of pos_list (device-side count:
+    no host synchronisation).  `table` may be pinned host memory and may be a row-strided view."""
+    _i64(index, "index"); _i64(pos_list, "pos_list"); _i64(count, "count")
+    _dev_or_pinned(table, "table", contiguous=False); _dev(out, "out")
+    dim = 1 if out.dim() == 1 else out.size(1)
+    _check(table.dtype == out.dtype, "table and out differ in dtype")
+    _lib.call("hades_fetch_listed", _ptr(table), _stride_of(table, dim), _ptr(index), _ptr(pos_list),
+              _ptr(count), pos_list.numel(), _ptr(out), dim, _dcode(out), _stream())
+    return out
+
+
+def set_listed(src, table, index, pos_list, count):
+    """table[index[p]] = src[p] for the first count[0] positions p of pos_list."""
+    _i64(index, "index"); _i64(pos_list, "pos_list"); _i64(count, "count")
+    _dev_or_pinned(table, "table", contiguous=False); _dev(src, "src")
+    dim = 1 if src.dim() == 1 else src.size(1)
+    _check(table.dtype == src.dtype, "table and src differ in dtype")
+    _lib.call("hades_set_listed", _ptr(src), _ptr(table), _stride_of(table, dim), _ptr(index),
+              _ptr(pos_list), _ptr(count), pos_list.numel(), dim, _dcode(src), _stream())
+
+
+def adagrad_update_listed_(row_index, grad, pos_list, count, w, s, lr, eps):
+    """Sparse Adagrad over the rows named by the first count[0] positions p of pos_list:
+    g = grad[p]; r = row_index[p]; s[r] += g*g; w[r] -= lr * g / (sqrt(s[r]) + eps).  w and s are
+    one table pair (device or pinned host) with the same row stride; they may be the two halves of
+    one interleaved table."""
+    _i64(row_index, "row_index"); _i64(pos_list, "pos_list"); _i64(count, "count"); _dev(grad, "grad")
+    _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
+    dim = grad.size(1)
+    for name, t in (("w", w), ("s", s)):
+        _dev_or_pinned(t, name, contiguous=False)
+        _check(t.dtype == torch.float32 and t.dim() == 2 and t.size(1) == dim, "%s: wrong dtype/width" % name)
+    stride = _stride_of(w, dim)
+    _check(_stride_of(s, dim) == stride, "w and s must have the same row stride")
+    _lib.call("hades_adagrad_update_listed", _ptr(row_index), _ptr(grad), _ptr(pos_list), _ptr(count),
+              pos_list.numel(), dim, _ptr(w), _ptr(s), stride, float(lr), float(eps), _stream())
+
+
 def split3_padded(ids, class_table, workspace=None):
     """Three-way split by the int8 class table (0 local, 1 remote-hot, 2 remote-cold) with the
     compacted position lists; no host synchronisation.  Returns (masks[3], pos[3], counts[3])."""

@@ -76,9 +76,13 @@ class _SparseRowOptimizer:
         gather kernel instead of being indexed on the CPU."""
         if cold.is_cuda:
             return cold[self.hot_ids].contiguous()
-        out = torch.empty((self.hot_ids.numel(),) + tuple(cold.shape[1:]), dtype=cold.dtype,
-                          device=self.device)
-        EmbCacheLib.cudaFetch2(cold, self.hot_ids, out)
+        h = self.hot_ids.numel()
+        out = torch.empty((h,) + tuple(cold.shape[1:]), dtype=cold.dtype, device=self.device)
+        if cold.is_contiguous():
+            EmbCacheLib.cudaFetch2(cold, self.hot_ids, out)
+        elif h:                                   # row-strided host table
+            ops.fetch_listed(cold, self.hot_ids, torch.arange(h, device=self.device),
+                             torch.tensor([h], dtype=torch.int64, device=self.device), out)
         return out
 
     def _new_state_like(self, cold, shape=None):
@@ -122,6 +126,113 @@ class _SparseRowOptimizer:
             plan.ready.record(stream)
         return plan
 
+    # ---- the split schedule: hot rows and cold rows on separate kernels and streams ----------
+    # The reference's forward path splits a batch by class first and then gathers per class
+    # (python/EmbCache/dist_emb.py:174-211).  Here: one lookup + stable partition, then the hot
+    # positions go through kernels that only touch HBM while the cold positions go through
+    # kernels that only touch the host table, on a second stream of the same priority, so the
+    # host-link time and the HBM time overlap instead of adding up.
+    def _split_state(self):
+        if getattr(self, "_cold_stream", None) is None:
+            self._cold_stream = torch.cuda.Stream(device=self.device)
+            self._split_bufs = {}
+            self._split_ws = ops.Workspace(self.device)
+            self._cold_done = None
+        return self._cold_stream
+
+    def _split_out(self, key, n):
+        bufs = self._split_bufs.get(key)
+        if bufs is None or bufs[0].numel() < n:
+            dev = self.device
+            bufs = (torch.empty(n, dtype=torch.int64, device=dev), torch.empty(n, dtype=torch.int64, device=dev),
+                    torch.empty(n, dtype=torch.int64, device=dev), torch.empty(2, dtype=torch.int64, device=dev))
+            self._split_bufs[key] = bufs
+        return bufs
+
+    def join(self):
+        """Makes torch's current stream wait for everything queued on the cold stream."""
+        if getattr(self, "_cold_done", None) is not None:
+            torch.cuda.current_stream().wait_event(self._cold_done)
+            self._cold_done = None
+
+    @staticmethod
+    def _timed(timing, name, stream, fn):
+        """Runs fn(); with timing = {name: (start, stop)} (torch events, enable_timing=True) the
+        pair is recorded on `stream` right before and after it."""
+        pair = timing.get(name) if timing else None
+        if pair:
+            pair[0].record(stream)
+        fn()
+        if pair:
+            pair[1].record(stream)
+
+    def fetch_split(self, ids, out=None, join=True, timing=None):
+        """cached_fetch as lookup -> stable hot/cold partition -> one gather per class: the hot
+        class from the HBM copy on the current stream, the cold class from the cold table on the
+        cold stream.  With join=False the caller calls join() before anything reads `out` or
+        writes the tables on the current stream.  `timing` may map "hot_fetch" / "cold_fetch" to
+        event pairs that are recorded around the two gather kernels on their streams."""
+        cold = self._split_state()
+        cur = torch.cuda.current_stream()
+        n = ids.numel()
+        if out is None:
+            out = torch.empty((n, self.dim), dtype=self.hot_w.dtype, device=self.device)
+        loc, hot_pos, cold_pos, counts = ops.lookup_split(
+            ids, self.hot_set, workspace=self._split_ws, out=self._split_out("fetch", n))
+        hot_pos, cold_pos = hot_pos[:n], cold_pos[:n]
+        split_done = torch.cuda.Event()
+        split_done.record(cur)
+        cold.wait_event(split_done)
+        with torch.cuda.stream(cold):
+            self._timed(timing, "cold_fetch", cold,
+                        lambda: ops.fetch_listed(self.cold_w, ids, cold_pos, counts[1:2], out))
+            self._cold_done = torch.cuda.Event()
+            self._cold_done.record(cold)
+        if self.hot_ids.numel():
+            self._timed(timing, "hot_fetch", cur,
+                        lambda: ops.fetch_listed(self.hot_w, loc, hot_pos, counts[0:1], out))
+        if join:
+            self.join()
+        return out
+
+    def _update_class(self, index, grad, pos, count, hot):
+        raise NotImplementedError
+
+    def update_split(self, uids, grad, num_unique=None, join=True, timing=None):
+        """The row update over a combined batch as lookup -> partition -> one update kernel per
+        class, hot on the current stream and cold on the cold stream ("hot_update" /
+        "cold_update" in `timing`)."""
+        cold = self._split_state()
+        cur = torch.cuda.current_stream()
+        n = uids.numel()
+        loc, hot_pos, cold_pos, counts = ops.lookup_split(
+            uids, self.hot_set, num_live=num_unique, workspace=self._split_ws,
+            out=self._split_out("update", n))
+        hot_pos, cold_pos = hot_pos[:n], cold_pos[:n]
+        split_done = torch.cuda.Event()
+        split_done.record(cur)
+        cold.wait_event(split_done)          # the cold stream also still orders after its own fetch
+        with torch.cuda.stream(cold):
+            self._timed(timing, "cold_update", cold,
+                        lambda: self._update_class(uids, grad, cold_pos, counts[1:2], hot=False))
+            self._cold_done = torch.cuda.Event()
+            self._cold_done.record(cold)
+        if self.hot_ids.numel():
+            self._timed(timing, "hot_update", cur,
+                        lambda: self._update_class(loc, grad, hot_pos, counts[0:1], hot=True))
+        if join:
+            self.join()
+
+    def step_split(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None):
+        """step() on the split schedule."""
+        if plan is None:
+            plan = ops.combine_plan(idx, self.dim, id_bound=self.num_rows, workspace=self._ws)
+        else:
+            torch.cuda.current_stream().wait_event(plan.ready)
+        uids, sums, cnts, nu = ops.combine_apply(plan, grad, mode, out=out)
+        self.update_split(uids, sums, nu)
+        return uids, sums, cnts, nu
+
     def step(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None):
         """combine the per-occurrence gradients, then update every distinct row once.
         No host synchronisation.  `plan` = what prepare(idx) returned, if it was called."""
@@ -139,11 +250,25 @@ class SparseAdagrad(_SparseRowOptimizer):
     (torch.optim.Adagrad with lr_decay = weight_decay = initial_accumulator_value = 0)."""
 
     def __init__(self, weight_cold, hot_ids, lr=0.01, eps=1e-10, device="cuda",
-                 state_on_device=False):
+                 state_on_device=False, cold_state=None):
+        """`cold_state` brings the cold Adagrad state instead of a new zero tensor; together with
+        a row-strided `weight_cold` it allows one host table [N, 2, D] that holds the weight row
+        and the state row of an id next to each other (weight_cold = t[:, 0], cold_state =
+        t[:, 1]): one burst per cold row and direction over the host link.  Row-strided cold
+        tables are served by the split schedule (fetch_split / update_split / step_split) only."""
         super().__init__(weight_cold, hot_ids, lr, device, state_on_device)
         self.eps = eps
-        self.cold_s = self._new_state_like(weight_cold)
+        if cold_state is not None:
+            if tuple(cold_state.shape) != tuple(weight_cold.shape) or cold_state.dtype != torch.float32:
+                raise RuntimeError("cold_state must be float32 of the weight table's shape")
+            self.cold_s = cold_state
+        else:
+            self.cold_s = self._new_state_like(weight_cold)
         self.hot_s = torch.zeros_like(self.hot_w)
+
+    def _update_class(self, index, grad, pos, count, hot):
+        w, s = (self.hot_w, self.hot_s) if hot else (self.cold_w, self.cold_s)
+        ops.adagrad_update_listed_(index, grad, pos, count, w, s, self.lr, self.eps)
 
     def update(self, uids, grad, num_unique=None):
         ops.adagrad_update_(uids, grad, self.hot_w, self.hot_s, self.cold_w, self.cold_s,

@@ -82,6 +82,12 @@ int hades_unpin(void* host_ptr);
  * existing memory is not possible.  The returned pointer is valid on host and device. */
 int hades_host_alloc(void** out_ptr, size_t bytes);
 int hades_host_free(void* ptr);
+/* The same with flags.  HADES_HOST_NONCOHERENT asks for coarse-grained host memory: the GPU may keep
+ * lines of it in its L2 and writes them back at kernel boundaries, so the host sees a kernel's
+ * writes only after the stream has been synchronised (which is when the reference's trainers read
+ * their tables anyway); in exchange reads and writes cross the host link in whole cache lines. */
+#define HADES_HOST_NONCOHERENT 1u
+int hades_host_alloc_flags(void** out_ptr, size_t bytes, unsigned flags);
 
 /* create_shared_mem / open_shared_mem / release_shared_mem (src/shm/shared_memory.h:14-58):
  * a POSIX shared-memory segment mapped read-write; pin != 0 also registers the mapping with the
@@ -185,6 +191,20 @@ int hades_split_compact(const int64_t* loc, int64_t n, uint8_t* hot_mask, int64_
                         int64_t* cold_pos, int64_t* counts, void* workspace, size_t workspace_bytes,
                         void* stream);
 
+/* Lookup and hot/cold split in one call: hades_lookup_sorted followed by hades_split_compact, with
+ * the slots written on the way (loc int64[n]).  This is the first step of the split schedule of
+ * the reference's forward path (python/EmbCache/dist_emb.py:174-211: split first, then a gather
+ * per class): the two position lists then drive hades_fetch_listed / hades_adagrad_update_listed
+ * over the hot tables in HBM and over the cold tables on the host, on separate streams.
+ * num_live (int64[1] on the device, may be NULL) limits the batch to its first num_live[0] entries
+ * (the padded output of hades_combine): later entries are in neither list and get no slot.
+ * hot_mask may be NULL.  Workspace as hades_split_compact. */
+int hades_lookup_split(const int64_t* q, const int64_t* num_live, int64_t n,
+                       const int64_t* sorted_hot, int64_t num_hot,
+                       const void* hot_index, int64_t* loc, uint8_t* hot_mask, int64_t* hot_pos,
+                       int64_t* cold_pos, int64_t* counts, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
 /* Three-way form of the same thing from the reference's class table (src/cuda/split.cu:11):
  * masks as hades_split, plus pos[k] = ascending positions of class k (each int64 capacity n) and
  * counts[0..2].  Any of the mask pointers may be NULL. */
@@ -213,6 +233,22 @@ int hades_cached_fetch_loc(const void* cold_src, const void* hot_src, const int6
 int hades_cached_set(const void* src, void* cold_dst, void* hot_dst, const int64_t* q, int64_t n,
                      const int64_t* sorted_hot, int64_t num_hot, const void* hot_index,
                      int64_t dim, int dtype, void* stream);
+
+/* Row gather / scatter over one half of a split (the per-class gathers of
+ * python/EmbCache/dist_emb.py:193-211, CUDAFetch2 / CUDASet semantics of src/cuda/uva_fetch.cu:72-105
+ * and src/cuda/uva_set.cu:35-68, driven by a position list whose length stays on the device):
+ *   fetch: for j < min(count[0], max_count): p = list[j];  dst[p, :] = src[src_index[p], :]
+ *   set  : for j < min(count[0], max_count): p = list[j];  dst[dst_index[p], :] = src[p, :]
+ * list int64[max_count] holds batch positions, *_index int64[positions] the table row of every
+ * position (the slot from hades_lookup_split for the hot table, the id itself for the cold table),
+ * count int64[1] on the device.  The table (src of fetch, dst of set) may be pinned host memory and
+ * its rows may lie *_stride elements apart (0 = dim).  A negative count is treated as 0. */
+int hades_fetch_listed(const void* src, int64_t src_stride, const int64_t* src_index,
+                       const int64_t* list, const int64_t* count, int64_t max_count, void* dst,
+                       int64_t dim, int dtype, void* stream);
+int hades_set_listed(const void* src, void* dst, int64_t dst_stride, const int64_t* dst_index,
+                     const int64_t* list, const int64_t* count, int64_t max_count, int64_t dim,
+                     int dtype, void* stream);
 
 /* combine: sort + dedup + segment-sum of duplicate-ID gradient rows; the arithmetic of
  * only_unique_grads (python/EmbCache/sparse_optim.py:132-139), which is also the
@@ -281,6 +317,18 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
                          const int64_t* sorted_hot, int64_t num_hot, const void* hot_index,
                          float* hot_w, float* hot_s, float* cold_w, float* cold_s,
                          float lr, float eps, void* stream);
+
+/* The same Adagrad arithmetic over one half of a split, against one table pair:
+ *   for j < min(count[0], max_count): p = list[j]; r = row_index[p]; g = grad[p, :]
+ *     s[r*stride ..] += g*g;  w[r*stride ..] -= lr * g / (sqrt(s) + eps)
+ * row_index is the slot (hot tables) or the id (cold tables) of every position of the combined
+ * batch, list/count one of the two lists hades_lookup_split made of its distinct ids.  w and s may
+ * be device or pinned host memory; rows lie `stride` floats apart (0 = dim), so the weight and
+ * state row of an id may be stored next to each other (s = w + dim, stride = 2*dim): one burst
+ * over the host link per cold row and direction instead of two. */
+int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,
+                                const int64_t* count, int64_t max_count, int64_t dim, float* w,
+                                float* s, int64_t stride, float lr, float eps, void* stream);
 
 /* SparseAdam row update, same fusion (python/EmbCache/sparse_optim.py:632-657,681):
  *   step += 1; m = b1*m + (1-b1)*g; v = b2*v + (1-b2)*g*g

@@ -229,6 +229,64 @@ def cached_set(src, cold, hot, q, sorted_hot):
 
 
 # ---------------------------------------------------------------------------
+# the split schedule: split first, then one gather / update per class
+# (python/EmbCache/dist_emb.py:174-211: cudaSplit, torch.nonzero per class, one cudaFetch per class
+# into the positions of that class)
+# ---------------------------------------------------------------------------
+def lookup_split(q, sorted_hot, num_live=None):
+    """(loc, hot_pos, cold_pos): slot of every query, ascending positions of each class; entries
+    at and beyond num_live are in neither list and keep loc as computed for the live ones only."""
+    q = np.asarray(q, dtype=np.int64)
+    live = q.size if num_live is None else max(0, min(int(num_live), q.size))
+    loc = lookup_sorted(q[:live], sorted_hot)
+    _, hot_pos, cold_pos = split_compact(loc)
+    return loc, hot_pos, cold_pos
+
+
+def fetch_listed(table, index, pos_list, count, out):
+    """out[p] = table[index[p]] for the first `count` positions of pos_list (cudaFetch with
+    dst_index = the positions of one class, python/EmbCache/dist_emb.py:205-211); in place."""
+    pos = np.asarray(pos_list, dtype=np.int64)[: max(0, int(count))]
+    out[pos] = np.asarray(table)[np.asarray(index, dtype=np.int64)[pos]]
+    return out
+
+
+def set_listed(src, table, index, pos_list, count):
+    """table[index[p]] = src[p] for the first `count` positions of pos_list; in place."""
+    pos = np.asarray(pos_list, dtype=np.int64)[: max(0, int(count))]
+    table[np.asarray(index, dtype=np.int64)[pos]] = np.asarray(src)[pos]
+    return table
+
+
+def fetch_split(cold, hot, q, sorted_hot):
+    """cached_fetch done class by class; must equal cached_fetch."""
+    q = np.asarray(q, dtype=np.int64)
+    loc, hot_pos, cold_pos = lookup_split(q, sorted_hot)
+    out = np.empty((q.size,) + np.asarray(hot).shape[1:], dtype=np.asarray(hot).dtype)
+    fetch_listed(hot, loc, hot_pos, hot_pos.size, out)
+    fetch_listed(cold, q, cold_pos, cold_pos.size, out)
+    return out
+
+
+def adagrad_listed(row_index, grad, pos_list, count, w, s, lr, eps):
+    """adagrad_rows on the rows row_index[p] of (w, s) with gradient grad[p], p over the first
+    `count` positions of pos_list; in place."""
+    pos = np.asarray(pos_list, dtype=np.int64)[: max(0, int(count))]
+    rows = np.asarray(row_index, dtype=np.int64)[pos]
+    w1, s1 = adagrad_rows(w[rows], s[rows], np.asarray(grad)[pos], lr, eps)
+    w[rows] = w1
+    s[rows] = s1
+
+
+def sparse_adagrad_step_split(cold_w, cold_s, hot_w, hot_s, sorted_hot, uids, g, lr, eps,
+                              num_live=None):
+    """sparse_adagrad_step done class by class; must equal sparse_adagrad_step."""
+    loc, hot_pos, cold_pos = lookup_split(uids, sorted_hot, num_live)
+    adagrad_listed(loc, g, hot_pos, hot_pos.size, hot_w, hot_s, lr, eps)
+    adagrad_listed(uids, g, cold_pos, cold_pos.size, cold_w, cold_s, lr, eps)
+
+
+# ---------------------------------------------------------------------------
 # combine: python/EmbCache/sparse_optim.py:132-157
 # ---------------------------------------------------------------------------
 def only_unique_grads(idx, grad):

@@ -1154,3 +1154,242 @@ def test_accumulator_rejects_negative_ids(lib):
     f_ids, f_sums, f_cnts = acc.flush()
     assert f_ids.tolist() == [5, 77] and f_cnts.tolist() == [1, 1]
     assert bool((f_sums == 1).all())
+
+
+# ---- the split schedule: lookup + partition, then one kernel per class -------------------
+def _split_case(rng, N, D, H, n, hot_frac):
+    """ids with a chosen share of hot ones; hot copies differ from the cold copies so that a row's
+    source shows in its value."""
+    cold = (rng.standard_normal((N, D)) * 0.01).astype(np.float32)
+    hot_ids = np.sort(rng.choice(N, H, replace=False)).astype(np.int64) if H else np.zeros(0, np.int64)
+    cold_ids = np.setdiff1d(np.arange(N, dtype=np.int64), hot_ids)
+    is_hot = rng.random(n) < hot_frac
+    if H == 0:
+        is_hot[:] = False
+    if cold_ids.size == 0:
+        is_hot[:] = True
+    q = np.where(is_hot, hot_ids[rng.integers(0, max(H, 1), n)] if H else 0,
+                 cold_ids[rng.integers(0, max(cold_ids.size, 1), n)] if cold_ids.size else 0).astype(np.int64)
+    return cold, hot_ids, q
+
+
+@pytest.mark.parametrize("N,D,H,n,hot_frac", [
+    (5000, 128, 500, 20_000, 0.9),      # the usual mix
+    (5000, 64, 500, 20_000, 1.0),       # all hot: the cold class is empty
+    (5000, 64, 500, 20_000, 0.0),       # all cold: the hot class is empty
+    (5000, 7, 0, 3000, 0.0),            # no hot set at all, scalar row path
+    (300, 100, 300, 4097, 1.0),         # every id hot
+    (70_000, 128, 9000, 2049, 0.5), (70_000, 128, 9000, 2048, 0.5), (70_000, 128, 9000, 1, 0.5),
+    (10, 4, 3, 0, 0.5),                 # empty batch
+])
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_split_schedule_fetch_and_update(lib, N, D, H, n, hot_frac, host_cold):
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad
+    rng = np.random.default_rng(N + n + int(10 * hot_frac))
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, hot_frac)
+    t_cold = torch.from_numpy(cold.copy())
+    t_cold = t_cold.pin_memory() if host_cold else t_cold.cuda()
+    opt = SparseAdagrad(t_cold, torch.from_numpy(hot_ids), lr=0.01, eps=1e-10)
+    opt.hot_w += 1.0                                     # hot copy != cold copy from here on
+    hw = opt.hot_w.cpu().numpy().copy()
+    # lookup + partition
+    t_q = dev(q)
+    loc, hot_pos, cold_pos, counts = ops.lookup_split(t_q, opt.hot_set)
+    w_loc, w_hp, w_cp = O.lookup_split(q, hot_ids)
+    nh, nc = counts.tolist()
+    assert (nh, nc) == (w_hp.size, w_cp.size)
+    assert np.array_equal(loc.cpu().numpy(), w_loc)
+    assert np.array_equal(hot_pos[:nh].cpu().numpy(), w_hp) and np.array_equal(cold_pos[:nc].cpu().numpy(), w_cp)
+    # fetch, class by class on two streams == the oracle's cached_fetch == the one-kernel fetch
+    want = O.cached_fetch(cold, hw, q, hot_ids)
+    got = opt.fetch_split(t_q)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    if n:
+        assert torch.equal(got, ops.cached_fetch(opt.cold_w, opt.hot_w, t_q, opt.hot_set))
+    # update: combine (EXACT), then the class-by-class Adagrad == oracle, bit for bit
+    grad = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+    cw, cs = cold.copy(), np.zeros_like(cold)
+    hs = np.zeros_like(hw)
+    for _ in range(2):
+        uids, sums, cnts, nu = opt.step_split(t_q, dev(grad), mode=ops.COMBINE_EXACT)
+        wu, ws, _ = O.combine_sequential(q, grad)
+        O.sparse_adagrad_step(cw, cs, hw, hs, hot_ids, wu, ws, 0.01, 1e-10)
+    torch.cuda.synchronize()
+    assert np.array_equal(opt.cold_w.cpu().numpy(), cw) and np.array_equal(opt.cold_s.cpu().numpy(), cs)
+    assert np.array_equal(opt.hot_w.cpu().numpy(), hw) and np.array_equal(opt.hot_s.cpu().numpy(), hs)
+
+
+def test_listed_operators_partial_counts_and_strided_tables(lib):
+    """fetch_listed / set_listed / adagrad_update_listed_ with a device-side count below, at and
+    above the list length, a negative count, and a host table whose weight and state rows are
+    interleaved ([N, 2, D]: one burst per row over the host link)."""
+    _, ops = lib
+    rng = np.random.default_rng(8)
+    N, D, n = 4000, 128, 3000
+    both = torch.empty((N, 2, D), dtype=torch.float32).pin_memory()
+    both.copy_(torch.from_numpy(rng.standard_normal((N, 2, D)).astype(np.float32)))
+    both[:, 1].abs_()
+    w, s = both[:, 0], both[:, 1]                       # row stride 2 * D
+    ref = both.numpy().copy()
+    idx = rng.permutation(N)[:n].astype(np.int64)
+    pos = rng.permutation(n).astype(np.int64)
+    t_idx, t_pos = dev(idx), dev(pos)
+    for count in (0, 1, 777, n, n + 5, -1):
+        live = max(0, min(count, n))
+        t_count = torch.tensor([count], dtype=torch.int64, device="cuda")
+        out = torch.full((n, D), -7.0, device="cuda")
+        ops.fetch_listed(w, t_idx, t_pos, t_count, out)
+        want = O.fetch_listed(ref[:, 0], idx, pos, live, np.full((n, D), -7.0, np.float32))
+        assert np.array_equal(out.cpu().numpy(), want)
+        g = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+        ops.adagrad_update_listed_(t_idx, dev(g), t_pos, t_count, w, s, 0.01, 1e-10)
+        rw, rs = ref[:, 0].copy(), ref[:, 1].copy()
+        O.adagrad_listed(idx, g, pos, live, rw, rs, 0.01, 1e-10)
+        ref[:, 0], ref[:, 1] = rw, rs
+        torch.cuda.synchronize()
+        assert np.array_equal(both.numpy(), ref)
+        src = np.abs(rng.standard_normal((n, D))).astype(np.float32)     # a state row: >= 0
+        ops.set_listed(dev(src), s, t_idx, t_pos, t_count)
+        rs = ref[:, 1].copy()
+        O.set_listed(src, rs, idx, pos, live)
+        ref[:, 1] = rs
+        torch.cuda.synchronize()
+        assert np.array_equal(both.numpy(), ref)
+    # the optimizer on the interleaved host table: split schedule, hot copies in HBM
+    hot_ids = np.sort(rng.choice(N, 300, replace=False)).astype(np.int64)
+    from hades_amd.sparse_optim import SparseAdagrad
+    both[:, 1].zero_()
+    ref = both.numpy().copy()
+    opt = SparseAdagrad(w, torch.from_numpy(hot_ids), cold_state=s)
+    q = rng.integers(0, N, 10_000).astype(np.int64)
+    grad = (rng.standard_normal((q.size, D)) * 1e-3).astype(np.float32)
+    rows = opt.fetch_split(dev(q))
+    assert np.array_equal(rows.cpu().numpy(), ref[:, 0][q])
+    opt.step_split(dev(q), dev(grad), mode=ops.COMBINE_EXACT)
+    torch.cuda.synchronize()
+    cw, cs = ref[:, 0].copy(), ref[:, 1].copy()
+    hw, hs = cw[hot_ids].copy(), cs[hot_ids].copy()
+    wu, ws, _ = O.combine_sequential(q, grad)
+    O.sparse_adagrad_step(cw, cs, hw, hs, hot_ids, wu, ws, 0.01, 1e-10)
+    assert np.array_equal(both[:, 0].numpy(), cw) and np.array_equal(both[:, 1].numpy(), cs)
+    assert np.array_equal(opt.hot_w.cpu().numpy(), hw) and np.array_equal(opt.hot_s.cpu().numpy(), hs)
+
+
+# ---- pinning and the library's own pinned allocation (src/cuda/pin_memory.cu:9-26) -------------
+def test_library_pinned_allocation_through_the_c_abi(lib):
+    """hades_host_alloc -> fill from the host -> hades_fetch2 / hades_set / hades_cached_fetch /
+    hades_adagrad_update on that memory -> oracle -> hades_host_free, all through the C ABI with
+    raw pointers."""
+    import ctypes
+    from hades_amd import _lib
+    L = _lib.load()
+    rng = np.random.default_rng(404)
+    N, D, n = 20_000, 96, 5_000
+    nbytes = N * D * 4
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for flags in (0, _lib.HOST_NONCOHERENT):
+        raw = ctypes.c_void_p()
+        _lib.call("hades_host_alloc_flags", ctypes.byref(raw), nbytes, flags)
+        assert raw.value
+        host = np.ctypeslib.as_array((ctypes.c_float * (N * D)).from_address(raw.value)).reshape(N, D)
+        host[:] = rng.standard_normal((N, D)).astype(np.float32)          # filled by the CPU
+        want_tab = host.copy()
+        idx = rng.permutation(N)[:n].astype(np.int64)
+        t_idx = dev(idx)
+        # gather out of the host table
+        out = torch.empty((n, D), device="cuda")
+        _lib.call("hades_fetch2", raw, ctypes.c_void_p(t_idx.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+                  n, D, _lib.F32, _lib.I64, st)
+        assert np.array_equal(out.cpu().numpy(), O.fetch2(want_tab, idx))
+        # scatter into it
+        src = rng.standard_normal((n, D)).astype(np.float32)
+        t_src = dev(src)
+        _lib.call("hades_set", ctypes.c_void_p(t_src.data_ptr()), raw, ctypes.c_void_p(t_idx.data_ptr()),
+                  n, D, _lib.F32, _lib.I64, st)
+        torch.cuda.synchronize()
+        O.set_rows(src, want_tab, idx)
+        assert np.array_equal(host, want_tab)
+        # the host table as the cold half of a cached fetch and of an Adagrad update
+        hot_ids = np.sort(rng.choice(N, 1500, replace=False)).astype(np.int64)
+        t_hot_ids = dev(hot_ids)
+        hot_w = dev(want_tab[hot_ids] + 1.0)
+        hot_s = torch.zeros_like(hot_w)
+        cold_s = torch.zeros((N, D), device="cuda")
+        q = rng.integers(0, N, n).astype(np.int64)
+        t_q = dev(q)
+        _lib.call("hades_cached_fetch", raw, ctypes.c_void_p(hot_w.data_ptr()), ctypes.c_void_p(t_q.data_ptr()), n,
+                  ctypes.c_void_p(t_hot_ids.data_ptr()), hot_ids.size, None, ctypes.c_void_p(out.data_ptr()),
+                  None, D, _lib.F32, st)
+        assert np.array_equal(out.cpu().numpy(), O.cached_fetch(want_tab, hot_w.cpu().numpy(), q, hot_ids))
+        uq = np.unique(q)
+        g = (rng.standard_normal((uq.size, D)) * 1e-3).astype(np.float32)
+        t_uq, t_g = dev(uq), dev(g)
+        _lib.call("hades_adagrad_update", ctypes.c_void_p(t_uq.data_ptr()), ctypes.c_void_p(t_g.data_ptr()), None,
+                  uq.size, D, ctypes.c_void_p(t_hot_ids.data_ptr()), hot_ids.size, None,
+                  ctypes.c_void_p(hot_w.data_ptr()), ctypes.c_void_p(hot_s.data_ptr()), raw,
+                  ctypes.c_void_p(cold_s.data_ptr()), 0.01, 1e-10, st)
+        torch.cuda.synchronize()
+        hw, hs, cs = (want_tab[hot_ids] + 1.0).astype(np.float32), np.zeros((1500, D), np.float32), np.zeros((N, D), np.float32)
+        O.sparse_adagrad_step(want_tab, cs, hw, hs, hot_ids, uq, g, 0.01, 1e-10)
+        assert np.array_equal(host, want_tab) and np.array_equal(hot_w.cpu().numpy(), hw)
+        assert np.array_equal(cold_s.cpu().numpy(), cs)
+        del host
+        _lib.call("hades_host_free", raw)
+    assert L.hades_host_free(None) == 0                   # freeing nothing is fine
+    assert L.hades_host_alloc(None, 16) == 1              # null out pointer: an error code, no crash
+
+
+def test_host_alloc_tensor_and_cudapin_on_pageable_memory(lib):
+    """EmbCacheLib.host_alloc gives a host tensor the kernels accept as a cold table; cudaPin on a
+    tensor that is already pinned is a no-op; on pageable memory it either registers the memory
+    (then a kernel can read it) or raises RuntimeError where the platform refuses hipHostRegister:
+    it never ends the process (the reference's CUDA_CALL does, src/utils.h:12-24)."""
+    E, ops = lib
+    rng = np.random.default_rng(1)
+    t = E.host_alloc((3000, 64), torch.float32)
+    assert not t.is_cuda and tuple(t.shape) == (3000, 64)
+    t.copy_(torch.from_numpy(rng.standard_normal((3000, 64)).astype(np.float32)))
+    idx = dev(rng.integers(0, 3000, 500).astype(np.int64))
+    out = torch.empty((500, 64), device="cuda")
+    E.cudaFetch2(t, idx, out)
+    assert torch.equal(out.cpu(), t[idx.cpu()])
+    E.cudaPin(t)                                           # already page-locked: nothing to do
+    E.host_free(t)
+    with pytest.raises(RuntimeError):
+        E.host_free(torch.empty(4))
+    pageable = torch.from_numpy(rng.standard_normal((1000, 16)).astype(np.float32))
+    with pytest.raises(RuntimeError, match="pageable"):
+        E.cudaFetch2(pageable, idx % 1000, torch.empty((500, 16), device="cuda"))
+    try:
+        E.cudaPin(pageable)
+    except RuntimeError as err:
+        assert "hipHostRegister" in str(err) or "hades_pin" in str(err)
+    else:
+        o2 = torch.empty((500, 16), device="cuda")
+        E.cudaFetch2(pageable, idx % 1000, o2)
+        assert torch.equal(o2.cpu(), pageable[(idx % 1000).cpu()])
+        E.cudaUnpin(pageable)
+    # the process and the HIP runtime are still in working order
+    assert torch.equal(ops.lookup(idx, torch.arange(3000, device="cuda")), idx)
+
+
+def test_index_cache_accepts_host_tensors_like_the_reference(lib):
+    """The reference calls IndexCache.lookup with CPU tensors and moves the result back
+    (python/EmbCache/dist_emb.py:183-185): CPU in gives CPU out, with the device path's values."""
+    from hades_amd.index_cache import IndexCache
+    rng = np.random.default_rng(12)
+    ic = IndexCache(4096)
+    model = O.SACacheIndexModel(4096)
+    ids = rng.integers(0, 100_000, 3000).astype(np.int64)
+    got = ic.add(torch.from_numpy(ids))
+    assert not got.is_cuda and np.array_equal(got.numpy(), model.add(ids))
+    probe = rng.integers(0, 100_000, 2000).astype(np.int64)
+    assert np.array_equal(ic.cudalookup(torch.from_numpy(probe)).numpy(), model.cudalookup(probe))
+    got = ic.lookup(torch.from_numpy(probe))
+    assert not got.is_cuda and np.array_equal(got.numpy(), model.lookup(probe))
+    assert np.array_equal(ic.lookup(dev(probe)).cpu().numpy(), model.lookup(probe))     # device path
+    ic.reset(torch.from_numpy(ids[:100]))
+    model.reset(ids[:100])
+    assert ic.get_valid_entries_num() == model.get_valid_entries_num()

@@ -562,3 +562,53 @@ def test_cold_cache_server_model_against_per_id_bookkeeping():
     due0 = [int(i) for i in (120, 149) if thr[i] <= 0]           # first flush: iter 0 >= thr never
     assert out_ids.tolist() == sorted([100] + due0)              # id 100 reached cnt_threshold
     assert np.array_equal(out_g[0], (lg[0] + lg[0]).astype(np.float32)) and out_c[0] == 2
+
+
+def test_split_schedule_equals_the_unsplit_operators():
+    """The class-by-class forms (python/EmbCache/dist_emb.py:174-211) against the one-kernel forms
+    and against brute force: every row comes from the table its class says, lists are ascending
+    and disjoint and cover the live prefix, entries beyond num_live are in neither list."""
+    rng = np.random.default_rng(31)
+    N, D, H, n = 3000, 5, 400, 2000
+    cold = rng.standard_normal((N, D)).astype(np.float32)
+    hot_ids = np.sort(rng.choice(N, H, replace=False)).astype(np.int64)
+    hot = cold[hot_ids] + 100.0      # hot copies differ from the cold copies: the source shows
+    q = rng.integers(0, N, n).astype(np.int64)
+    loc, hot_pos, cold_pos = O.lookup_split(q, hot_ids)
+    member = {int(v): k for k, v in enumerate(hot_ids)}
+    assert [member.get(int(v), -1) for v in q] == loc.tolist()
+    assert sorted(hot_pos.tolist() + cold_pos.tolist()) == list(range(n))
+    assert np.all(np.diff(hot_pos) > 0) and np.all(np.diff(cold_pos) > 0)
+    assert all(int(q[p]) in member for p in hot_pos) and not any(int(q[p]) in member for p in cold_pos)
+    out = O.fetch_split(cold, hot, q, hot_ids)
+    assert np.array_equal(out, O.cached_fetch(cold, hot, q, hot_ids))
+    assert np.array_equal(out[hot_pos], hot[loc[hot_pos]]) and np.array_equal(out[cold_pos], cold[q[cold_pos]])
+    # num_live
+    loc2, hp2, cp2 = O.lookup_split(q, hot_ids, num_live=700)
+    assert hp2.tolist() == [p for p in hot_pos if p < 700] and cp2.tolist() == [p for p in cold_pos if p < 700]
+    assert O.lookup_split(q, hot_ids, num_live=-1)[1].size == 0
+    # a partial count leaves the other positions alone
+    out3 = np.full((n, D), -7.0, np.float32)
+    O.fetch_listed(cold, q, cold_pos, 10, out3)
+    assert np.array_equal(out3[cold_pos[:10]], cold[q[cold_pos[:10]]])
+    rest = np.ones(n, bool); rest[cold_pos[:10]] = False
+    assert np.all(out3[rest] == -7.0)
+    # set_listed is the inverse scatter
+    uq = rng.permutation(N)[:n].astype(np.int64)
+    l3, hp3, cp3 = O.lookup_split(uq, hot_ids)
+    src = rng.standard_normal((n, D)).astype(np.float32)
+    c_a, h_a = cold.copy(), hot.copy()
+    O.set_listed(src, h_a, l3, hp3, hp3.size)
+    O.set_listed(src, c_a, uq, cp3, cp3.size)
+    c_b, h_b = cold.copy(), hot.copy()
+    O.cached_set(src, c_b, h_b, uq, hot_ids)
+    assert np.array_equal(c_a, c_b) and np.array_equal(h_a, h_b)
+    # the update, class by class == the fused form; rows of no class do not move
+    g = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+    s0 = np.abs(rng.standard_normal((N, D))).astype(np.float32)
+    a = [cold.copy(), s0.copy(), hot.copy(), s0[hot_ids].copy()]
+    b = [x.copy() for x in a]
+    O.sparse_adagrad_step(a[0], a[1], a[2], a[3], hot_ids, uq[:1500], g[:1500], 0.01, 1e-10)
+    O.sparse_adagrad_step_split(b[0], b[1], b[2], b[3], hot_ids, uq, g, 0.01, 1e-10, num_live=1500)
+    for x, y in zip(a, b):
+        assert np.array_equal(x, y)
