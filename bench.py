@@ -1,7 +1,7 @@
 """Benchmark of the embedding-cache hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]      the headline workload (cfg3) + cfg2 nested
-    python bench.py --workload cfg2|cfg3|cfg5 [--mode fast|exact] [--schedule serial|split|overlap|graph]
+    python bench.py --workload cfg2|cfg3|cfg5 [--mode fast|exact] [--schedule serial|keyed|split|overlap|graph]
     python bench.py --workload cfg4          cold-gradient accumulator with delayed write-back
     python bench.py --workload cfg4 --flush-rule staleness    the cache server's own per-row rule
     python bench.py --workload neighbours    pre-exchange bucketing, index cache, cold-data cache
@@ -9,9 +9,11 @@
 One step = lookup + cached_fetch of the query rows, combine of the per-query gradients, and the
 sparse Adagrad update of every distinct row, on one batch of synthetic Zipf ids that is already
 resident in HBM.  The headline workload keeps 10 % of a 111 M x 128 table in HBM and the rest in
-pinned host memory; its step runs on the split schedule: lookup + stable hot/cold partition, then
-the hot rows through kernels that only touch HBM and the cold rows through kernels that only touch
-the host table, on two streams.  Prints ONE JSON line: whole-step throughput in query rows/s
+pinned host memory; its step runs on the keyed schedule: one lookup + stable hot/cold partition per
+query batch, then the hot rows through kernels that only touch HBM and the cold rows through narrow
+kernels that only touch the host table, on two streams; the combine sorts class-ordered keys, so
+the cold class is summed first and its update crosses the host link while the hot class is still
+being summed and updated.  Prints ONE JSON line: whole-step throughput in query rows/s
 (mean, median, p10/p90 over the timed steps), the HBM roofline of every row kernel (algorithmic
 bytes / HIP-event time of its launches inside the timed region), the host-link roofline of the
 cold-row kernels against the nominal 64 GB/s and against pinned hipMemcpyAsync rates measured in
@@ -55,11 +57,14 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
-    ap.add_argument("--schedule", default=None, choices=["serial", "split", "overlap", "graph"],
+    ap.add_argument("--schedule", default=None, choices=["serial", "keyed", "split", "overlap", "graph"],
                     help="serial: every kernel of the step on one stream, hot and cold rows in the "
-                         "same kernels (default when the whole table is in HBM); split: lookup + "
-                         "hot/cold partition, hot rows on one stream, cold rows on another (default "
-                         "when the cold table is in host memory); overlap: serial with the sort of "
+                         "same kernels (default when the whole table is in HBM); keyed: one lookup + "
+                         "hot/cold partition per batch, hot rows on one stream, cold rows on "
+                         "another, combine over class-ordered keys so that the cold update starts "
+                         "first (default when the cold table is in host memory); split: the same "
+                         "two streams with a plain combine and a second lookup of the distinct "
+                         "ids; overlap: serial with the sort of "
                          "the ids on a side stream next to the fetch; graph: serial, every step the "
                          "replay of a HIP graph captured once per batch")
     ap.add_argument("--flush-rule", default="every8", choices=["every8", "staleness"],
@@ -270,8 +275,9 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
     n, D, N = wl.n, wl.D, wl.N
     K = args.steps
     if schedule is None:
-        schedule = "split" if wl.host_cold else "serial"
+        schedule = "keyed" if wl.host_cold else "serial"
     split = schedule == "split"
+    keyed = schedule == "keyed"
     overlap = schedule == "overlap"
 
     def new_events(count):
@@ -298,7 +304,15 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
         out_ids = (uids_o[:sizes], nu_o)
         out_sum = (sums_o[:sizes], cnts_o[:sizes])
         if events: events[0].record()
-        if split:
+        if keyed:
+            # forward: lookup + partition + both gathers + sort of the class-ordered keys; the
+            # join inside it is where a trainer's forward and backward would sit.  backward: cold
+            # sums, cold update on the cold stream, hot sums and hot update beside it, join.
+            _, state = opt.forward_keyed(q, out=rows, timing=timing)
+            if events: events[1].record()
+            if events: events[2].record()
+            res = opt.backward_keyed(state, g, cmode, timing=timing)
+        elif split:
             opt.fetch_split(q, out=rows, join=False, timing=timing)
             plan = ops.combine_plan(q, D, id_bound=N, workspace=opt._ws, out=out_ids)
             opt.join()
@@ -324,9 +338,20 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
     def step(i, events=None, timing=None):
         run_step(wl.ids[i % nb], wl.grads[i % nb], mode, events, timing)
 
+    def gate_step(q, g, m):
+        """one step for the parity gate: rows and the distinct rows in id order"""
+        rows, res = run_step(q, g, m)
+        if keyed:
+            ukeys, sums, cnts, nu, _ = res
+            ids = opt.distinct_ids_of(ukeys, nu)
+            order = torch.argsort(ids)
+            u = ids.numel()
+            return rows, (ids[order], sums[:u][order], cnts[:u][order], nu)
+        return rows, res
+
     gate = None
     if with_gate:
-        gate = parity_gate(wl, lambda q, g, m: run_step(q, g, m))
+        gate = parity_gate(wl, gate_step)
         log("parity gate passed: %s" % json.dumps(gate["max_rel_err"]))
     link = link_probe(dev) if (with_link and wl.host_cold) else None
     if link:
@@ -350,12 +375,14 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
     every = max(1, args.event_every)
     sampled = [i for i in range(K) if i % every == 0]
     seg_name = "seg_chunk_kernel" if args.mode == "fast" else "seg_exact_kernel + seg_exact_long_kernel"
-    if split:
+    if split or keyed:
+        upd = "hades_adagrad_update_class" if keyed else "hades_adagrad_update_listed"
         knames = {"hot_fetch": "row_move_listed_kernel<gather> over the hot class (hades_fetch_listed)",
                   "cold_fetch": "row_move_listed_kernel<gather> over the cold class (hades_fetch_listed)",
-                  "seg_sum": seg_name + " (hades_combine_apply)",
-                  "hot_update": "adagrad_listed_kernel over the hot class (hades_adagrad_update_listed)",
-                  "cold_update": "adagrad_listed_kernel over the cold class (hades_adagrad_update_listed)"}
+                  "seg_sum": seg_name + (" over the hot class (hades_combine_apply_class)" if keyed
+                                         else " (hades_combine_apply)"),
+                  "hot_update": "adagrad_listed_kernel over the hot class (%s)" % upd,
+                  "cold_update": "adagrad_listed_kernel over the cold class (%s)" % upd}
         hook_of = {"seg_sum": ops.KERNEL_SEG_SUM}
     else:
         knames = {"fetch": "row_move_kernel<AddrFetchSorted> (hades_cached_fetch)",
@@ -411,7 +438,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
             tim = None
             if i % every == 0:
                 j = i // every
-                if split:
+                if split or keyed:
                     tim = {k: kev[i][k] for k in knames if k not in hook_of}
                     hk = "seg_sum"
                     armed[i] = list(knames)
@@ -431,6 +458,20 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
         for k in names:
             kernel_ms[k].append(kev[i][k][0].elapsed_time(kev[i][k][1]))
     step_ms = [step_ev[i].elapsed_time(step_ev[i + 1]) for i in range(K)]
+
+    # the same kernels undisturbed: a few untimed steps with both classes on one stream
+    alone_ms = {}
+    if split or keyed:
+        opt.one_stream = True
+        aev = [{k: new_events(2) for k in knames} for _ in range(3)]
+        for j in range(3):
+            tim = {k: aev[j][k] for k in knames if k not in hook_of}
+            ops.profile_kernel(hook_of["seg_sum"], aev[j]["seg_sum"][0], aev[j]["seg_sum"][1])
+            step(j, timing=tim)
+        ops.profile_kernel(0)
+        torch.cuda.synchronize()
+        opt.one_stream = False
+        alone_ms = {k: sum(aev[j][k][0].elapsed_time(aev[j][k][1]) for j in range(3)) / 3 for k in knames}
 
     # phases: a second, untimed pass with four event records per step on the main stream
     for i in range(K):
@@ -461,7 +502,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
     # the update (weights; the cold Adagrad state sits in HBM).
     row_f, row_u = 16 + 8 * D, 8 + 20 * D
     alg_bytes = {"fetch": n * row_f, "combine": n * (8 + 4 * D) + U * (16 + 4 * D), "update": U * row_u}
-    kbytes = {"fetch": n * row_f, "update": U * row_u, "seg_sum": n * (8 + 4 * D) + U * 4 * D,
+    kbytes = {"fetch": n * row_f, "update": U * row_u,
+              "seg_sum": (n_hot * (8 + 4 * D) + U_hot * 4 * D) if keyed else (n * (8 + 4 * D) + U * 4 * D),
               "hot_fetch": n_hot * row_f, "cold_fetch": n_cold * row_f,
               "hot_update": U_hot * row_u, "cold_update": U_cold * row_u}
     traffic = measured_traffic(workload, args.mode)
@@ -473,6 +515,12 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
         gbs = kbytes[k] / (ms * 1e-3) / 1e9
         entry = {"kernel": name, "us": round(ms * 1e3, 2), "launches_timed": len(kernel_ms[k]),
                  "bytes_per_launch": int(kbytes[k]), "GB/s": round(gbs, 1)}
+        if k in alone_ms:
+            a_ms = alone_ms[k]
+            entry["us_alone"] = round(a_ms * 1e3, 2)
+            entry["GB/s_alone"] = round(kbytes[k] / (a_ms * 1e-3) / 1e9, 1)
+            if not (k.startswith("cold_") and wl.host_cold):
+                entry["frac_alone"] = round(kbytes[k] / (a_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
         if k.startswith("cold_") and wl.host_cold:
             entry["bound"] = "pcie"
         else:
@@ -498,17 +546,32 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
                 "timing": "HIP events recorded on the launch stream right before and after the "
                           "launch: the kernel plus about 3 us of dispatch latency",
                 "bytes_per_launch": mk["bytes_per_launch"]}
-    if split:
+    if split or keyed:
         hot_b = sum(kbytes[k] for k in ("hot_fetch", "seg_sum", "hot_update"))
         hot_ms = sum(kernels[k]["us"] for k in ("hot_fetch", "seg_sum", "hot_update")) / 1e3
         roofline["hot_traffic_all_row_kernels"] = {
             "GB/s": round(hot_b / (hot_ms * 1e-3) / 1e9, 1),
             "frac": round(hot_b / (hot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "note": "hot gather + segmented sum + hot update: algorithmic bytes over the sum of "
-                    "their kernel times"}
+                    "their kernel times in the timed region, where the segmented sum and the hot "
+                    "update run beside the cold update and slow down with it"}
+        if alone_ms:
+            a_ms = sum(alone_ms[k] for k in ("hot_fetch", "seg_sum", "hot_update"))
+            roofline["hot_traffic_all_row_kernels"]["GB/s_alone"] = round(hot_b / (a_ms * 1e-3) / 1e9, 1)
+            roofline["hot_traffic_all_row_kernels"]["frac_alone"] = round(
+                hot_b / (a_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            roofline["hot_traffic_all_row_kernels"]["alone_note"] = (
+                "the same kernels in three untimed steps with both classes on one stream "
+                "(nothing on the host link beside them)")
+    if keyed:       # the sums are interleaved with the updates: one backward phase
+        phase_ms = {"fetch": phase_ms["fetch"], "combine+update": phase_ms["combine"] + phase_ms["update"]}
+        phase_bytes = {"fetch": alg_bytes["fetch"], "combine+update": alg_bytes["combine"] + alg_bytes["update"]}
+        phases = tuple(phase_ms)
+    else:
+        phase_bytes = alg_bytes
     per_phase = {p: {"ms": round(phase_ms[p], 4),
-                     "GB/s": round(alg_bytes[p] / (phase_ms[p] * 1e-3) / 1e9, 1),
-                     "frac_hbm": round(alg_bytes[p] / (phase_ms[p] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                     "GB/s": round(phase_bytes[p] / (phase_ms[p] * 1e-3) / 1e9, 1),
+                     "frac_hbm": round(phase_bytes[p] / (phase_ms[p] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
                  for p in phases}
     total_bytes = sum(alg_bytes.values())
     res = {"workload": wl.describe(), "schedule": schedule, "n": n,
@@ -522,7 +585,11 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
            "phases_note": "from a second, untimed pass with four event records per step (each adds "
                           "3-4 us to its phase)" +
                           ("; fetch = both gathers and the id sort that runs beside the cold one"
-                           if split else ""),
+                           if split else "") +
+                          ("; fetch = the forward half (lookup, partition, both gathers, sort of the "
+                           "keys beside the cold gather); combine is inside update = the backward "
+                           "half (cold sums, cold update beside hot sums and hot update)"
+                           if keyed else ""),
            "step_alg_GB": round(total_bytes / 1e9, 4),
            "step_GB/s": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
            "step_frac_hbm": round(total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -537,7 +604,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
         pcie = {"bound": "pcie", "peak": PCIE_PEAK_GBS, "unit": "GB/s per direction",
                 "cold_query_rows": round(n_cold, 1), "cold_unique_rows": round(U_cold, 1),
                 "memcpy": link}
-        if split:
+        if split or keyed:
             f, f_gbs = link_entry(n_cold, kernels["cold_fetch"]["us"] / 1e3)
             u, u_gbs = link_entry(U_cold, kernels["cold_update"]["us"] / 1e3)
             timing_note = "cold-class kernels bracketed by HIP events on the cold stream"
@@ -974,6 +1041,10 @@ def main():
                    "schedule": {"serial": "one stream, hot and cold rows in the same kernels",
                                 "split": "lookup + hot/cold partition; hot rows on the main stream, "
                                          "cold rows on a second stream of the same priority",
+                                "keyed": "one lookup + hot/cold partition per batch; hot rows on the "
+                                         "main stream, cold rows on a second stream of the same "
+                                         "priority; combine over class-ordered keys: the cold class "
+                                         "is summed first and its update overlaps the hot class",
                                 "overlap": "one stream + the sort of the step's ids on a side stream, "
                                            "concurrent with its fetch",
                                 "graph": "one stream, every step replayed from a HIP graph captured "

@@ -49,13 +49,13 @@ constexpr int kScanFrom = 64;  // groups of tiles from which the group counts ge
 
 // ---- key transforms ---------------------------------------------------------
 template <typename KeyT>
-__device__ __forceinline__ KeyT key_from_id(int64_t id);
+__host__ __device__ __forceinline__ KeyT key_from_id(int64_t id);
 template <>
-__device__ __forceinline__ uint32_t key_from_id<uint32_t>(int64_t id) {
+__host__ __device__ __forceinline__ uint32_t key_from_id<uint32_t>(int64_t id) {
   return static_cast<uint32_t>(id);
 }
 template <>
-__device__ __forceinline__ uint64_t key_from_id<uint64_t>(int64_t id) {
+__host__ __device__ __forceinline__ uint64_t key_from_id<uint64_t>(int64_t id) {
   return static_cast<uint64_t>(id) ^ (uint64_t(1) << 63);  // signed order -> unsigned order
 }
 template <typename KeyT>
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
     const uint32_t* __restrict__ blk_cnt, int64_t* __restrict__ uids,
     uint32_t* __restrict__ seg_start, uint32_t* __restrict__ seg_of,
     int64_t* __restrict__ num_unique, int32_t* __restrict__ inverse,
-    const int32_t* __restrict__ bad_blk, int64_t nbad) {
+    const int32_t* __restrict__ bad_blk, int64_t nbad, KeyT thr, int64_t* __restrict__ class_split) {
   __shared__ uint32_t smem[kWaves + 1];
   // the block that writes num_unique first learns whether the first count pass saw an id outside
   // [0, id_bound): it then reports -1 distinct ids, which every consumer treats as "no live rows"
@@ -361,10 +361,20 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
         if (flag[k]) {
           uids[seg] = id_from_key<KeyT>(kk[k]);
           seg_start[seg] = static_cast<uint32_t>(j);
+          // the first key at or above the threshold opens the upper class (keys are ascending)
+          if (class_split != nullptr && kk[k] >= thr &&
+              (j == 0 || (k > 0 ? kk[k - 1] : keys[j - 1]) < thr)) {
+            class_split[0] = j;
+            class_split[1] = static_cast<int64_t>(seg);
+          }
         }
         if (j == n - 1) {
           seg_start[u] = static_cast<uint32_t>(n);
           num_unique[0] = violated ? int64_t(-1) : static_cast<int64_t>(u);
+          if (class_split != nullptr && kk[k] < thr) {   // no key reaches the threshold
+            class_split[0] = n;
+            class_split[1] = static_cast<int64_t>(u);
+          }
         }
       }
     }
@@ -410,7 +420,22 @@ struct SegArgs {
   int64_t dim;
   int group;       // lanes per group
   int col_tiles;   // ceil(dim / (group * VEC))
+  // optional restriction to one class of a class-ordered plan: class_split = {first sorted
+  // position, first run} of the upper class; which = 0 lower class, 1 upper class, -1 everything
+  const int64_t* class_split;
+  int which;
 };
+
+// [*pos_lo, *pos_hi) sorted positions and [*run_lo, *run_hi) runs of the class a launch works on
+__device__ __forceinline__ void class_range(const SegArgs& a, int64_t U, int64_t* pos_lo,
+                                            int64_t* pos_hi, int64_t* run_lo, int64_t* run_hi) {
+  *pos_lo = 0; *pos_hi = a.n; *run_lo = 0; *run_hi = U;
+  if (a.class_split != nullptr && a.which >= 0) {
+    const int64_t sp = a.class_split[0], sr = a.class_split[1];
+    if (a.which == 0) { *pos_hi = sp; *run_hi = sr < U ? sr : U; }
+    else { *pos_lo = sp; *run_lo = sr; }
+  }
+}
 
 // FAST, kernel 1.  A block covers (kThreads / group) * kChunk consecutive sorted positions.
 template <int VEC>
@@ -426,6 +451,12 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
   const int ngroups = kThreads / G;
   const int bp = ngroups * kChunk;
   const int64_t B0 = static_cast<int64_t>(blockIdx.x) * bp;
+  if (a.class_split != nullptr && a.which >= 0) {
+    // a block works if its span touches the class; the block that straddles the class border
+    // runs in both launches and writes the same values twice (runs never cross that border)
+    const int64_t sp = a.class_split[0];
+    if (a.which == 0 ? B0 >= sp : B0 + bp <= sp) return;
+  }
   for (int t = threadIdx.x; t < bp + 2; t += kThreads) {
     const int64_t j = B0 - 1 + t;
     s_seg[t] = (j >= 0 && j < a.n) ? a.seg_of[j] : kNoRun;
@@ -557,8 +588,10 @@ __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
   typedef typename RowVec<VEC>::type V;
   __shared__ V s_part[kThreads];
   const int64_t U = a.num_unique[0];
+  int64_t pos_lo, pos_hi, run_lo, run_hi;
+  class_range(a, U, &pos_lo, &pos_hi, &run_lo, &run_hi);
   const int64_t gtid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (gtid < U)
+  if (gtid >= run_lo && gtid < run_hi)
     a.cnts[gtid] = static_cast<int64_t>(a.seg_start[gtid + 1]) - static_cast<int64_t>(a.seg_start[gtid]);
 
   const int G = a.group;
@@ -567,6 +600,7 @@ __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
   const int64_t c = blockIdx.x;
   const int64_t border = (c + 1) * span;
   if (border >= a.n) return;
+  if (border - 1 < pos_lo || border >= pos_hi) return;   // both sides of the border in the class
   const uint32_t u = a.seg_of[border - 1];
   if (a.seg_of[border] != u) return;           // no run crosses this border
   const int64_t start = a.seg_start[u];
@@ -627,7 +661,9 @@ __global__ __launch_bounds__(kThreads) void seg_exact_kernel(SegArgs a) {
   const int64_t gtid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   const int64_t u = gtid / a.group;
   const int gl = static_cast<int>(gtid & (a.group - 1));
-  if (u >= U) return;
+  int64_t pos_lo, pos_hi, run_lo, run_hi;
+  class_range(a, U, &pos_lo, &pos_hi, &run_lo, &run_hi);
+  if (u < run_lo || u >= run_hi) return;
   const int64_t j0 = a.seg_start[u];
   const int64_t j1 = a.seg_start[u + 1];
   if (gl == 0) a.cnts[u] = j1 - j0;
@@ -672,6 +708,10 @@ __global__ __launch_bounds__(kLongThreads) void seg_exact_long_kernel(SegArgs a)
   const int64_t start = a.seg_start[u];
   const int64_t end = a.seg_start[u + 1];
   if (start < span0 || end - start < kLongRun) return;
+  if (a.class_split != nullptr && a.which >= 0) {
+    const int64_t sp = a.class_split[0];
+    if (a.which == 0 ? start >= sp : start < sp) return;
+  }
 
   // A block takes a 32-float slice of the columns (blockIdx.y): every element's chain is
   // independent of the other columns, and one CU alone cannot pull whole rows of a long run fast
@@ -892,13 +932,15 @@ int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, con
 
 template <typename KeyT>
 int run_runs(const void* sorted_keys, const uint32_t* perm, int64_t n, const Plan& p, const Ws& w,
-             int64_t* uids, int64_t* num_unique, int32_t* inverse, hipStream_t st) {
+             int64_t* uids, int64_t* num_unique, int32_t* inverse, hipStream_t st,
+             int64_t threshold = 0, int64_t* class_split = nullptr) {
   const KeyT* keys = static_cast<const KeyT*>(sorted_keys);
   const dim3 rgrid(static_cast<unsigned>(p.nblocks_runs)), block(kThreads);
   HADES_LAUNCH((run_count_kernel<KeyT>), rgrid, block, 0, st, keys, n, w.run_cnt);
   HADES_LAUNCH_CHECK();
   HADES_LAUNCH((run_emit_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt, uids,
-                     w.seg_start, w.seg_of, num_unique, inverse, w.sort.bad, w.sort.nbad);
+                     w.seg_start, w.seg_of, num_unique, inverse, w.sort.bad, w.sort.nbad,
+                     key_from_id<KeyT>(threshold), class_split);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }
@@ -940,9 +982,19 @@ size_t hades_combine_workspace_bytes(int64_t n, int64_t dim) {
   return carve(nullptr, n, dim).bytes;
 }
 
-int hades_combine_plan(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bound, int64_t* uids,
-                       int64_t* num_unique, int32_t* inverse, void* workspace,
-                       size_t workspace_bytes, void* stream) {
+namespace {
+
+__global__ void set_i64x2_kernel(int64_t* p, int64_t a, int64_t b) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    p[0] = a;
+    p[1] = b;
+  }
+}
+
+int combine_plan_impl(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bound, int64_t* uids,
+                      int64_t* num_unique, int32_t* inverse, void* workspace,
+                      size_t workspace_bytes, void* stream, int64_t threshold,
+                      int64_t* class_split) {
   HADES_REQUIRE(n >= 0 && dim >= 1, "n must be >= 0 and dim >= 1");
   HADES_REQUIRE(n < (int64_t(1) << 30), "combine: n must be below 2^30 (got %lld)", (long long)n);
   HADES_REQUIRE(id_bound >= 0, "id_bound must be >= 0");
@@ -950,6 +1002,8 @@ int hades_combine_plan(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bo
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (n == 0) {
     HADES_LAUNCH(set_i64_kernel, dim3(1), dim3(64), 0, st, num_unique, int64_t(0));
+    if (class_split != nullptr)
+      HADES_LAUNCH(set_i64x2_kernel, dim3(1), dim3(64), 0, st, class_split, int64_t(0), int64_t(0));
     return HADES_OK;
   }
   HADES_REQUIRE(idx && uids, "null pointer argument");
@@ -965,13 +1019,37 @@ int hades_combine_plan(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bo
   int rc = p.key64 ? run_sort<uint64_t>(idx, n, id_bound, p, w.sort, st, &sorted_keys, &perm)
                    : run_sort<uint32_t>(idx, n, id_bound, p, w.sort, st, &sorted_keys, &perm);
   if (rc != HADES_OK) return rc;
-  return p.key64 ? run_runs<uint64_t>(sorted_keys, perm, n, p, w, uids, num_unique, inverse, st)
-                 : run_runs<uint32_t>(sorted_keys, perm, n, p, w, uids, num_unique, inverse, st);
+  return p.key64 ? run_runs<uint64_t>(sorted_keys, perm, n, p, w, uids, num_unique, inverse, st,
+                                      threshold, class_split)
+                 : run_runs<uint32_t>(sorted_keys, perm, n, p, w, uids, num_unique, inverse, st,
+                                      threshold, class_split);
 }
 
-int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bound, int mode,
-                        float* sums, int64_t* cnts, const int64_t* num_unique, void* workspace,
-                        size_t workspace_bytes, void* stream) {
+}  // namespace
+
+int hades_combine_plan(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bound, int64_t* uids,
+                       int64_t* num_unique, int32_t* inverse, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+  return combine_plan_impl(idx, n, dim, id_bound, uids, num_unique, inverse, workspace,
+                           workspace_bytes, stream, 0, nullptr);
+}
+
+int hades_combine_plan_classed(const int64_t* keys, int64_t n, int64_t dim, int64_t key_bound,
+                               int64_t threshold, int64_t* ukeys, int64_t* num_unique,
+                               int64_t* class_split, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  HADES_REQUIRE(class_split != nullptr, "class_split must not be null");
+  HADES_REQUIRE(key_bound > 0 && threshold >= 0 && threshold <= key_bound,
+                "key_bound must be > 0 and threshold in [0, key_bound]");
+  return combine_plan_impl(keys, n, dim, key_bound, ukeys, num_unique, nullptr, workspace,
+                           workspace_bytes, stream, threshold, class_split);
+}
+
+namespace {
+
+int combine_apply_impl(const float* grad, int64_t n, int64_t dim, int64_t id_bound, int mode,
+                       float* sums, int64_t* cnts, const int64_t* num_unique, void* workspace,
+                       size_t workspace_bytes, void* stream, const int64_t* class_split, int which) {
   HADES_REQUIRE(n >= 0 && dim >= 1, "n must be >= 0 and dim >= 1");
   HADES_REQUIRE(n < (int64_t(1) << 30), "combine: n must be below 2^30 (got %lld)", (long long)n);
   HADES_REQUIRE(id_bound >= 0, "id_bound must be >= 0");
@@ -1002,6 +1080,8 @@ int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bo
   a.dim = dim;
   a.group = p.group;
   a.col_tiles = p.col_tiles;
+  a.class_split = class_split;
+  a.which = class_split != nullptr ? which : -1;
   if (mode == HADES_COMBINE_EXACT) {
     const int64_t blocks = ceil_div(n * p.group, kThreads);
     HADES_REQUIRE(blocks < (int64_t(1) << 31), "combine: too many rows");
@@ -1050,6 +1130,25 @@ int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bo
     HADES_LAUNCH_CHECK();
   }
   return HADES_OK;
+}
+
+}  // namespace
+
+int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bound, int mode,
+                        float* sums, int64_t* cnts, const int64_t* num_unique, void* workspace,
+                        size_t workspace_bytes, void* stream) {
+  return combine_apply_impl(grad, n, dim, id_bound, mode, sums, cnts, num_unique, workspace,
+                            workspace_bytes, stream, nullptr, -1);
+}
+
+int hades_combine_apply_class(const float* grad, int64_t n, int64_t dim, int64_t key_bound, int mode,
+                              int which, float* sums, int64_t* cnts, const int64_t* num_unique,
+                              const int64_t* class_split, void* workspace, size_t workspace_bytes,
+                              void* stream) {
+  HADES_REQUIRE(class_split != nullptr, "class_split must not be null");
+  HADES_REQUIRE(which == 0 || which == 1, "which must be 0 (below the threshold) or 1");
+  return combine_apply_impl(grad, n, dim, key_bound, mode, sums, cnts, num_unique, workspace,
+                            workspace_bytes, stream, class_split, which);
 }
 
 int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim, int64_t id_bound,

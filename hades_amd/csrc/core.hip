@@ -37,12 +37,12 @@ bool is_host_memory(const void* p) {
 // Measured on 76 K rows of 512 bytes: a gather reaches the link's read rate (55 GB/s) from 32 to
 // 128 blocks; an update, which has reads and writes in flight, peaks at 128 (42.6 GB/s each way).
 int64_t host_link_blocks(bool read_and_write) {
-  const char* e = getenv("HADES_HOST_LINK_BLOCKS");   // tuning override
-  if (e != nullptr) {
+  const char* e = getenv(read_and_write ? "HADES_HOST_LINK_BLOCKS_RW" : "HADES_HOST_LINK_BLOCKS");
+  if (e != nullptr) {                                  // tuning override
     const long v = atol(e);
     if (v >= 1) return v;
   }
-  return read_and_write ? 128 : 64;
+  return read_and_write ? 128 : 16;
 }
 
 }  // namespace hades

@@ -284,10 +284,14 @@ struct ClassifyLookup {
   HotSet hs;
   int64_t* loc;
   const int64_t* num_live;   // optional: only the first num_live[0] queries count
+  int64_t* sort_keys;        // optional: class-ordered sort key of every query (see the header)
+  int key_bits;
   __device__ __forceinline__ uint32_t operator()(int64_t i) const {
     if (num_live != nullptr && i >= num_live[0]) return kNone;
-    const int64_t l = hs.slot(q[i]);
+    const int64_t id = q[i];
+    const int64_t l = hs.slot(id);
     loc[i] = l;
+    if (sort_keys != nullptr) sort_keys[i] = l >= 0 ? ((int64_t(1) << key_bits) | l) : id;
     return l >= 0 ? 0u : 1u;
   }
 };
@@ -505,14 +509,17 @@ int hades_split_compact(const int64_t* loc, int64_t n, uint8_t* hot_mask, int64_
 int hades_lookup_split(const int64_t* q, const int64_t* num_live, int64_t n,
                        const int64_t* sorted_hot, int64_t num_hot,
                        const void* hot_index, int64_t* loc, uint8_t* hot_mask, int64_t* hot_pos,
-                       int64_t* cold_pos, int64_t* counts, void* workspace, size_t workspace_bytes,
-                       void* stream) {
+                       int64_t* cold_pos, int64_t* counts, int64_t* sort_keys, int key_bits,
+                       void* workspace, size_t workspace_bytes, void* stream) {
   HADES_REQUIRE(n >= 0 && num_hot >= 0, "n and num_hot must be >= 0");
+  HADES_REQUIRE(sort_keys == nullptr || (key_bits >= 1 && key_bits <= 61 &&
+                                         num_hot <= (int64_t(1) << key_bits)),
+                "key_bits must be in [1, 61] and leave room for every hot slot");
   HADES_REQUIRE(n == 0 || (q && loc), "null pointer argument");
   HADES_REQUIRE(num_hot == 0 || sorted_hot, "sorted_hot is null but num_hot > 0");
   CompactOut out{{hot_mask, nullptr, nullptr}, {hot_pos, cold_pos, nullptr}};
   ClassifyLookup cf{q, HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}, loc,
-                    num_live};
+                    num_live, sort_keys, key_bits};
   return run_compact(cf, n, 2, out, counts, workspace, workspace_bytes,
                      static_cast<hipStream_t>(stream));
 }

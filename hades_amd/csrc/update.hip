@@ -131,9 +131,14 @@ __global__ __launch_bounds__(kThreads) void adagrad_kernel(AdagradArgs a) {
 struct AdagradListedArgs {
   const int64_t* row_index;
   const float* grad;
-  const int64_t* list;
-  const int64_t* count;
+  const int64_t* list;      // null: positions are the range itself (class form)
+  const int64_t* count;     // listed form: number of live list entries
   int64_t max_count;
+  // class form: rows [class_split[1], num_unique[0]) (which = 1) or [0, class_split[1]) (which = 0)
+  const int64_t* num_unique;
+  const int64_t* class_split;
+  int which;
+  int64_t index_mask;       // table row = row_index[p] & index_mask
   int64_t dim;
   float* w;
   float* s;
@@ -146,16 +151,27 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
   typedef typename Vf<VEC>::type V;
   __shared__ int64_t s_row[kRows];    // element offset of the row in w and s
   __shared__ int64_t s_grad[kRows];   // element offset of the row in grad
-  int64_t cnt = a.count[0];
-  cnt = cnt < a.max_count ? cnt : a.max_count;
+  int64_t first = 0, cnt;
+  if (a.list != nullptr) {
+    cnt = a.count[0];
+    cnt = cnt < a.max_count ? cnt : a.max_count;
+  } else {
+    int64_t U = a.num_unique[0];
+    U = U < a.max_count ? U : a.max_count;
+    int64_t sr = a.class_split[1];
+    sr = sr < U ? sr : U;
+    sr = sr > 0 ? sr : 0;
+    first = a.which ? sr : 0;
+    cnt = a.which ? U : sr;
+  }
   const int cpr = static_cast<int>(a.dim / VEC);
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRows; row0 < cnt;
+  for (int64_t row0 = first + static_cast<int64_t>(blockIdx.x) * kRows; row0 < cnt;
        row0 += static_cast<int64_t>(gridDim.x) * kRows) {
     const int64_t left = cnt - row0;
     const int rows_here = left < kRows ? static_cast<int>(left) : kRows;
     for (int r = threadIdx.x; r < rows_here; r += kThreads) {
-      const int64_t p = a.list[row0 + r];
-      s_row[r] = a.row_index[p] * a.stride;
+      const int64_t p = a.list != nullptr ? a.list[row0 + r] : row0 + r;
+      s_row[r] = (a.row_index[p] & a.index_mask) * a.stride;
       s_grad[r] = p * a.dim;
     }
     __syncthreads();
@@ -278,6 +294,10 @@ int check_rows(const int64_t* uids, const float* grad, int64_t max_rows, int64_t
 
 using namespace hades;
 
+namespace {
+int launch_adagrad_listed(const AdagradListedArgs& a, void* stream);
+}
+
 extern "C" {
 
 int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
@@ -310,7 +330,35 @@ int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, con
   if (max_count == 0) return HADES_OK;
   HADES_REQUIRE(row_index && grad && list && count && w && s, "null pointer argument");
   if (stride == 0) stride = dim;
-  AdagradListedArgs a{row_index, grad, list, count, max_count, dim, w, s, stride, lr, eps};
+  AdagradListedArgs a{row_index, grad, list, count, max_count, nullptr, nullptr, 0, int64_t(-1),
+                      dim, w, s, stride, lr, eps};
+  return launch_adagrad_listed(a, stream);
+}
+
+int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
+                               const int64_t* class_split, int which, int64_t key_mask,
+                               int64_t max_rows, int64_t dim, float* w, float* s, int64_t stride,
+                               float lr, float eps, void* stream) {
+  HADES_REQUIRE(max_rows >= 0 && dim >= 1, "max_rows must be >= 0 and dim >= 1");
+  HADES_REQUIRE(stride == 0 || stride >= dim, "stride must be 0 or >= dim");
+  HADES_REQUIRE(dim * kRows < (int64_t(1) << 30), "dim too large");
+  HADES_REQUIRE(which == 0 || which == 1, "which must be 0 or 1");
+  if (max_rows == 0) return HADES_OK;
+  HADES_REQUIRE(ukeys && grad && num_unique && class_split && w && s, "null pointer argument");
+  if (stride == 0) stride = dim;
+  AdagradListedArgs a{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
+                      key_mask, dim, w, s, stride, lr, eps};
+  return launch_adagrad_listed(a, stream);
+}
+
+}  // extern "C"
+
+namespace {
+int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
+  float* w = a.w;
+  float* s = a.s;
+  const float* grad = a.grad;
+  const int64_t max_count = a.max_count, dim = a.dim, stride = a.stride;
   int64_t blocks = ceil_div(max_count, kRows);
   if (blocks > 16384) blocks = 16384;
   // rows that cross the host link: a narrow grid that strides over the list
@@ -324,6 +372,9 @@ int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, con
     HADES_LAUNCH((adagrad_listed_kernel<1>), grid, block, 0, st, a);
   return HADES_OK;
 }
+}  // namespace
+
+extern "C" {
 
 int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                       int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,

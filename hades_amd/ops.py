@@ -162,14 +162,21 @@ def split(loc, workspace=None):
     return hot_mask, hot_pos[:nh], cold_pos[:nc]
 
 
-def lookup_split(ids, sorted_hot, num_live=None, workspace=None, out=None):
+def key_bits_for(num_rows):
+    """Bits that hold every id of a table of num_rows rows (at least 1)."""
+    return max(1, int(num_rows - 1).bit_length())
+
+
+def lookup_split(ids, sorted_hot, num_live=None, workspace=None, out=None, sort_keys=None,
+                 key_bits=0):
     """Lookup and hot/cold split in one call, no host synchronisation.
 
     Returns (loc int64[n], hot_pos int64[n], cold_pos int64[n], counts int64[2]): the slot of every
     id in the hot set (or -1), the ascending positions of the hot and of the cold ids (the first
     counts[0] / counts[1] entries are live) and the two counts.  `num_live` (int64[1] on the device)
     limits the batch to its first num_live[0] entries, e.g. the padded output of combine_padded.
-    `out` may bring the four tensors."""
+    `out` may bring the four tensors.  `sort_keys` (int64[n]) receives the class-ordered sort key
+    of every id - the id itself if cold, (1 << key_bits) | slot if hot - for combine_plan_classed."""
     _i64(ids, "ids")
     hp, hn, hi = _hot_args(sorted_hot)
     n, dev = ids.numel(), ids.device
@@ -181,8 +188,12 @@ def lookup_split(ids, sorted_hot, num_live=None, workspace=None, out=None):
            "lookup_split outputs too small")
     nbytes = _lib.query("hades_split_compact_workspace_bytes", n)
     ws = (workspace or _ws(dev, "split")).get(nbytes)
+    if sort_keys is not None:
+        _i64(sort_keys, "sort_keys")
+        _check(sort_keys.numel() >= n, "sort_keys too small")
     _lib.call("hades_lookup_split", _ptr(ids), _opt(num_live), n, hp, hn, hi, _ptr(loc), _NULL, _ptr(hot_pos),
-              _ptr(cold_pos), _ptr(counts), _ptr(ws), ws.numel(), _stream())
+              _ptr(cold_pos), _ptr(counts), _opt(sort_keys), int(key_bits), _ptr(ws), ws.numel(),
+              _stream())
     return loc, hot_pos, cold_pos, counts
 
 
@@ -403,6 +414,59 @@ def combine_apply(plan, grad, mode=COMBINE_FAST, out=None):
     _lib.call("hades_combine_apply", _ptr(grad), plan.n, plan.dim, plan.id_bound, int(mode),
               _ptr(sums), _ptr(cnts), _ptr(plan.num_unique), _ptr(ws), ws.numel(), _stream())
     return plan.uids, sums, cnts, plan.num_unique
+
+
+def combine_plan_classed(keys, dim, key_bits, workspace=None, out=None):
+    """combine_plan over the class-ordered keys that lookup_split(..., sort_keys=, key_bits=) made.
+    The plan also carries class_split (int64[2] on the device): first sorted position and first
+    run of the hot class.  `out` = (ukeys int64[n], num_unique int64[1], class_split int64[2])."""
+    _i64(keys, "keys")
+    n, dev = keys.numel(), keys.device
+    if out is None:
+        out = (torch.empty(n, dtype=torch.int64, device=dev), torch.empty(1, dtype=torch.int64, device=dev),
+               torch.empty(2, dtype=torch.int64, device=dev))
+    ukeys, num_unique, class_split = out
+    workspace = workspace or Workspace(dev)
+    ws = workspace.get(_lib.query("hades_combine_workspace_bytes", n, int(dim)))
+    bound, thr = 1 << (int(key_bits) + 1), 1 << int(key_bits)
+    _lib.call("hades_combine_plan_classed", _ptr(keys), n, int(dim), bound, thr, _ptr(ukeys),
+              _ptr(num_unique), _ptr(class_split), _ptr(ws), ws.numel(), _stream())
+    plan = CombinePlan(n, int(dim), bound, ukeys, num_unique, None, workspace, ws)
+    plan.class_split, plan.key_bits = class_split, int(key_bits)
+    return plan
+
+
+def combine_apply_class(plan, grad, which, mode=COMBINE_FAST, out=None):
+    """Segmented sums and counts of one class of a classed plan: which = 0 the cold runs (rows
+    [0, class_split[1]) of the outputs), 1 the hot runs (the rows after them).  Both calls write
+    into the same `out` = (sums float32[n, D], cnts int64[n])."""
+    _dev(grad, "grad")
+    _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
+    _check(grad.size(0) == plan.n and grad.size(1) == plan.dim, "grad does not match the plan")
+    if out is None:
+        out = (torch.empty((plan.n, plan.dim), dtype=torch.float32, device=grad.device),
+               torch.empty(plan.n, dtype=torch.int64, device=grad.device))
+    sums, cnts = out
+    ws = plan.check_live()
+    _lib.call("hades_combine_apply_class", _ptr(grad), plan.n, plan.dim, plan.id_bound, int(mode),
+              int(which), _ptr(sums), _ptr(cnts), _ptr(plan.num_unique), _ptr(plan.class_split),
+              _ptr(ws), ws.numel(), _stream())
+    return sums, cnts
+
+
+def adagrad_update_class_(plan, sums, which, w, s, lr, eps):
+    """Sparse Adagrad over one class of a classed plan: the table row of run u is
+    plan.uids[u] & (2^key_bits - 1) - the id for the cold class, the slot for the hot class."""
+    _dev(sums, "sums")
+    dim = sums.size(1)
+    for name, t in (("w", w), ("s", s)):
+        _dev_or_pinned(t, name, contiguous=False)
+        _check(t.dtype == torch.float32 and t.dim() == 2 and t.size(1) == dim, "%s: wrong dtype/width" % name)
+    stride = _stride_of(w, dim)
+    _check(_stride_of(s, dim) == stride, "w and s must have the same row stride")
+    _lib.call("hades_adagrad_update_class", _ptr(plan.uids), _ptr(sums), _ptr(plan.num_unique),
+              _ptr(plan.class_split), int(which), (1 << plan.key_bits) - 1, plan.uids.numel(), dim,
+              _ptr(w), _ptr(s), stride, float(lr), float(eps), _stream())
 
 
 def combine(idx, grad, id_bound=0, mode=COMBINE_FAST, workspace=None):

@@ -132,13 +132,17 @@ class _SparseRowOptimizer:
     # positions go through kernels that only touch HBM while the cold positions go through
     # kernels that only touch the host table, on a second stream of the same priority, so the
     # host-link time and the HBM time overlap instead of adding up.
+    # one_stream = True runs the cold class on the caller's stream too (no overlap): the same
+    # kernels one after the other, e.g. to time each of them undisturbed
+    one_stream = False
+
     def _split_state(self):
         if getattr(self, "_cold_stream", None) is None:
             self._cold_stream = torch.cuda.Stream(device=self.device)
             self._split_bufs = {}
             self._split_ws = ops.Workspace(self.device)
             self._cold_done = None
-        return self._cold_stream
+        return torch.cuda.current_stream() if self.one_stream else self._cold_stream
 
     def _split_out(self, key, n):
         bufs = self._split_bufs.get(key)
@@ -223,6 +227,94 @@ class _SparseRowOptimizer:
         if join:
             self.join()
 
+    # ---- the keyed step: one lookup per query serves the gather, the combine and the update ----
+    def forward_keyed(self, ids, out=None, timing=None, bufs=None):
+        """Forward half of a training step on the split schedule.  One lookup gives every query
+        its slot, its class list and a class-ordered sort key; the hot rows are gathered on the
+        current stream and the cold rows on the cold stream; meanwhile the keys are sorted (the
+        id-only half of the combine).  Returns (rows, state) after joining the two streams: the
+        rows are complete, `state` goes to backward_keyed with the gradients."""
+        cold = self._split_state()
+        cur = torch.cuda.current_stream()
+        n = ids.numel()
+        if out is None:
+            out = torch.empty((n, self.dim), dtype=self.hot_w.dtype, device=self.device)
+        kb = ops.key_bits_for(max(self.num_rows, self.hot_ids.numel(), 2))
+        if bufs is None:
+            bufs = self._keyed_bufs(n)
+        loc, hot_pos, cold_pos, counts = ops.lookup_split(
+            ids, self.hot_set, workspace=self._split_ws, out=bufs["split"],
+            sort_keys=bufs["keys"], key_bits=kb)
+        hot_pos, cold_pos = hot_pos[:n], cold_pos[:n]
+        split_done = torch.cuda.Event()
+        split_done.record(cur)
+        cold.wait_event(split_done)
+        with torch.cuda.stream(cold):
+            self._timed(timing, "cold_fetch", cold,
+                        lambda: ops.fetch_listed(self.cold_w, ids, cold_pos, counts[1:2], out))
+            self._cold_done = torch.cuda.Event()
+            self._cold_done.record(cold)
+        if self.hot_ids.numel():
+            self._timed(timing, "hot_fetch", cur,
+                        lambda: ops.fetch_listed(self.hot_w, loc, hot_pos, counts[0:1], out))
+        plan = ops.combine_plan_classed(bufs["keys"][:n], self.dim, kb, workspace=self._ws,
+                                        out=(bufs["ukeys"][:n], bufs["nu"], bufs["class_split"]))
+        self.join()
+        return out, (plan, bufs)
+
+    def _keyed_bufs(self, n):
+        b = getattr(self, "_kbufs", None)
+        if b is None or b["keys"].numel() < n:
+            dev = self.device
+            i64 = lambda k: torch.empty(k, dtype=torch.int64, device=dev)
+            b = {"split": (i64(n), i64(n), i64(n), i64(2)), "keys": i64(n), "ukeys": i64(n),
+                 "nu": i64(1), "class_split": i64(2),
+                 "sums": torch.empty((n, self.dim), dtype=torch.float32, device=dev), "cnts": i64(n)}
+            self._kbufs = b
+        return b
+
+    def backward_keyed(self, state, grad, mode=ops.COMBINE_FAST, timing=None):
+        """Backward half: segmented sums of the cold class, whose update then starts on the cold
+        stream while the hot class is summed and updated on the current stream; joins at the end.
+        Returns (ukeys, sums, cnts, num_unique, class_split): the distinct rows in class order -
+        cold ids ascending, then hot slots ascending with bit key_bits set."""
+        plan, bufs = state
+        cold = self._split_state()
+        cur = torch.cuda.current_stream()
+        n = plan.n
+        out = (bufs["sums"][:n], bufs["cnts"][:n])
+        self._timed(timing, "cold_seg_sum", cur,
+                    lambda: ops.combine_apply_class(plan, grad, 0, mode, out=out))
+        cold_summed = torch.cuda.Event()
+        cold_summed.record(cur)
+        cold.wait_event(cold_summed)
+        with torch.cuda.stream(cold):
+            self._timed(timing, "cold_update", cold, lambda: self._update_keyed(plan, out[0], 0))
+            self._cold_done = torch.cuda.Event()
+            self._cold_done.record(cold)
+        self._timed(timing, "seg_sum", cur,
+                    lambda: ops.combine_apply_class(plan, grad, 1, mode, out=out))
+        if self.hot_ids.numel():
+            self._timed(timing, "hot_update", cur, lambda: self._update_keyed(plan, out[0], 1))
+        self.join()
+        return plan.uids, out[0], out[1], plan.num_unique, plan.class_split
+
+    def _update_keyed(self, plan, sums, which):
+        raise NotImplementedError
+
+    def distinct_ids_of(self, ukeys, num_unique, key_bits=None):
+        """The real ids behind the class-ordered keys of a keyed step (one host synchronisation):
+        cold keys are ids, hot keys name a slot of the hot set."""
+        kb = key_bits if key_bits is not None else ops.key_bits_for(max(self.num_rows, self.hot_ids.numel(), 2))
+        u = int(num_unique.item())
+        if u < 0:
+            raise ops._bound_error()
+        k = ukeys[:u]
+        hot = k >= (1 << kb)
+        ids = k.clone()
+        ids[hot] = self.hot_ids[k[hot] - (1 << kb)]
+        return ids
+
     def step_split(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None):
         """step() on the split schedule."""
         if plan is None:
@@ -269,6 +361,10 @@ class SparseAdagrad(_SparseRowOptimizer):
     def _update_class(self, index, grad, pos, count, hot):
         w, s = (self.hot_w, self.hot_s) if hot else (self.cold_w, self.cold_s)
         ops.adagrad_update_listed_(index, grad, pos, count, w, s, self.lr, self.eps)
+
+    def _update_keyed(self, plan, sums, which):
+        w, s = (self.hot_w, self.hot_s) if which else (self.cold_w, self.cold_s)
+        ops.adagrad_update_class_(plan, sums, which, w, s, self.lr, self.eps)
 
     def update(self, uids, grad, num_unique=None):
         ops.adagrad_update_(uids, grad, self.hot_w, self.hot_s, self.cold_w, self.cold_s,

@@ -198,12 +198,17 @@ int hades_split_compact(const int64_t* loc, int64_t n, uint8_t* hot_mask, int64_
  * over the hot tables in HBM and over the cold tables on the host, on separate streams.
  * num_live (int64[1] on the device, may be NULL) limits the batch to its first num_live[0] entries
  * (the padded output of hades_combine): later entries are in neither list and get no slot.
+ * sort_keys (int64[n], may be NULL) receives a class-ordered sort key per query, for
+ * hades_combine_plan_classed:  cold: the id itself;  hot: (1 << key_bits) | slot.  key_bits must
+ * cover the table's ids (ids < 2^key_bits).  Sorted by this key a batch has its cold ids first, in
+ * id order, then its hot ids in slot order (which is id order too), and the key of a hot run is
+ * its row in the hot tables: one lookup per query serves the gather, the combine and the update.
  * hot_mask may be NULL.  Workspace as hades_split_compact. */
 int hades_lookup_split(const int64_t* q, const int64_t* num_live, int64_t n,
                        const int64_t* sorted_hot, int64_t num_hot,
                        const void* hot_index, int64_t* loc, uint8_t* hot_mask, int64_t* hot_pos,
-                       int64_t* cold_pos, int64_t* counts, void* workspace, size_t workspace_bytes,
-                       void* stream);
+                       int64_t* cold_pos, int64_t* counts, int64_t* sort_keys, int key_bits,
+                       void* workspace, size_t workspace_bytes, void* stream);
 
 /* Three-way form of the same thing from the reference's class table (src/cuda/split.cu:11):
  * masks as hades_split, plus pos[k] = ascending positions of class k (each int64 capacity n) and
@@ -282,6 +287,26 @@ int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bo
                         float* sums, int64_t* cnts, const int64_t* num_unique, void* workspace,
                         size_t workspace_bytes, void* stream);
 
+/* The combine over class-ordered keys (sort_keys of hades_lookup_split), in the same two halves,
+ * with the class border kept on the device so that each class can go its own way:
+ *   plan : as hades_combine_plan over `keys` (all below key_bound); ukeys = ascending distinct
+ *          keys; class_split (int64[2], device) = {first sorted position, first run} whose key is
+ *          >= threshold (= {n, num_unique} if there is none).
+ *   apply: the segmented sums and counts of ONE class: which = 0 the runs below the threshold
+ *          (rows [0, class_split[1]) of sums / cnts), which = 1 the runs at or above it.  The two
+ *          calls together give exactly what hades_combine_apply gives; made one after the other
+ *          they let the update of the first class start while the second class is still summed.
+ * The reference has no such split (it combines once, python/EmbCache/sparse_optim.py:614, and
+ * splits the distinct ids afterwards, :243-259); the arithmetic per id is the same. */
+int hades_combine_plan_classed(const int64_t* keys, int64_t n, int64_t dim, int64_t key_bound,
+                               int64_t threshold, int64_t* ukeys, int64_t* num_unique,
+                               int64_t* class_split, void* workspace, size_t workspace_bytes,
+                               void* stream);
+int hades_combine_apply_class(const float* grad, int64_t n, int64_t dim, int64_t key_bound, int mode,
+                              int which, float* sums, int64_t* cnts, const int64_t* num_unique,
+                              const int64_t* class_split, void* workspace, size_t workspace_bytes,
+                              void* stream);
+
 /* hades_combine with the scratch memory inside the library.  No counterpart in the reference.  It
  * is for callers that cannot allocate device memory or hand over a workspace: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  The call allocates and frees
@@ -329,6 +354,15 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
 int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,
                                 const int64_t* count, int64_t max_count, int64_t dim, float* w,
                                 float* s, int64_t stride, float lr, float eps, void* stream);
+
+/* The same arithmetic over one class of a class-ordered combine: the rows u of (ukeys, grad) in
+ * [0, class_split[1]) for which = 0 or [class_split[1], num_unique[0]) for which = 1; the table row
+ * is ukeys[u] & key_mask (the id for the cold class, the slot for the hot class, whose keys carry
+ * the class bit above key_mask).  No lookup: the keys already name the rows. */
+int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
+                               const int64_t* class_split, int which, int64_t key_mask,
+                               int64_t max_rows, int64_t dim, float* w, float* s, int64_t stride,
+                               float lr, float eps, void* stream);
 
 /* SparseAdam row update, same fusion (python/EmbCache/sparse_optim.py:632-657,681):
  *   step += 1; m = b1*m + (1-b1)*g; v = b2*v + (1-b2)*g*g

@@ -286,6 +286,33 @@ def sparse_adagrad_step_split(cold_w, cold_s, hot_w, hot_s, sorted_hot, uids, g,
     adagrad_listed(uids, g, cold_pos, cold_pos.size, cold_w, cold_s, lr, eps)
 
 
+def class_ordered_keys(q, sorted_hot, key_bits):
+    """Sort key of every query for the keyed step: the id if cold, (1 << key_bits) | slot if hot.
+    Ascending keys = the cold ids in id order, then the hot ids in slot order (= id order)."""
+    q = np.asarray(q, dtype=np.int64)
+    loc = lookup_sorted(q, sorted_hot)
+    return np.where(loc >= 0, (np.int64(1) << np.int64(key_bits)) | loc, q).astype(np.int64)
+
+
+def keyed_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps, key_bits):
+    """One combine + Adagrad step done the keyed way: combine over the class-ordered keys
+    (only_unique_grads arithmetic, python/EmbCache/sparse_optim.py:132-139, on another key), then
+    the cold runs update the cold tables at row = key and the hot runs the hot tables at row =
+    key minus the class bit.  In place.  Must equal combine_sequential on the ids followed by
+    sparse_adagrad_step.  Returns (ukeys, sums, cnts, first hot run)."""
+    keys = class_ordered_keys(q, sorted_hot, key_bits)
+    ukeys, sums, cnts = combine_sequential(keys, grad)
+    thr = np.int64(1) << np.int64(key_bits)
+    split = int(np.searchsorted(ukeys, thr, side="left"))
+    rows = ukeys[:split]
+    w1, s1 = adagrad_rows(cold_w[rows], cold_s[rows], sums[:split], lr, eps)
+    cold_w[rows], cold_s[rows] = w1, s1
+    slots = ukeys[split:] - thr
+    w1, s1 = adagrad_rows(hot_w[slots], hot_s[slots], sums[split:], lr, eps)
+    hot_w[slots], hot_s[slots] = w1, s1
+    return ukeys, sums, cnts, split
+
+
 # ---------------------------------------------------------------------------
 # combine: python/EmbCache/sparse_optim.py:132-157
 # ---------------------------------------------------------------------------

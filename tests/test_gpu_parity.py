@@ -1393,3 +1393,61 @@ def test_index_cache_accepts_host_tensors_like_the_reference(lib):
     ic.reset(torch.from_numpy(ids[:100]))
     model.reset(ids[:100])
     assert ic.get_valid_entries_num() == model.get_valid_entries_num()
+
+
+@pytest.mark.parametrize("N,D,H,n,hot_frac", [
+    (5000, 128, 500, 20_000, 0.9), (5000, 64, 500, 20_000, 1.0), (5000, 64, 500, 20_000, 0.0),
+    (5000, 7, 0, 3000, 0.0), (300, 100, 300, 4097, 1.0),
+    (70_000, 128, 9000, 257, 0.5), (70_000, 128, 9000, 256, 0.5), (70_000, 128, 9000, 1, 0.5),
+    (1_000_000, 32, 100_000, 300_000, 0.9),          # several blocks either side of the class border
+    (10, 4, 3, 0, 0.5),
+])
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_keyed_step_forward_and_backward(lib, N, D, H, n, hot_frac, host_cold):
+    """forward_keyed / backward_keyed (one lookup per query; combine over class-ordered keys; cold
+    class summed and updated first) against the oracle: fetched rows, distinct keys, sums, counts,
+    class border and all four tables bit-exact in the deterministic-order mode; FAST sums within
+    1e-5 per row and the same keys and counts."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad
+    rng = np.random.default_rng(N + n + int(10 * hot_frac) + 1)
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, hot_frac)
+    if n > 1000:
+        q[: n // 4] = q[0]                       # a long run in one class
+    t_cold = torch.from_numpy(cold.copy())
+    t_cold = t_cold.pin_memory() if host_cold else t_cold.cuda()
+    opt = SparseAdagrad(t_cold, torch.from_numpy(hot_ids), lr=0.01, eps=1e-10)
+    opt.hot_w += 1.0
+    hw = opt.hot_w.cpu().numpy().copy()
+    kb = ops.key_bits_for(max(N, H, 2))
+    t_q = dev(q)
+    cw, cs, hs = cold.copy(), np.zeros_like(cold), np.zeros_like(hw)
+    for it in range(2):
+        grad = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+        want_rows = O.cached_fetch(cw, hw, q, hot_ids)
+        rows, state = opt.forward_keyed(t_q)
+        assert np.array_equal(rows.cpu().numpy(), want_rows)
+        if it == 0 and n:
+            # the fast mode on the same plan first (it writes only the outputs, not the tables)
+            plan, bufs = state
+            fs, fc = ops.combine_apply_class(plan, dev(grad), 0, ops.COMBINE_FAST)
+            ops.combine_apply_class(plan, dev(grad), 1, ops.COMBINE_FAST, out=(fs, fc))
+            keys = O.class_ordered_keys(q, hot_ids, kb)
+            wk, _, wc = O.combine_sequential(keys, grad)
+            _, w64, _ = O.combine_float64(keys, grad)
+            U = int(plan.num_unique.item())
+            assert U == wk.size and np.array_equal(plan.uids[:U].cpu().numpy(), wk)
+            assert np.array_equal(fc[:U].cpu().numpy(), wc)
+            assert combine_tol_ok(fs[:U].cpu().numpy(), w64)
+        ukeys, sums, cnts, nu, split = opt.backward_keyed(state, dev(grad), mode=ops.COMBINE_EXACT)
+        torch.cuda.synchronize()
+        wk, ws, wc, wsplit = O.keyed_step(cw, cs, hw, hs, hot_ids, q, grad, 0.01, 1e-10, kb)
+        U = int(nu.item())
+        assert U == wk.size and np.array_equal(ukeys[:U].cpu().numpy(), wk)
+        assert np.array_equal(cnts[:U].cpu().numpy(), wc) and np.array_equal(sums[:U].cpu().numpy(), ws)
+        assert split.tolist() == [int((O.lookup_sorted(q, hot_ids) < 0).sum()), wsplit]
+        if U:
+            ids = opt.distinct_ids_of(ukeys, nu)
+            assert np.array_equal(np.sort(ids.cpu().numpy()), np.unique(q))
+    assert np.array_equal(opt.cold_w.cpu().numpy(), cw) and np.array_equal(opt.cold_s.cpu().numpy(), cs)
+    assert np.array_equal(opt.hot_w.cpu().numpy(), hw) and np.array_equal(opt.hot_s.cpu().numpy(), hs)

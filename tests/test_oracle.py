@@ -612,3 +612,29 @@ def test_split_schedule_equals_the_unsplit_operators():
     O.sparse_adagrad_step_split(b[0], b[1], b[2], b[3], hot_ids, uq, g, 0.01, 1e-10, num_live=1500)
     for x, y in zip(a, b):
         assert np.array_equal(x, y)
+
+
+def test_keyed_step_equals_combine_then_update_on_the_ids():
+    """Sorting by (class, id-or-slot) instead of by id changes the order of the distinct rows and
+    nothing else: same sums per id (same occurrence order inside a run), same tables afterwards."""
+    rng = np.random.default_rng(77)
+    N, D, H, n = 5000, 6, 700, 9000
+    kb = 13
+    cold = rng.standard_normal((N, D)).astype(np.float32)
+    hot_ids = np.sort(rng.choice(N, H, replace=False)).astype(np.int64)
+    q = np.minimum(rng.pareto(0.8, n).astype(np.int64) * 37 % N, N - 1)
+    g = (rng.standard_normal((n, D)) * 1e-2).astype(np.float32)
+    a = [cold.copy(), np.zeros((N, D), np.float32), cold[hot_ids] + 1, np.zeros((H, D), np.float32)]
+    b = [x.copy() for x in a]
+    for _ in range(2):
+        wu, ws, wc = O.combine_sequential(q, g)
+        O.sparse_adagrad_step(a[0], a[1], a[2], a[3], hot_ids, wu, ws, 0.01, 1e-10)
+        ukeys, sums, cnts, split = O.keyed_step(b[0], b[1], b[2], b[3], hot_ids, q, g, 0.01, 1e-10, kb)
+        # the keyed rows are the id rows in another order
+        ids = np.where(ukeys >= (1 << kb), hot_ids[np.maximum(ukeys - (1 << kb), 0) % H], ukeys)
+        order = np.argsort(ids, kind="stable")
+        assert np.array_equal(ids[order], wu) and np.array_equal(sums[order], ws) and np.array_equal(cnts[order], wc)
+        assert np.all(np.diff(ukeys) > 0) and np.all(ukeys[:split] < (1 << kb)) and np.all(ukeys[split:] >= (1 << kb))
+        assert not np.isin(ukeys[:split], hot_ids).any()
+    for x, y in zip(a, b):
+        assert np.array_equal(x, y)
