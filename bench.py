@@ -5,6 +5,7 @@
     python bench.py --workload cfg4          cold-gradient accumulator with delayed write-back
     python bench.py --workload cfg4 --flush-rule staleness    the cache server's own per-row rule
     python bench.py --workload neighbours    pre-exchange bucketing, index cache, cold-data cache
+    python bench.py --workload random-rows   what distinct random 512-byte rows of a 2 GB table cost
 
 One step = lookup + cached_fetch of the query rows, combine of the per-query gradients, and the
 sparse Adagrad update of every distinct row, on one batch of synthetic Zipf ids that is already
@@ -55,7 +56,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours", "random-rows"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
     ap.add_argument("--schedule", default=None, choices=["serial", "keyed", "split", "overlap", "graph"],
                     help="serial: every kernel of the step on one stream, hot and cold rows in the "
@@ -965,6 +966,61 @@ def run_neighbours(args):
     print(json.dumps(line))
 
 
+def run_random_rows(args):
+    """The ceiling of the access pattern itself: rows that are distinct, random and 512 bytes
+    long, in tables of 4 M rows (2.1 GB, the size of the cold-gradient accumulator), moved by the
+    plain listed gather, the listed scatter and the listed Adagrad update.  No row is touched
+    twice and no two rows share a DRAM page, so neither L2 nor the memory-side cache helps: this
+    is what the segmented sum (gradient rows in sort order) and the accumulator (slot rows) can
+    reach at best.  Prints its own JSON line."""
+    import torch
+    from hades_amd import ops
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    S, D, U = 4_194_304, 128, 353_000
+    g = torch.Generator().manual_seed(3)
+    slots = torch.randperm(S, generator=g)[:U].to(dev)
+    pos = torch.arange(U, device=dev)
+    cnt = torch.tensor([U], device=dev)
+    grad = torch.randn((U, D), device=dev) * 1e-3
+    w = torch.zeros((S, D), device=dev)
+    st = torch.zeros((S, D), device=dev)
+    out = torch.empty((U, D), device=dev)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        tot = 0.0
+        for _ in range(args.steps):
+            ev[0].record(); fn(); ev[1].record()
+            torch.cuda.synchronize()
+            tot += ev[0].elapsed_time(ev[1])
+        return tot / args.steps
+
+    res = {}
+    for name, fn, nbytes in (
+            ("gather (hades_fetch_listed)", lambda: ops.fetch_listed(w, slots, pos, cnt, out), U * (16 + 8 * D)),
+            ("scatter (hades_set_listed)", lambda: ops.set_listed(grad, w, slots, pos, cnt), U * (16 + 8 * D)),
+            ("Adagrad (hades_adagrad_update_listed)",
+             lambda: ops.adagrad_update_listed_(slots, grad, pos, cnt, w, st, 0.01, 1e-10), U * (16 + 20 * D))):
+        ms = timed(fn)
+        res[name] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
+                     "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        log("%s: %.1f us" % (name, ms * 1e3))
+    a = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
+    b = torch.empty_like(a)
+    ms = timed(lambda: b.copy_(a))
+    res["plain 256 MiB device copy (torch)"] = {"us": round(ms * 1e3, 1), "GB/s": round(2 * a.numel() * 4 / ms / 1e6, 1),
+                                                "frac_hbm": round(2 * a.numel() * 4 / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    print(json.dumps({"metric": "distinct random 512-byte rows of a 2.1 GB table, GB/s of algorithmic bytes",
+                      "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                      "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": "%d distinct random rows of %d x %d fp32 tables" % (U, S, D)},
+                      "operators": res}))
+
+
 def run_cpu_baseline(wl_name, seconds):
     """The same step with the CPU oracle (torch CPU ops, all host threads), on a bounded sample:
     the benchmark's own batches at full table size when that fits the host, repeated for about
@@ -1018,6 +1074,9 @@ def main():
         return
     if args.workload == "neighbours":
         run_neighbours(args)
+        return
+    if args.workload == "random-rows":
+        run_random_rows(args)
         return
     res = run_gpu(args, args.workload, args.schedule)
     ms_per_step = res.pop("ms_per_step")

@@ -69,7 +69,11 @@ __global__ __launch_bounds__(kThreads) void hash_accumulate_kernel(AccArgs a) {
     // bounded probe: every wave leaves the loop after at most num_slots steps
     for (int64_t probe = 0; id >= 0 && probe < a.num_slots; ++probe) {
       unsigned long long* kp = reinterpret_cast<unsigned long long*>(a.keys + h);
-      int64_t k = static_cast<int64_t>(__hip_atomic_load(kp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      // A plain load is enough to look: a key, once stored, stays until the flush, so a
+      // non-empty value is never stale in a harmful way, and a stale "empty" only sends the
+      // thread to the compare-and-swap below, which is the arbiter (device-scope atomics are
+      // executed beyond the per-XCD L2 and cost a round trip of their own).
+      int64_t k = a.keys[h];
       if (k == kEmpty) {
         k = static_cast<int64_t>(atomicCAS(kp, static_cast<unsigned long long>(kEmpty),
                                            static_cast<unsigned long long>(id)));
@@ -104,7 +108,9 @@ __global__ __launch_bounds__(kThreads) void hash_accumulate_kernel(AccArgs a) {
         const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
         if (s_slot[r] >= 0) {
           sp[k] = reinterpret_cast<V*>(a.accum + s_slot[r] * a.dim + col);
-          g[k] = *reinterpret_cast<const V*>(a.grad + (row0 + r) * a.dim + col);
+          // gradient rows are read exactly once: keep them from displacing table rows in L2
+          g[k] = __builtin_nontemporal_load(
+              reinterpret_cast<const V*>(a.grad + (row0 + r) * a.dim + col));
           s[k] = *sp[k];
         }
       }
