@@ -104,16 +104,32 @@ __global__ __launch_bounds__(kGroup * kThreads) void radix_count_kernel(
   const int64_t tile = static_cast<int64_t>(blockIdx.x) * kGroup + g;
   const int64_t tile0 = tile * (kThreads * IPT);
   bool bad = false;
+  const int lane = t & (kWave - 1);
 #pragma unroll
   for (int r = 0; r < IPT; ++r) {
     const int64_t i = tile0 + r * kThreads + t;
-    if (i < n) {
+    const bool valid = i < n;
+    uint32_t d = 0;
+    if (valid) {
       if (FIRST) {
         const int64_t id = static_cast<const int64_t*>(keys_in)[i];
         bad = bad || (id_bound > 0 && (id < 0 || id >= id_bound));
       }
       const KeyT k = load_key<KeyT, FIRST>(keys_in, i);
-      atomicAdd(&s_hist[g][static_cast<uint32_t>(k >> shift) & mask], 1u);
+      d = static_cast<uint32_t>(k >> shift) & mask;
+    }
+    // After the first pass equal keys sit next to each other, and 64 lanes adding to one LDS
+    // counter are served one after the other (the counters showed bank-conflict cycles at 7-9
+    // times the useful LDS cycles).  Lanes with the digit of their left neighbour stay silent;
+    // the first lane of every stretch adds the length of the stretch.
+    const uint32_t left = __shfl_up(d, 1);
+    const bool head = valid && (lane == 0 || left != d);
+    const uint64_t heads = __ballot(head);
+    const uint64_t live = __ballot(valid);          // the valid lanes form a prefix of the wave
+    if (head) {
+      const uint64_t above = lane == kWave - 1 ? 0 : heads >> (lane + 1);
+      const int next = above ? lane + 1 + __builtin_ctzll(above) : __popcll(live);
+      atomicAdd(&s_hist[g][d], static_cast<uint32_t>(next - lane));
     }
   }
   // the first pass also checks the promise 0 <= id < id_bound: one flag per block, written by
