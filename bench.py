@@ -198,6 +198,50 @@ def link_probe(dev, nbytes=256 << 20, reps=4):
     return out
 
 
+def link_kernel_probe(wl, reps=3):
+    """What the host link gives kernels on this box for the workload's own cold rows (batch 0):
+    the listed gather alone (host -> HBM), the listed scatter alone (HBM -> host; it writes back
+    the rows just read, so the table does not change), and both at once on two streams."""
+    import torch
+    from hades_amd import ops
+    opt = wl.opt
+    q = wl.ids[0]
+    loc, hot_pos, cold_pos, counts = ops.lookup_split(q, opt.hot_set)
+    n_cold = int(counts[1].item())
+    cnt = counts[1:2]
+    rows = wl.rows_out
+    ops.fetch_listed(opt.cold_w, q, cold_pos, cnt, rows)
+    src = rows.clone()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    mb = n_cold * wl.D * 4 / 1e6
+
+    def gather():
+        with torch.cuda.stream(s1):
+            ops.fetch_listed(opt.cold_w, q, cold_pos, cnt, rows)
+
+    def scatter():
+        with torch.cuda.stream(s2):
+            ops.set_listed(src, opt.cold_w, q, cold_pos, cnt)
+
+    def rate(fns):
+        best = 0.0
+        for _ in range(reps + 1):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for f in fns:
+                f()
+            torch.cuda.synchronize()
+            best = max(best, mb / ((time.perf_counter() - t0) * 1e3))
+        return round(best, 2)
+
+    out = {"rows": n_cold, "gather_GB/s": rate([gather]), "scatter_GB/s": rate([scatter]),
+           "both_ways_each_GB/s": rate([gather, scatter]),
+           "note": "listed gather / scatter kernels over the cold rows of batch 0, wall clock "
+                   "around one call (launch latency included), best of %d" % (reps + 1)}
+    del src
+    return out
+
+
 def parity_gate(wl, step_fn, rows=20_000):
     """One untimed step in the deterministic-order mode on the first `rows` ids of batch 0,
     through the same schedule as the timed steps, checked against torch's own device operators:
@@ -356,6 +400,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
         log("parity gate passed: %s" % json.dumps(gate["max_rel_err"]))
     link = link_probe(dev) if (with_link and wl.host_cold) else None
     if link:
+        link["kernels"] = link_kernel_probe(wl)
         log("host link: %s" % json.dumps(link))
 
     for i in range(args.warmup):
@@ -617,6 +662,9 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
             f["frac_memcpy_h2d"] = round(f_gbs / link["h2d_GB/s"], 4)
             u["frac_memcpy_h2d"] = round(u_gbs / link["h2d_GB/s"], 4)
             u["frac_memcpy_both_ways"] = round(u_gbs / link["both_ways_each_GB/s"], 4)
+            if "kernels" in link:
+                u["frac_kernel_probe_both_ways"] = round(u_gbs / link["kernels"]["both_ways_each_GB/s"], 4)
+                f["frac_kernel_probe_gather"] = round(f_gbs / link["kernels"]["gather_GB/s"], 4)
         pcie["fetch_host_to_device"] = f
         pcie["update_each_way_at_once"] = u
         pcie["achieved"] = round(min(f_gbs, u_gbs), 2)
