@@ -68,6 +68,10 @@ def parse_args():
                          "ids; overlap: serial with the sort of "
                          "the ids on a side stream next to the fetch; graph: serial, every step the "
                          "replay of a HIP graph captured once per batch")
+    ap.add_argument("--reuse-rows", action="store_true",
+                    help="keyed schedule only: the cold update takes the old weight rows from the "
+                         "rows the step's own fetch brought in instead of reading the host table "
+                         "again (valid with one batch in flight per table)")
     ap.add_argument("--flush-rule", default="every8", choices=["every8", "staleness"],
                     help="cfg4 only: write the accumulated cold gradients back every 8 steps (hash "
                          "accumulator), or per row by the cache server's staleness rule (cold-data "
@@ -308,7 +312,7 @@ def parity_gate(wl, step_fn, rows=20_000):
                        "Adagrad closed form)"}
 
 
-def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
+def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows=False):
     import torch
     from hades_amd import ops
     dev = torch.device("cuda:0")
@@ -356,7 +360,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
             _, state = opt.forward_keyed(q, out=rows, timing=timing)
             if events: events[1].record()
             if events: events[2].record()
-            res = opt.backward_keyed(state, g, cmode, timing=timing)
+            res = opt.backward_keyed(state, g, cmode, timing=timing,
+                                     fetched_rows=rows if reuse_rows else None)
         elif split:
             opt.fetch_split(q, out=rows, join=False, timing=timing)
             plan = ops.combine_plan(q, D, id_bound=N, workspace=opt._ws, out=out_ids)
@@ -666,11 +671,18 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True):
                 u["frac_kernel_probe_both_ways"] = round(u_gbs / link["kernels"]["both_ways_each_GB/s"], 4)
                 f["frac_kernel_probe_gather"] = round(f_gbs / link["kernels"]["gather_GB/s"], 4)
         pcie["fetch_host_to_device"] = f
-        pcie["update_each_way_at_once"] = u
+        if reuse_rows and keyed:
+            pcie["update_device_to_host_only"] = u
+            pcie["update_note"] = ("the cold update takes the old weights from the rows this step's "
+                                   "fetch brought in: it only writes over the link")
+        else:
+            pcie["update_each_way_at_once"] = u
         pcie["achieved"] = round(min(f_gbs, u_gbs), 2)
         pcie["frac"] = round(min(f_gbs, u_gbs) / PCIE_PEAK_GBS, 4)
-        pcie["note"] = ("%s; the update reads and writes the cold weight rows (4D bytes each way "
-                        "per distinct cold row); achieved/frac = the lower of the two" % timing_note)
+        pcie["note"] = ("%s; %s; achieved/frac = the lower of the two" % (
+            timing_note, "the update only writes the cold weight rows (4D bytes per distinct cold row)"
+            if (reuse_rows and keyed) else
+            "the update reads and writes the cold weight rows (4D bytes each way per distinct cold row)"))
         res["pcie"] = pcie
     del wl, opt
     torch.cuda.empty_cache()
@@ -1126,7 +1138,7 @@ def main():
     if args.workload == "random-rows":
         run_random_rows(args)
         return
-    res = run_gpu(args, args.workload, args.schedule)
+    res = run_gpu(args, args.workload, args.schedule, reuse_rows=args.reuse_rows)
     ms_per_step = res.pop("ms_per_step")
     n = res.pop("n")
     schedule = res.pop("schedule")
@@ -1143,7 +1155,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": res.pop("workload"), "combine_mode": args.mode,
+        "config": {"workload": res.pop("workload") + (
+                       "; cold update reuses the rows fetched by the same step" if args.reuse_rows else ""),
+                   "combine_mode": args.mode,
                    "optimizer": "sparse Adagrad lr=0.01 eps=1e-10",
                    "schedule": {"serial": "one stream, hot and cold rows in the same kernels",
                                 "split": "lookup + hot/cold partition; hot rows on the main stream, "
@@ -1166,6 +1180,19 @@ def main():
             "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
             "step_us": sec["step_us"], "step_frac_hbm": sec["step_frac_hbm"],
             "roofline": sec["roofline"], "kernels": sec["kernels"], "phases": sec["phases"]}}
+        if schedule == "keyed" and not args.reuse_rows:
+            log("secondary: cfg3 again with the cold update reusing the fetched rows")
+            sec = run_gpu(args, "cfg3", "keyed", with_gate=True, with_link=False, reuse_rows=True)
+            line["secondary"]["cfg3_reuse_fetched_rows"] = {
+                "what": "the headline workload and schedule, but the cold update takes the old weight "
+                        "rows from the rows the step's own fetch brought in instead of reading the "
+                        "host table a second time (bit-identical results; valid with one batch in "
+                        "flight per table; opt-in: backward_keyed(fetched_rows=...))",
+                "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
+                "step_us": sec["step_us"], "phases": sec["phases"], "pcie": sec["pcie"],
+                "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
+                            for k, v in sec["kernels"].items()},
+                "parity_gate": sec["parity_gate"]}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = run_cpu_baseline(args.workload, args.cpu_seconds)
     print(json.dumps(line))

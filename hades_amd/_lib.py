@@ -59,9 +59,9 @@ _SIGNATURES = {
     "hades_cached_fetch_loc": [_P, _P, _P, _P, _L, _P, _L, c_int, _P],
     "hades_cached_set": [_P, _P, _P, _P, _L, _P, _L, _P, _L, c_int, _P],
     "hades_combine": [_P, _P, _L, _L, _L, c_int, _P, _P, _P, _P, _P, _P, c_size_t, _P],
-    "hades_combine_plan_classed": [_P, _L, _L, _L, _L, _P, _P, _P, _P, c_size_t, _P],
+    "hades_combine_plan_classed": [_P, _L, _L, _L, _L, _P, _P, _P, _P, _P, c_size_t, _P],
     "hades_combine_apply_class": [_P, _L, _L, _L, c_int, c_int, _P, _P, _P, _P, _P, c_size_t, _P],
-    "hades_adagrad_update_class": [_P, _P, _P, _P, c_int, _L, _L, _L, _P, _P, _L, c_float, c_float, _P],
+    "hades_adagrad_update_class": [_P, _P, _P, _P, c_int, _L, _L, _L, _P, _P, _L, _P, _P, c_float, c_float, _P],
     "hades_combine_static": [_P, _P, _L, _L, _L, c_int, _P, _P, _P, _P, _P, _P],
     "hades_combine_plan": [_P, _L, _L, _L, _P, _P, _P, _P, c_size_t, _P],
     "hades_combine_apply": [_P, _L, _L, _L, c_int, _P, _P, _P, _P, c_size_t, _P],

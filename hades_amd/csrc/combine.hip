@@ -328,7 +328,8 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
     const uint32_t* __restrict__ blk_cnt, int64_t* __restrict__ uids,
     uint32_t* __restrict__ seg_start, uint32_t* __restrict__ seg_of,
     int64_t* __restrict__ num_unique, int32_t* __restrict__ inverse,
-    const int32_t* __restrict__ bad_blk, int64_t nbad, KeyT thr, int64_t* __restrict__ class_split) {
+    const int32_t* __restrict__ bad_blk, int64_t nbad, KeyT thr, int64_t* __restrict__ class_split,
+    int32_t* __restrict__ first_pos) {
   __shared__ uint32_t smem[kWaves + 1];
   // the block that writes num_unique first learns whether the first count pass saw an id outside
   // [0, id_bound): it then reports -1 distinct ids, which every consumer treats as "no live rows"
@@ -377,6 +378,7 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
         if (flag[k]) {
           uids[seg] = id_from_key<KeyT>(kk[k]);
           seg_start[seg] = static_cast<uint32_t>(j);
+          if (first_pos != nullptr) first_pos[seg] = static_cast<int32_t>(perm[j]);
           // the first key at or above the threshold opens the upper class (keys are ascending)
           if (class_split != nullptr && kk[k] >= thr &&
               (j == 0 || (k > 0 ? kk[k - 1] : keys[j - 1]) < thr)) {
@@ -949,14 +951,14 @@ int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, con
 template <typename KeyT>
 int run_runs(const void* sorted_keys, const uint32_t* perm, int64_t n, const Plan& p, const Ws& w,
              int64_t* uids, int64_t* num_unique, int32_t* inverse, hipStream_t st,
-             int64_t threshold = 0, int64_t* class_split = nullptr) {
+             int64_t threshold = 0, int64_t* class_split = nullptr, int32_t* first_pos = nullptr) {
   const KeyT* keys = static_cast<const KeyT*>(sorted_keys);
   const dim3 rgrid(static_cast<unsigned>(p.nblocks_runs)), block(kThreads);
   HADES_LAUNCH((run_count_kernel<KeyT>), rgrid, block, 0, st, keys, n, w.run_cnt);
   HADES_LAUNCH_CHECK();
   HADES_LAUNCH((run_emit_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt, uids,
                      w.seg_start, w.seg_of, num_unique, inverse, w.sort.bad, w.sort.nbad,
-                     key_from_id<KeyT>(threshold), class_split);
+                     key_from_id<KeyT>(threshold), class_split, first_pos);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }
@@ -1010,7 +1012,7 @@ __global__ void set_i64x2_kernel(int64_t* p, int64_t a, int64_t b) {
 int combine_plan_impl(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bound, int64_t* uids,
                       int64_t* num_unique, int32_t* inverse, void* workspace,
                       size_t workspace_bytes, void* stream, int64_t threshold,
-                      int64_t* class_split) {
+                      int64_t* class_split, int32_t* first_pos) {
   HADES_REQUIRE(n >= 0 && dim >= 1, "n must be >= 0 and dim >= 1");
   HADES_REQUIRE(n < (int64_t(1) << 30), "combine: n must be below 2^30 (got %lld)", (long long)n);
   HADES_REQUIRE(id_bound >= 0, "id_bound must be >= 0");
@@ -1036,9 +1038,9 @@ int combine_plan_impl(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bou
                    : run_sort<uint32_t>(idx, n, id_bound, p, w.sort, st, &sorted_keys, &perm);
   if (rc != HADES_OK) return rc;
   return p.key64 ? run_runs<uint64_t>(sorted_keys, perm, n, p, w, uids, num_unique, inverse, st,
-                                      threshold, class_split)
+                                      threshold, class_split, first_pos)
                  : run_runs<uint32_t>(sorted_keys, perm, n, p, w, uids, num_unique, inverse, st,
-                                      threshold, class_split);
+                                      threshold, class_split, first_pos);
 }
 
 }  // namespace
@@ -1047,18 +1049,18 @@ int hades_combine_plan(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bo
                        int64_t* num_unique, int32_t* inverse, void* workspace,
                        size_t workspace_bytes, void* stream) {
   return combine_plan_impl(idx, n, dim, id_bound, uids, num_unique, inverse, workspace,
-                           workspace_bytes, stream, 0, nullptr);
+                           workspace_bytes, stream, 0, nullptr, nullptr);
 }
 
 int hades_combine_plan_classed(const int64_t* keys, int64_t n, int64_t dim, int64_t key_bound,
                                int64_t threshold, int64_t* ukeys, int64_t* num_unique,
-                               int64_t* class_split, void* workspace, size_t workspace_bytes,
-                               void* stream) {
+                               int64_t* class_split, int32_t* first_pos, void* workspace,
+                               size_t workspace_bytes, void* stream) {
   HADES_REQUIRE(class_split != nullptr, "class_split must not be null");
   HADES_REQUIRE(key_bound > 0 && threshold >= 0 && threshold <= key_bound,
                 "key_bound must be > 0 and threshold in [0, key_bound]");
   return combine_plan_impl(keys, n, dim, key_bound, ukeys, num_unique, nullptr, workspace,
-                           workspace_bytes, stream, threshold, class_split);
+                           workspace_bytes, stream, threshold, class_split, first_pos);
 }
 
 namespace {

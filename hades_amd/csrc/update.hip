@@ -139,6 +139,10 @@ struct AdagradListedArgs {
   const int64_t* class_split;
   int which;
   int64_t index_mask;       // table row = row_index[p] & index_mask
+  // optional: the old weight row of position p is row first_pos[p] of w_rows (rows fetched from
+  // the same table earlier and still valid) instead of being read from the table again
+  const float* w_rows;
+  const int32_t* first_pos;
   int64_t dim;
   float* w;
   float* s;
@@ -151,6 +155,7 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
   typedef typename Vf<VEC>::type V;
   __shared__ int64_t s_row[kRows];    // element offset of the row in w and s
   __shared__ int64_t s_grad[kRows];   // element offset of the row in grad
+  __shared__ int64_t s_old[kRows];    // element offset of the old weight row in w_rows
   int64_t first = 0, cnt;
   if (a.list != nullptr) {
     cnt = a.count[0];
@@ -173,6 +178,7 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
       const int64_t p = a.list != nullptr ? a.list[row0 + r] : row0 + r;
       s_row[r] = (a.row_index[p] & a.index_mask) * a.stride;
       s_grad[r] = p * a.dim;
+      if (a.w_rows != nullptr) s_old[r] = static_cast<int64_t>(a.first_pos[p]) * a.dim;
     }
     __syncthreads();
     const int total = rows_here * cpr;
@@ -190,7 +196,7 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
           wp[k] = reinterpret_cast<V*>(a.w + s_row[r] + col);
           g[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(a.grad + s_grad[r] + col));
           s[k] = *sp[k];
-          w[k] = *wp[k];
+          w[k] = a.w_rows != nullptr ? *reinterpret_cast<const V*>(a.w_rows + s_old[r] + col) : *wp[k];
         }
       }
 #pragma unroll
@@ -331,23 +337,25 @@ int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, con
   HADES_REQUIRE(row_index && grad && list && count && w && s, "null pointer argument");
   if (stride == 0) stride = dim;
   AdagradListedArgs a{row_index, grad, list, count, max_count, nullptr, nullptr, 0, int64_t(-1),
-                      dim, w, s, stride, lr, eps};
+                      nullptr, nullptr, dim, w, s, stride, lr, eps};
   return launch_adagrad_listed(a, stream);
 }
 
 int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
                                const int64_t* class_split, int which, int64_t key_mask,
                                int64_t max_rows, int64_t dim, float* w, float* s, int64_t stride,
-                               float lr, float eps, void* stream) {
+                               const float* w_rows, const int32_t* first_pos, float lr, float eps,
+                               void* stream) {
   HADES_REQUIRE(max_rows >= 0 && dim >= 1, "max_rows must be >= 0 and dim >= 1");
   HADES_REQUIRE(stride == 0 || stride >= dim, "stride must be 0 or >= dim");
   HADES_REQUIRE(dim * kRows < (int64_t(1) << 30), "dim too large");
   HADES_REQUIRE(which == 0 || which == 1, "which must be 0 or 1");
   if (max_rows == 0) return HADES_OK;
   HADES_REQUIRE(ukeys && grad && num_unique && class_split && w && s, "null pointer argument");
+  HADES_REQUIRE((w_rows == nullptr) == (first_pos == nullptr), "w_rows and first_pos go together");
   if (stride == 0) stride = dim;
   AdagradListedArgs a{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
-                      key_mask, dim, w, s, stride, lr, eps};
+                      key_mask, w_rows, first_pos, dim, w, s, stride, lr, eps};
   return launch_adagrad_listed(a, stream);
 }
 
@@ -366,7 +374,7 @@ int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
     blocks = host_link_blocks(true);
   const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dim % 4 == 0 && stride % 4 == 0 && aligned16({grad, w, s}))
+  if (dim % 4 == 0 && stride % 4 == 0 && aligned16({grad, w, s, a.w_rows}))
     HADES_LAUNCH((adagrad_listed_kernel<4>), grid, block, 0, st, a);
   else
     HADES_LAUNCH((adagrad_listed_kernel<1>), grid, block, 0, st, a);

@@ -416,10 +416,12 @@ def combine_apply(plan, grad, mode=COMBINE_FAST, out=None):
     return plan.uids, sums, cnts, plan.num_unique
 
 
-def combine_plan_classed(keys, dim, key_bits, workspace=None, out=None):
+def combine_plan_classed(keys, dim, key_bits, workspace=None, out=None, first_pos=None):
     """combine_plan over the class-ordered keys that lookup_split(..., sort_keys=, key_bits=) made.
     The plan also carries class_split (int64[2] on the device): first sorted position and first
-    run of the hot class.  `out` = (ukeys int64[n], num_unique int64[1], class_split int64[2])."""
+    run of the hot class.  `out` = (ukeys int64[n], num_unique int64[1], class_split int64[2]).
+    `first_pos` (int32[n]) receives the batch position of the first occurrence of every distinct
+    key (plan.first_pos)."""
     _i64(keys, "keys")
     n, dev = keys.numel(), keys.device
     if out is None:
@@ -429,10 +431,13 @@ def combine_plan_classed(keys, dim, key_bits, workspace=None, out=None):
     workspace = workspace or Workspace(dev)
     ws = workspace.get(_lib.query("hades_combine_workspace_bytes", n, int(dim)))
     bound, thr = 1 << (int(key_bits) + 1), 1 << int(key_bits)
+    if first_pos is not None:
+        _check(first_pos.dtype == torch.int32 and first_pos.is_cuda and first_pos.numel() >= n,
+               "first_pos must be an int32 device tensor of n entries")
     _lib.call("hades_combine_plan_classed", _ptr(keys), n, int(dim), bound, thr, _ptr(ukeys),
-              _ptr(num_unique), _ptr(class_split), _ptr(ws), ws.numel(), _stream())
+              _ptr(num_unique), _ptr(class_split), _opt(first_pos), _ptr(ws), ws.numel(), _stream())
     plan = CombinePlan(n, int(dim), bound, ukeys, num_unique, None, workspace, ws)
-    plan.class_split, plan.key_bits = class_split, int(key_bits)
+    plan.class_split, plan.key_bits, plan.first_pos = class_split, int(key_bits), first_pos
     return plan
 
 
@@ -454,9 +459,12 @@ def combine_apply_class(plan, grad, which, mode=COMBINE_FAST, out=None):
     return sums, cnts
 
 
-def adagrad_update_class_(plan, sums, which, w, s, lr, eps):
+def adagrad_update_class_(plan, sums, which, w, s, lr, eps, fetched_rows=None):
     """Sparse Adagrad over one class of a classed plan: the table row of run u is
-    plan.uids[u] & (2^key_bits - 1) - the id for the cold class, the slot for the hot class."""
+    plan.uids[u] & (2^key_bits - 1) - the id for the cold class, the slot for the hot class.
+    `fetched_rows` (float32[n, D], the rows the forward pass fetched for this batch) makes the
+    kernel take the old weight rows from there (row plan.first_pos[u]) instead of reading the
+    table again; valid only while nothing has written those table rows since the fetch."""
     _dev(sums, "sums")
     dim = sums.size(1)
     for name, t in (("w", w), ("s", s)):
@@ -464,9 +472,16 @@ def adagrad_update_class_(plan, sums, which, w, s, lr, eps):
         _check(t.dtype == torch.float32 and t.dim() == 2 and t.size(1) == dim, "%s: wrong dtype/width" % name)
     stride = _stride_of(w, dim)
     _check(_stride_of(s, dim) == stride, "w and s must have the same row stride")
+    fp = None
+    if fetched_rows is not None:
+        _dev(fetched_rows, "fetched_rows")
+        _check(plan.first_pos is not None, "the plan was made without first_pos")
+        _check(fetched_rows.dtype == torch.float32 and tuple(fetched_rows.shape) == (plan.n, dim),
+               "fetched_rows must be float32 [n, dim]")
+        fp = plan.first_pos
     _lib.call("hades_adagrad_update_class", _ptr(plan.uids), _ptr(sums), _ptr(plan.num_unique),
               _ptr(plan.class_split), int(which), (1 << plan.key_bits) - 1, plan.uids.numel(), dim,
-              _ptr(w), _ptr(s), stride, float(lr), float(eps), _stream())
+              _ptr(w), _ptr(s), stride, _opt(fetched_rows), _opt(fp), float(lr), float(eps), _stream())
 
 
 def combine(idx, grad, id_bound=0, mode=COMBINE_FAST, workspace=None):

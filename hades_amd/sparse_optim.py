@@ -258,7 +258,8 @@ class _SparseRowOptimizer:
             self._timed(timing, "hot_fetch", cur,
                         lambda: ops.fetch_listed(self.hot_w, loc, hot_pos, counts[0:1], out))
         plan = ops.combine_plan_classed(bufs["keys"][:n], self.dim, kb, workspace=self._ws,
-                                        out=(bufs["ukeys"][:n], bufs["nu"], bufs["class_split"]))
+                                        out=(bufs["ukeys"][:n], bufs["nu"], bufs["class_split"]),
+                                        first_pos=bufs["first_pos"][:n])
         self.join()
         return out, (plan, bufs)
 
@@ -269,15 +270,21 @@ class _SparseRowOptimizer:
             i64 = lambda k: torch.empty(k, dtype=torch.int64, device=dev)
             b = {"split": (i64(n), i64(n), i64(n), i64(2)), "keys": i64(n), "ukeys": i64(n),
                  "nu": i64(1), "class_split": i64(2),
+                 "first_pos": torch.empty(n, dtype=torch.int32, device=dev),
                  "sums": torch.empty((n, self.dim), dtype=torch.float32, device=dev), "cnts": i64(n)}
             self._kbufs = b
         return b
 
-    def backward_keyed(self, state, grad, mode=ops.COMBINE_FAST, timing=None):
+    def backward_keyed(self, state, grad, mode=ops.COMBINE_FAST, timing=None, fetched_rows=None):
         """Backward half: segmented sums of the cold class, whose update then starts on the cold
         stream while the hot class is summed and updated on the current stream; joins at the end.
         Returns (ukeys, sums, cnts, num_unique, class_split): the distinct rows in class order -
-        cold ids ascending, then hot slots ascending with bit key_bits set."""
+        cold ids ascending, then hot slots ascending with bit key_bits set.
+
+        `fetched_rows` = the rows forward_keyed returned for this batch: the cold update then takes
+        the old weights from them instead of reading the cold table a second time (half the
+        host-link traffic of the update).  The caller vouches that nothing has written the table
+        since that forward pass - true for a trainer with one batch in flight."""
         plan, bufs = state
         cold = self._split_state()
         cur = torch.cuda.current_stream()
@@ -289,7 +296,8 @@ class _SparseRowOptimizer:
         cold_summed.record(cur)
         cold.wait_event(cold_summed)
         with torch.cuda.stream(cold):
-            self._timed(timing, "cold_update", cold, lambda: self._update_keyed(plan, out[0], 0))
+            self._timed(timing, "cold_update", cold,
+                        lambda: self._update_keyed(plan, out[0], 0, fetched_rows))
             self._cold_done = torch.cuda.Event()
             self._cold_done.record(cold)
         self._timed(timing, "seg_sum", cur,
@@ -299,7 +307,7 @@ class _SparseRowOptimizer:
         self.join()
         return plan.uids, out[0], out[1], plan.num_unique, plan.class_split
 
-    def _update_keyed(self, plan, sums, which):
+    def _update_keyed(self, plan, sums, which, fetched_rows=None):
         raise NotImplementedError
 
     def distinct_ids_of(self, ukeys, num_unique, key_bits=None):
@@ -362,9 +370,9 @@ class SparseAdagrad(_SparseRowOptimizer):
         w, s = (self.hot_w, self.hot_s) if hot else (self.cold_w, self.cold_s)
         ops.adagrad_update_listed_(index, grad, pos, count, w, s, self.lr, self.eps)
 
-    def _update_keyed(self, plan, sums, which):
+    def _update_keyed(self, plan, sums, which, fetched_rows=None):
         w, s = (self.hot_w, self.hot_s) if which else (self.cold_w, self.cold_s)
-        ops.adagrad_update_class_(plan, sums, which, w, s, self.lr, self.eps)
+        ops.adagrad_update_class_(plan, sums, which, w, s, self.lr, self.eps, fetched_rows=fetched_rows)
 
     def update(self, uids, grad, num_unique=None):
         ops.adagrad_update_(uids, grad, self.hot_w, self.hot_s, self.cold_w, self.cold_s,

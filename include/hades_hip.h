@@ -291,7 +291,8 @@ int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bo
  * with the class border kept on the device so that each class can go its own way:
  *   plan : as hades_combine_plan over `keys` (all below key_bound); ukeys = ascending distinct
  *          keys; class_split (int64[2], device) = {first sorted position, first run} whose key is
- *          >= threshold (= {n, num_unique} if there is none).
+ *          >= threshold (= {n, num_unique} if there is none); first_pos (int32[n], may be NULL):
+ *          the batch position of the first occurrence of every distinct key.
  *   apply: the segmented sums and counts of ONE class: which = 0 the runs below the threshold
  *          (rows [0, class_split[1]) of sums / cnts), which = 1 the runs at or above it.  The two
  *          calls together give exactly what hades_combine_apply gives; made one after the other
@@ -300,8 +301,8 @@ int hades_combine_apply(const float* grad, int64_t n, int64_t dim, int64_t id_bo
  * splits the distinct ids afterwards, :243-259); the arithmetic per id is the same. */
 int hades_combine_plan_classed(const int64_t* keys, int64_t n, int64_t dim, int64_t key_bound,
                                int64_t threshold, int64_t* ukeys, int64_t* num_unique,
-                               int64_t* class_split, void* workspace, size_t workspace_bytes,
-                               void* stream);
+                               int64_t* class_split, int32_t* first_pos, void* workspace,
+                               size_t workspace_bytes, void* stream);
 int hades_combine_apply_class(const float* grad, int64_t n, int64_t dim, int64_t key_bound, int mode,
                               int which, float* sums, int64_t* cnts, const int64_t* num_unique,
                               const int64_t* class_split, void* workspace, size_t workspace_bytes,
@@ -358,11 +359,19 @@ int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, con
 /* The same arithmetic over one class of a class-ordered combine: the rows u of (ukeys, grad) in
  * [0, class_split[1]) for which = 0 or [class_split[1], num_unique[0]) for which = 1; the table row
  * is ukeys[u] & key_mask (the id for the cold class, the slot for the hot class, whose keys carry
- * the class bit above key_mask).  No lookup: the keys already name the rows. */
+ * the class bit above key_mask).  No lookup: the keys already name the rows.
+ * w_rows / first_pos (both or neither): take the OLD weight row of run u from row first_pos[u] of
+ * w_rows - the rows the forward pass fetched for this very batch (hades_fetch_listed output) -
+ * instead of reading it from the table again; the new row is still written to the table.  For a
+ * cold table in host memory this halves what the update moves over the link.  Only valid while
+ * nothing has written those table rows since they were fetched (one batch in flight per table:
+ * the reference's trainers are of that kind, python/EmbCache/sparse_optim.py:590-685 runs between
+ * a batch's forward and the next one's). */
 int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
                                const int64_t* class_split, int which, int64_t key_mask,
                                int64_t max_rows, int64_t dim, float* w, float* s, int64_t stride,
-                               float lr, float eps, void* stream);
+                               const float* w_rows, const int32_t* first_pos, float lr, float eps,
+                               void* stream);
 
 /* SparseAdam row update, same fusion (python/EmbCache/sparse_optim.py:632-657,681):
  *   step += 1; m = b1*m + (1-b1)*g; v = b2*v + (1-b2)*g*g

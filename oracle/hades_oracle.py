@@ -294,18 +294,25 @@ def class_ordered_keys(q, sorted_hot, key_bits):
     return np.where(loc >= 0, (np.int64(1) << np.int64(key_bits)) | loc, q).astype(np.int64)
 
 
-def keyed_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps, key_bits):
+def keyed_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps, key_bits,
+               fetched_rows=None):
     """One combine + Adagrad step done the keyed way: combine over the class-ordered keys
     (only_unique_grads arithmetic, python/EmbCache/sparse_optim.py:132-139, on another key), then
     the cold runs update the cold tables at row = key and the hot runs the hot tables at row =
     key minus the class bit.  In place.  Must equal combine_sequential on the ids followed by
-    sparse_adagrad_step.  Returns (ukeys, sums, cnts, first hot run)."""
+    sparse_adagrad_step.  With fetched_rows (one row per query, what the forward pass fetched) the
+    old weight of a cold run is the fetched row of its first occurrence instead of the table row.
+    Returns (ukeys, sums, cnts, first hot run)."""
     keys = class_ordered_keys(q, sorted_hot, key_bits)
     ukeys, sums, cnts = combine_sequential(keys, grad)
     thr = np.int64(1) << np.int64(key_bits)
     split = int(np.searchsorted(ukeys, thr, side="left"))
     rows = ukeys[:split]
-    w1, s1 = adagrad_rows(cold_w[rows], cold_s[rows], sums[:split], lr, eps)
+    old = cold_w[rows]
+    if fetched_rows is not None:
+        first = np.array([np.flatnonzero(keys == k)[0] for k in rows], dtype=np.int64)
+        old = np.asarray(fetched_rows)[first] if rows.size else old
+    w1, s1 = adagrad_rows(old, cold_s[rows], sums[:split], lr, eps)
     cold_w[rows], cold_s[rows] = w1, s1
     slots = ukeys[split:] - thr
     w1, s1 = adagrad_rows(hot_w[slots], hot_s[slots], sums[split:], lr, eps)

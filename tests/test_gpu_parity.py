@@ -1451,3 +1451,47 @@ def test_keyed_step_forward_and_backward(lib, N, D, H, n, hot_frac, host_cold):
             assert np.array_equal(np.sort(ids.cpu().numpy()), np.unique(q))
     assert np.array_equal(opt.cold_w.cpu().numpy(), cw) and np.array_equal(opt.cold_s.cpu().numpy(), cs)
     assert np.array_equal(opt.hot_w.cpu().numpy(), hw) and np.array_equal(opt.hot_s.cpu().numpy(), hs)
+
+
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_keyed_backward_with_the_forward_rows(lib, host_cold):
+    """backward_keyed(fetched_rows=rows): the cold update takes the old weights from the rows the
+    forward pass fetched.  With untouched rows the result is that of the plain path, bit for bit;
+    with rows altered on purpose the cold weights follow the altered rows (so they are what is
+    read) while the hot class, which never uses them, is unaffected."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad
+    rng = np.random.default_rng(4242)
+    N, D, H, n = 30_000, 128, 3000, 40_000
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, 0.7)
+    q[:500] = q[0]
+    grad = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+    kb = ops.key_bits_for(N)
+
+    def make():
+        t = torch.from_numpy(cold.copy())
+        return SparseAdagrad(t.pin_memory() if host_cold else t.cuda(), torch.from_numpy(hot_ids))
+
+    plain, reuse, altered = make(), make(), make()
+    t_q, t_g = dev(q), dev(grad)
+    for it in range(2):
+        rows, st = plain.forward_keyed(t_q)
+        plain.backward_keyed(st, t_g, mode=ops.COMBINE_EXACT)
+        rows2, st2 = reuse.forward_keyed(t_q)
+        assert torch.equal(rows, rows2)
+        reuse.backward_keyed(st2, t_g, mode=ops.COMBINE_EXACT, fetched_rows=rows2)
+        torch.cuda.synchronize()
+        for a, b in ((plain.cold_w, reuse.cold_w), (plain.cold_s, reuse.cold_s),
+                     (plain.hot_w, reuse.hot_w), (plain.hot_s, reuse.hot_s)):
+            assert torch.equal(a.cpu(), b.cpu())
+    # altered rows: the oracle with the same altered rows
+    cw, cs = cold.copy(), np.zeros_like(cold)
+    hw, hs = cold[hot_ids].copy(), np.zeros((H, D), np.float32)
+    rows3, st3 = altered.forward_keyed(t_q)
+    bent = rows3 + 0.25
+    altered.backward_keyed(st3, t_g, mode=ops.COMBINE_EXACT, fetched_rows=bent)
+    torch.cuda.synchronize()
+    O.keyed_step(cw, cs, hw, hs, hot_ids, q, grad, 0.01, 1e-10, kb, fetched_rows=bent.cpu().numpy())
+    assert np.array_equal(altered.cold_w.cpu().numpy(), cw) and np.array_equal(altered.cold_s.cpu().numpy(), cs)
+    assert np.array_equal(altered.hot_w.cpu().numpy(), hw) and np.array_equal(altered.hot_s.cpu().numpy(), hs)
+    assert not np.array_equal(cw, plain.cold_w.cpu().numpy())

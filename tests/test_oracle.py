@@ -638,3 +638,10 @@ def test_keyed_step_equals_combine_then_update_on_the_ids():
         assert not np.isin(ukeys[:split], hot_ids).any()
     for x, y in zip(a, b):
         assert np.array_equal(x, y)
+    # with the rows a forward pass fetched (= the table rows) nothing changes
+    c = [x.copy() for x in b]
+    O.keyed_step(b[0], b[1], b[2], b[3], hot_ids, q, g, 0.01, 1e-10, kb)
+    O.keyed_step(c[0], c[1], c[2], c[3], hot_ids, q, g, 0.01, 1e-10, kb,
+                 fetched_rows=O.cached_fetch(c[0], c[2], q, hot_ids))
+    for x, y in zip(b, c):
+        assert np.array_equal(x, y)
