@@ -109,20 +109,24 @@ __global__ __launch_bounds__(kThreads) void split_masks_kernel(const I* __restri
 // of the class predicate and a count of the set bits below the lane (mbcnt); the (round, wave)
 // counts of a tile are prefixed in LDS, and the tiles before it are summed from the per-tile
 // counts of the first kernel.  Positions inside every class list are ascending.
-constexpr int kRounds = 8;
-constexpr int kTile = kThreads * kRounds;
+// Rounds per thread: 8 for classifiers that only read their element; 2 for the fused lookup, whose
+// dependent table and id reads per element would otherwise run one after the other in a thread
+// while three quarters of the CU's wave slots stay empty (1 M lookups: 43 us with 8 rounds).
+constexpr int kRoundsDefault = 8;
+constexpr int kRoundsLookup = 2;
 constexpr int kWaves = kThreads / kWave;
 constexpr uint32_t kNone = 3;           // class code of an element that belongs to no list
 constexpr int64_t kSumTilesInKernel = 4096;  // above this many tiles a scan kernel prefixes them
 
 // classify + per-tile counts.  Classifier returns the class code (0..2, or kNone) of element i;
 // it is called exactly once per element and may write per-element results of its own.
-template <typename Classifier>
+template <typename Classifier, int kRounds>
 __global__ __launch_bounds__(kThreads) void classify_count_kernel(Classifier cf, int64_t n,
                                                                  uint8_t* __restrict__ cls,
                                                                  uint32_t* __restrict__ blk_cnt,
                                                                  int64_t nblocks) {
   __shared__ uint32_t s_cnt[kWaves][3];
+  constexpr int kTile = kThreads * kRounds;
   const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kTile;
   uint32_t cnt[3] = {0, 0, 0};   // wave-uniform
 #pragma unroll
@@ -173,6 +177,7 @@ struct CompactOut {
   int64_t* pos[3];
 };
 
+template <int kRounds>
 __global__ __launch_bounds__(kThreads) void compact_kernel(const uint8_t* __restrict__ cls,
                                                           const uint32_t* __restrict__ blk_cnt,
                                                           const int64_t* __restrict__ blk_off,
@@ -184,6 +189,7 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(const uint8_t* __rest
   __shared__ uint32_t s_cnt[kRounds][kWaves][3];   // counts, then exclusive offsets inside the tile
   const int lane = lane_id();
   const int wave = threadIdx.x / kWave;
+  constexpr int kTile = kThreads * kRounds;
   const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kTile;
 
   // the tile's class codes first, so that their latency overlaps the sum over earlier tiles
@@ -310,7 +316,7 @@ struct CompactWs {
   size_t bytes;
 };
 CompactWs carve_compact(void* ws, int64_t n) {
-  const int64_t nblocks = ceil_div(n > 0 ? n : 1, kTile);
+  const int64_t nblocks = ceil_div(n > 0 ? n : 1, kThreads * kRoundsLookup);   // the most tiles any form uses
   Carver c(ws);
   CompactWs w;
   w.cls = c.take<uint8_t>(n > 0 ? n : 1);
@@ -320,9 +326,10 @@ CompactWs carve_compact(void* ws, int64_t n) {
   return w;
 }
 
-template <typename Classifier>
+template <typename Classifier, int kRounds = kRoundsDefault>
 int run_compact(const Classifier& cf, int64_t n, int num_classes, const CompactOut& out,
                 int64_t* counts, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  constexpr int kTile = kThreads * kRounds;
   HADES_REQUIRE(n >= 0 && n < (int64_t(1) << 40), "n out of range: %lld", (long long)n);
   HADES_REQUIRE(counts != nullptr, "counts must not be null");
   const CompactWs w = carve_compact(workspace, n);
@@ -332,16 +339,16 @@ int run_compact(const Classifier& cf, int64_t n, int num_classes, const CompactO
   HADES_REQUIRE((align_of_ptr(workspace) & 255) == 0, "workspace must be 256-byte aligned");
   const int64_t nblocks = ceil_div(n > 0 ? n : 1, kTile);
   HADES_REQUIRE(nblocks < (int64_t(1) << 31), "n too large");
-  HADES_LAUNCH((classify_count_kernel<Classifier>), dim3((unsigned)nblocks), dim3(kThreads), 0,
-                     st, cf, n, w.cls, w.blk_cnt, nblocks);
+  HADES_LAUNCH((classify_count_kernel<Classifier, kRounds>), dim3((unsigned)nblocks), dim3(kThreads),
+                     0, st, cf, n, w.cls, w.blk_cnt, nblocks);
   const int64_t* blk_off = nullptr;
   if (nblocks > kSumTilesInKernel) {
     HADES_LAUNCH(block_prefix_kernel, dim3(1), dim3(kThreads), 0, st, w.blk_cnt, w.blk_off,
                        nblocks, num_classes);
     blk_off = w.blk_off;
   }
-  HADES_LAUNCH(compact_kernel, dim3((unsigned)nblocks), dim3(kThreads), 0, st, w.cls, w.blk_cnt,
-                     blk_off, nblocks, n, num_classes, out, counts);
+  HADES_LAUNCH((compact_kernel<kRounds>), dim3((unsigned)nblocks), dim3(kThreads), 0, st, w.cls,
+                     w.blk_cnt, blk_off, nblocks, n, num_classes, out, counts);
   return HADES_OK;
 }
 
@@ -520,8 +527,8 @@ int hades_lookup_split(const int64_t* q, const int64_t* num_live, int64_t n,
   CompactOut out{{hot_mask, nullptr, nullptr}, {hot_pos, cold_pos, nullptr}};
   ClassifyLookup cf{q, HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}, loc,
                     num_live, sort_keys, key_bits};
-  return run_compact(cf, n, 2, out, counts, workspace, workspace_bytes,
-                     static_cast<hipStream_t>(stream));
+  return run_compact<ClassifyLookup, kRoundsLookup>(cf, n, 2, out, counts, workspace, workspace_bytes,
+                                                    static_cast<hipStream_t>(stream));
 }
 
 int hades_split3_compact(const void* ids, int id_type, const int8_t* class_table, int64_t n,

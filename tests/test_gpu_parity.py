@@ -1495,3 +1495,25 @@ def test_keyed_backward_with_the_forward_rows(lib, host_cold):
     assert np.array_equal(altered.cold_w.cpu().numpy(), cw) and np.array_equal(altered.cold_s.cpu().numpy(), cs)
     assert np.array_equal(altered.hot_w.cpu().numpy(), hw) and np.array_equal(altered.hot_s.cpu().numpy(), hs)
     assert not np.array_equal(cw, plain.cold_w.cpu().numpy())
+
+
+def test_lookup_split_beyond_the_in_kernel_tile_sum(lib):
+    """More than 4 096 tiles of queries: the per-tile counts are prefixed by a scan kernel of their
+    own instead of being summed inside every compaction block.  Same lists, same slots."""
+    _, ops = lib
+    rng = np.random.default_rng(99)
+    N, H, n = 50_000, 7_000, 2_200_001
+    hot_ids = np.sort(rng.choice(N, H, replace=False)).astype(np.int64)
+    q = rng.integers(0, N, n).astype(np.int64)
+    hs = ops.HotSet(dev(hot_ids))
+    keys = torch.empty(n, dtype=torch.int64, device="cuda")
+    loc, hot_pos, cold_pos, counts = ops.lookup_split(dev(q), hs, sort_keys=keys, key_bits=16)
+    w_loc, w_hp, w_cp = O.lookup_split(q, hot_ids)
+    nh, nc = counts.tolist()
+    assert (nh, nc) == (w_hp.size, w_cp.size)
+    assert np.array_equal(loc.cpu().numpy(), w_loc)
+    assert np.array_equal(hot_pos[:nh].cpu().numpy(), w_hp) and np.array_equal(cold_pos[:nc].cpu().numpy(), w_cp)
+    assert np.array_equal(keys.cpu().numpy(), O.class_ordered_keys(q, hot_ids, 16))
+    # the plain two-class split of the same slots (8 rounds per thread: 1 075 tiles) agrees
+    _, hp2, cp2 = ops.split(loc)
+    assert torch.equal(hp2, hot_pos[:nh]) and torch.equal(cp2, cold_pos[:nc])
