@@ -53,6 +53,49 @@ def test_argument_errors_are_codes_and_messages():
         _lib.call("hades_hash_clear", one, one, one, 1000, 8, null)
 
 
+def test_argument_errors_of_the_split_schedule_entry_points():
+    """The listed / class / static entry points check their arguments before any HIP call."""
+    lib = _lib.load()
+    null = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(256)     # never dereferenced: the checks fail first
+    # listed gather / scatter: dtype, stride, null pointers; an empty list is fine
+    assert lib.hades_fetch_listed(one, 0, one, one, one, 10, one, 8, 7, null) == 1
+    assert b"float or double" in lib.hades_last_error()
+    assert lib.hades_fetch_listed(one, 4, one, one, one, 10, one, 8, _lib.F32, null) == 1     # stride < dim
+    assert b"stride" in lib.hades_last_error()
+    assert lib.hades_fetch_listed(one, 0, one, null, one, 10, one, 8, _lib.F32, null) == 1
+    assert lib.hades_fetch_listed(null, 0, null, null, null, 0, null, 8, _lib.F32, null) == 0
+    assert lib.hades_set_listed(one, one, 3, one, one, one, 10, 8, _lib.F32, null) == 1
+    assert lib.hades_set_listed(null, null, 0, null, null, null, 0, 8, _lib.F32, null) == 0
+    # listed / class Adagrad
+    assert lib.hades_adagrad_update_listed(one, one, one, one, 10, 8, one, one, 4, 0.01, 1e-10, null) == 1
+    assert lib.hades_adagrad_update_listed(one, one, one, null, 10, 8, one, one, 0, 0.01, 1e-10, null) == 1
+    assert lib.hades_adagrad_update_listed(null, null, null, null, 0, 8, null, null, 0, 0.01, 1e-10, null) == 0
+    assert lib.hades_adagrad_update_class(one, one, one, one, 2, 255, 10, 8, one, one, 0, null, null,
+                                          0.01, 1e-10, null) == 1                              # which
+    assert lib.hades_adagrad_update_class(one, one, one, one, 0, 255, 10, 8, one, one, 0, one, null,
+                                          0.01, 1e-10, null) == 1                              # rows without positions
+    assert b"go together" in lib.hades_last_error()
+    # lookup + split: key bits must leave room for the slots
+    assert lib.hades_lookup_split(one, null, 10, one, 1 << 20, null, one, null, one, one, one, one, 8,
+                                  one, 1 << 20, null) == 1
+    assert b"key_bits" in lib.hades_last_error()
+    assert lib.hades_lookup_split(one, null, 10, one, 100, null, one, null, one, one, one, null, 0,
+                                  one, 16, null) == 3                                          # workspace
+    # classed combine
+    assert lib.hades_combine_plan_classed(one, 10, 8, 1 << 20, 1 << 19, one, one, null, null, one, 1 << 20, null) == 1
+    assert lib.hades_combine_plan_classed(one, 10, 8, 1 << 20, 1 << 21, one, one, one, null, one, 1 << 20, null) == 1
+    assert lib.hades_combine_apply_class(one, 10, 8, 1 << 20, 0, 2, one, one, one, one, one, 1 << 20, null) == 1
+    # static combine: refused beyond its scratch, before anything else
+    assert lib.hades_combine_static(one, one, 1_000_000, 128, 0, 0, one, one, one, one, null, null) == 1
+    assert b"scratch" in lib.hades_last_error()
+    # pinned allocation: flags and null out pointer
+    p = ctypes.c_void_p()
+    assert lib.hades_host_alloc_flags(ctypes.byref(p), 16, 4) == 1
+    assert lib.hades_host_alloc_flags(None, 16, 0) == 1
+    assert lib.hades_host_alloc_flags(ctypes.byref(p), 0, 0) == 0 and not p.value
+
+
 def test_workspace_queries():
     assert _lib.query("hades_combine_workspace_bytes", 0, 8) > 0
     a = _lib.query("hades_combine_workspace_bytes", 200_000, 128)
