@@ -119,3 +119,30 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
                        capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_key_bits_and_class_ordered_keys():
+    """Host-side arithmetic of the keyed step: the bits that hold a table's ids, and the order the
+    class-ordered keys induce (cold ids ascending, then hot ids ascending)."""
+    from hades_amd import ops
+    assert [ops.key_bits_for(n) for n in (1, 2, 3, 4, 5, 1 << 20, (1 << 20) + 1, 111_000_000, 244_000_000)] == \
+        [1, 1, 2, 2, 3, 20, 21, 27, 28]
+    rng = np.random.default_rng(3)
+    N, H = 1000, 120
+    hot = np.sort(rng.choice(N, H, replace=False)).astype(np.int64)
+    q = rng.integers(0, N, 5000).astype(np.int64)
+    kb = ops.key_bits_for(N)
+    keys = O.class_ordered_keys(q, hot, kb)
+    order = np.argsort(keys, kind="stable")
+    is_hot = np.isin(q[order], hot)
+    first_hot = int(np.argmax(is_hot)) if is_hot.any() else q.size
+    assert not is_hot[:first_hot].any() and is_hot[first_hot:].all()
+    assert np.all(np.diff(q[order][:first_hot]) >= 0) and np.all(np.diff(q[order][first_hot:]) >= 0)
+    assert np.all(keys[~np.isin(q, hot)] == q[~np.isin(q, hot)])
+    assert np.all((keys[np.isin(q, hot)] >> kb) == 1)
+
+
+def test_split_schedule_objects_need_no_gpu_to_import():
+    from hades_amd import sparse_optim
+    for name in ("fetch_split", "update_split", "step_split", "forward_keyed", "backward_keyed", "join"):
+        assert callable(getattr(sparse_optim.SparseAdagrad, name))
