@@ -295,14 +295,29 @@ int check_rows(const int64_t* uids, const float* grad, int64_t max_rows, int64_t
   return HADES_OK;
 }
 
+int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
+  float* w = a.w;
+  float* s = a.s;
+  const float* grad = a.grad;
+  const int64_t max_count = a.max_count, dim = a.dim, stride = a.stride;
+  int64_t blocks = ceil_div(max_count, kRows);
+  if (blocks > 16384) blocks = 16384;
+  // rows that cross the host link: a narrow grid that strides over the list
+  if ((is_host_memory(w) || is_host_memory(s)) && blocks > host_link_blocks(true))
+    blocks = host_link_blocks(true);
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dim % 4 == 0 && stride % 4 == 0 && aligned16({grad, w, s, a.w_rows}))
+    HADES_LAUNCH((adagrad_listed_kernel<4>), grid, block, 0, st, a);
+  else
+    HADES_LAUNCH((adagrad_listed_kernel<1>), grid, block, 0, st, a);
+  return HADES_OK;
+}
+
 }  // namespace
 }  // namespace hades
 
 using namespace hades;
-
-namespace {
-int launch_adagrad_listed(const AdagradListedArgs& a, void* stream);
-}
 
 extern "C" {
 
@@ -358,31 +373,6 @@ int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const in
                       key_mask, w_rows, first_pos, dim, w, s, stride, lr, eps};
   return launch_adagrad_listed(a, stream);
 }
-
-}  // extern "C"
-
-namespace {
-int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
-  float* w = a.w;
-  float* s = a.s;
-  const float* grad = a.grad;
-  const int64_t max_count = a.max_count, dim = a.dim, stride = a.stride;
-  int64_t blocks = ceil_div(max_count, kRows);
-  if (blocks > 16384) blocks = 16384;
-  // rows that cross the host link: a narrow grid that strides over the list
-  if ((is_host_memory(w) || is_host_memory(s)) && blocks > host_link_blocks(true))
-    blocks = host_link_blocks(true);
-  const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dim % 4 == 0 && stride % 4 == 0 && aligned16({grad, w, s, a.w_rows}))
-    HADES_LAUNCH((adagrad_listed_kernel<4>), grid, block, 0, st, a);
-  else
-    HADES_LAUNCH((adagrad_listed_kernel<1>), grid, block, 0, st, a);
-  return HADES_OK;
-}
-}  // namespace
-
-extern "C" {
 
 int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                       int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,

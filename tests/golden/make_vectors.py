@@ -130,12 +130,61 @@ def accumulator_case(rng):
     return out
 
 
+def split_schedule_case(rng):
+    """One training step done class by class (split first: python/EmbCache/dist_emb.py:174-211),
+    all by loops and dicts: slots, the two position lists, the class-ordered sort keys, the
+    distinct keys with their sequential float32 sums and counts, the class border, and the tables
+    after one Adagrad step (torch.optim.Adagrad on the gathered rows of each class)."""
+    num_rows, dim, key_bits = 1500, 8, 11
+    hot = np.sort(rng.choice(num_rows, 200, replace=False)).astype(np.int64)
+    w = 1.0 / np.arange(1, num_rows + 1)
+    q = rng.permutation(num_rows)[rng.choice(num_rows, 900, p=w / w.sum())].astype(np.int64)
+    grad = (rng.standard_normal((q.size, dim)) * 1e-3).astype(np.float32)
+    cold = (rng.standard_normal((num_rows, dim)) * 0.01).astype(np.float32)
+    hot_rows = (rng.standard_normal((hot.size, dim)) * 0.01).astype(np.float32)
+    slot_of = {int(h): k for k, h in enumerate(hot)}
+    loc = np.array([slot_of.get(int(x), -1) for x in q], dtype=np.int64)
+    hot_pos = np.array([p for p, x in enumerate(q) if int(x) in slot_of], dtype=np.int64)
+    cold_pos = np.array([p for p, x in enumerate(q) if int(x) not in slot_of], dtype=np.int64)
+    keys = np.array([(1 << key_bits) | slot_of[int(x)] if int(x) in slot_of else int(x) for x in q],
+                    dtype=np.int64)
+    sums, cnts, first = {}, {}, {}
+    for p, k in enumerate(keys):                                  # occurrence order, float32
+        k = int(k)
+        sums[k] = (sums.get(k, np.zeros(dim, np.float32)) + grad[p]).astype(np.float32)
+        cnts[k] = cnts.get(k, 0) + 1
+        first.setdefault(k, p)
+    ukeys = np.array(sorted(sums), dtype=np.int64)
+    usums = np.stack([sums[int(k)] for k in ukeys]).astype(np.float32)
+    ucnts = np.array([cnts[int(k)] for k in ukeys], dtype=np.int64)
+    ufirst = np.array([first[int(k)] for k in ukeys], dtype=np.int32)
+    split_run = int(sum(1 for k in ukeys if k < (1 << key_bits)))
+    cold_after, hot_after = cold.copy(), hot_rows.copy()
+    cold_state, hot_state = np.zeros_like(cold), np.zeros_like(hot_rows)
+    for table, state, rows, g in ((cold_after, cold_state, ukeys[:split_run], usums[:split_run]),
+                                  (hot_after, hot_state, ukeys[split_run:] - (1 << key_bits), usums[split_run:])):
+        prm = torch.nn.Parameter(torch.from_numpy(table[rows].copy()))
+        opt = torch.optim.Adagrad([prm], lr=0.01, eps=1e-10)
+        prm.grad = torch.from_numpy(g.copy())
+        opt.step()
+        table[rows] = prm.detach().numpy()
+        state[rows] = opt.state[prm]["sum"].numpy()
+    return {"ss_hot": hot, "ss_q": q, "ss_grad": grad, "ss_cold": cold, "ss_hot_rows": hot_rows,
+            "ss_key_bits": np.array([key_bits], np.int64), "ss_loc": loc, "ss_hot_pos": hot_pos,
+            "ss_cold_pos": cold_pos, "ss_keys": keys, "ss_ukeys": ukeys, "ss_usums": usums,
+            "ss_ucnts": ucnts, "ss_first_pos": ufirst,
+            "ss_class_split": np.array([cold_pos.size, split_run], np.int64),
+            "ss_cold_after": cold_after, "ss_hot_after": hot_after, "ss_cold_state": cold_state,
+            "ss_hot_state": hot_state}
+
+
 def main():
     rng = np.random.default_rng(20240611)
     torch.manual_seed(0)
     vec = {}
     for case in (lookup_case, split_case, rows_case, combine_case, adagrad_case, adam_case,
-                 accumulator_case):
+                 accumulator_case, split_schedule_case):      # new cases go last: the earlier
+        # arrays depend on the generator's position and must not change
         vec.update(case(rng))
     path = os.path.join(HERE, "vectors.npz")
     np.savez_compressed(path, **vec)

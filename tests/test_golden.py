@@ -83,6 +83,30 @@ def test_oracle_accumulator_golden():
     assert _eq(sums, VEC["acc_flush_sums"])
 
 
+def _keyed_close(cw, cs, hw, hs):
+    """as _adagrad_close: torch.optim.Adagrad is one rounding apart from the row arithmetic"""
+    assert np.allclose(cw, VEC["ss_cold_after"], rtol=1e-5, atol=1e-8)
+    assert np.allclose(hw, VEC["ss_hot_after"], rtol=1e-5, atol=1e-8)
+    assert np.allclose(cs, VEC["ss_cold_state"], rtol=1e-6, atol=0)
+    assert np.allclose(hs, VEC["ss_hot_state"], rtol=1e-6, atol=0)
+
+
+def test_oracle_split_schedule_golden():
+    hot, q, kb = VEC["ss_hot"], VEC["ss_q"], int(VEC["ss_key_bits"][0])
+    loc, hot_pos, cold_pos = O.lookup_split(q, hot)
+    assert _eq(loc, VEC["ss_loc"]) and _eq(hot_pos, VEC["ss_hot_pos"]) and _eq(cold_pos, VEC["ss_cold_pos"])
+    assert _eq(O.class_ordered_keys(q, hot, kb), VEC["ss_keys"])
+    cw, cs = VEC["ss_cold"].copy(), np.zeros_like(VEC["ss_cold"])
+    hw, hs = VEC["ss_hot_rows"].copy(), np.zeros_like(VEC["ss_hot_rows"])
+    ukeys, sums, cnts, split = O.keyed_step(cw, cs, hw, hs, hot, q, VEC["ss_grad"], 0.01, 1e-10, kb)
+    assert _eq(ukeys, VEC["ss_ukeys"]) and _eq(sums, VEC["ss_usums"]) and _eq(cnts, VEC["ss_ucnts"])
+    assert split == int(VEC["ss_class_split"][1])
+    _keyed_close(cw, cs, hw, hs)
+    # the fetch, class by class
+    want = np.stack([VEC["ss_hot_rows"][l] if l >= 0 else VEC["ss_cold"][x] for l, x in zip(VEC["ss_loc"], q)])
+    assert _eq(O.fetch_split(VEC["ss_cold"], VEC["ss_hot_rows"], q, hot), want)
+
+
 # ------------------------------------------------------------------------ HIP library vs vectors
 def _d(name, dev):
     return torch.from_numpy(VEC[name].copy()).to(dev)
@@ -179,3 +203,40 @@ def test_hip_accumulator_golden(cuda_device):
     assert _eq(sums.cpu().numpy(), VEC["acc_flush_sums"])
     ids2, _, _ = acc.flush()
     assert ids2.numel() == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_hip_split_schedule_golden(cuda_device, host_cold):
+    from hades_amd import ops
+    from hades_amd.sparse_optim import SparseAdagrad
+    kb = int(VEC["ss_key_bits"][0])
+    q = _d("ss_q", cuda_device)
+    hs = ops.HotSet(_d("ss_hot", cuda_device))
+    keys = torch.empty_like(q)
+    loc, hot_pos, cold_pos, counts = ops.lookup_split(q, hs, sort_keys=keys, key_bits=kb)
+    nh, nc = counts.tolist()
+    assert _eq(loc.cpu().numpy(), VEC["ss_loc"]) and _eq(keys.cpu().numpy(), VEC["ss_keys"])
+    assert _eq(hot_pos[:nh].cpu().numpy(), VEC["ss_hot_pos"]) and _eq(cold_pos[:nc].cpu().numpy(), VEC["ss_cold_pos"])
+    first_pos = torch.empty(q.numel(), dtype=torch.int32, device=cuda_device)
+    plan = ops.combine_plan_classed(keys, VEC["ss_grad"].shape[1], kb, first_pos=first_pos)
+    g = _d("ss_grad", cuda_device)
+    sums, cnts = ops.combine_apply_class(plan, g, 0, ops.COMBINE_EXACT)
+    ops.combine_apply_class(plan, g, 1, ops.COMBINE_EXACT, out=(sums, cnts))
+    U = int(plan.num_unique.item())
+    assert _eq(plan.uids[:U].cpu().numpy(), VEC["ss_ukeys"]) and _eq(cnts[:U].cpu().numpy(), VEC["ss_ucnts"])
+    assert _eq(sums[:U].cpu().numpy(), VEC["ss_usums"])
+    assert _eq(plan.class_split.cpu().numpy(), VEC["ss_class_split"])
+    assert _eq(first_pos[:U].cpu().numpy(), VEC["ss_first_pos"])
+    # the whole step through the optimizer, cold table in HBM or in pinned host memory
+    cold = torch.from_numpy(VEC["ss_cold"].copy())
+    cold = cold.pin_memory() if host_cold else cold.to(cuda_device)
+    opt = SparseAdagrad(cold, torch.from_numpy(VEC["ss_hot"].copy()), lr=0.01, eps=1e-10)
+    opt.hot_w.copy_(_d("ss_hot_rows", cuda_device))
+    assert ops.key_bits_for(opt.num_rows) == kb
+    rows, state = opt.forward_keyed(q)
+    want = np.stack([VEC["ss_hot_rows"][l] if l >= 0 else VEC["ss_cold"][x] for l, x in zip(VEC["ss_loc"], VEC["ss_q"])])
+    assert _eq(rows.cpu().numpy(), want)
+    opt.backward_keyed(state, g, mode=ops.COMBINE_EXACT)
+    torch.cuda.synchronize()
+    _keyed_close(opt.cold_w.cpu().numpy(), opt.cold_s.cpu().numpy(), opt.hot_w.cpu().numpy(), opt.hot_s.cpu().numpy())
