@@ -1517,3 +1517,43 @@ def test_lookup_split_beyond_the_in_kernel_tile_sum(lib):
     # the plain two-class split of the same slots (8 rounds per thread: 1 075 tiles) agrees
     _, hp2, cp2 = ops.split(loc)
     assert torch.equal(hp2, hot_pos[:nh]) and torch.equal(cp2, cold_pos[:nc])
+
+
+@pytest.mark.parametrize("dim,fdt", [(1, torch.float32), (3, torch.float32), (7, torch.float64),
+                                     (100, torch.float32), (128, torch.float64), (260, torch.float32)])
+@pytest.mark.parametrize("host", [False, True])
+def test_listed_gather_and_scatter_row_shapes(lib, dim, fdt, host):
+    """hades_fetch_listed / hades_set_listed over row widths that take the 16-, 8- and 4-byte
+    paths, float32 and float64, 1-D tables, device and pinned-host tables, unaligned row-strided
+    views."""
+    _, ops = lib
+    rng = np.random.default_rng(dim)
+    N, n = 3000, 2500
+    width = dim + 3                                       # rows of a wider table: stride > dim
+    base = torch.from_numpy(rng.standard_normal((N, width)).astype(NP_F[fdt]))
+    base = base.pin_memory() if host else base.cuda()
+    table = base[:, 1:1 + dim]                            # starts one element in: unaligned rows
+    ref = base.cpu().numpy().copy()
+    idx = rng.integers(0, N, n).astype(np.int64)
+    pos = rng.permutation(n)[: n - 100].astype(np.int64)
+    cnt = torch.tensor([pos.size - 7], dtype=torch.int64, device="cuda")
+    out = torch.full((n, dim), -3.0, dtype=fdt, device="cuda")
+    ops.fetch_listed(table, dev(idx), dev(pos), cnt, out)
+    want = O.fetch_listed(ref[:, 1:1 + dim], idx, pos, pos.size - 7, np.full((n, dim), -3.0, NP_F[fdt]))
+    assert np.array_equal(out.cpu().numpy(), want)
+    # scatter distinct rows back
+    uidx = rng.permutation(N)[:n].astype(np.int64)
+    src = rng.standard_normal((n, dim)).astype(NP_F[fdt])
+    ops.set_listed(dev(src), table, dev(uidx), dev(pos), cnt)
+    torch.cuda.synchronize()
+    view = ref[:, 1:1 + dim].copy()
+    O.set_listed(src, view, uidx, pos, pos.size - 7)
+    ref[:, 1:1 + dim] = view
+    assert np.array_equal(base.cpu().numpy(), ref)        # the columns outside the view are untouched
+    if dim == 1:                                          # the 1-D form
+        flat = torch.from_numpy(rng.standard_normal(N).astype(NP_F[fdt]))
+        flat = flat.pin_memory() if host else flat.cuda()
+        o1 = torch.zeros(n, dtype=fdt, device="cuda")
+        ops.fetch_listed(flat, dev(idx), dev(pos), cnt, o1)
+        w1 = O.fetch_listed(flat.cpu().numpy(), idx, pos, pos.size - 7, np.zeros(n, NP_F[fdt]))
+        assert np.array_equal(o1.cpu().numpy(), w1)
