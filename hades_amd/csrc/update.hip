@@ -124,62 +124,90 @@ __global__ __launch_bounds__(kThreads) void adagrad_kernel(AdagradArgs a) {
   }
 }
 
-// Adagrad over the rows named by a position list whose length lives in device memory (one half of
-// a hot/cold split): for j < count[0], p = list[j]; the gradient is row p of grad, the weight and
-// state rows are row row_index[p] of w and s, whose rows lie `stride` floats apart (w and s of a
-// row may sit next to each other in one table: s = w + dim, stride = 2 * dim).
-struct AdagradListedArgs {
+// Row updates over the rows named by a position list whose length lives in device memory (one half
+// of a hot/cold split), or over one class of the distinct rows of a class-ordered combine.
+// Listed form: for j < count[0], p = list[j].  Class form: p runs over [class_split[1],
+// num_unique[0]) (which = 1) or [0, class_split[1]) (which = 0).  The gradient is row p of grad;
+// the table row is row_index[p] & index_mask, and rows of the weight table and of the per-element
+// state tables lie `stride` floats apart (weights and state of a row may sit next to each other
+// in one table: s = w + dim, stride = 2 * dim).
+struct ListedRows {
   const int64_t* row_index;
   const float* grad;
-  const int64_t* list;      // null: positions are the range itself (class form)
+  const int64_t* list;      // null: class form
   const int64_t* count;     // listed form: number of live list entries
   int64_t max_count;
-  // class form: rows [class_split[1], num_unique[0]) (which = 1) or [0, class_split[1]) (which = 0)
   const int64_t* num_unique;
   const int64_t* class_split;
   int which;
-  int64_t index_mask;       // table row = row_index[p] & index_mask
+  int64_t index_mask;
   // optional: the old weight row of position p is row first_pos[p] of w_rows (rows fetched from
   // the same table earlier and still valid) instead of being read from the table again
   const float* w_rows;
   const int32_t* first_pos;
   int64_t dim;
+  int64_t stride;
+};
+
+struct AdagradListedArgs {
+  ListedRows r;
   float* w;
   float* s;
-  int64_t stride;
   float lr, eps;
 };
+
+struct AdamListedArgs {
+  ListedRows r;
+  float* w;
+  float* step;              // one float per table row
+  float* m;
+  float* v;
+  float lr, beta1, beta2, one_minus_beta1, one_minus_beta2, eps;
+};
+
+// the positions [first, end) a launch walks
+__device__ __forceinline__ void listed_range(const ListedRows& a, int64_t* first, int64_t* end) {
+  if (a.list != nullptr) {
+    const int64_t cnt = a.count[0];
+    *first = 0;
+    *end = cnt < a.max_count ? cnt : a.max_count;
+    return;
+  }
+  int64_t U = a.num_unique[0];
+  U = U < a.max_count ? U : a.max_count;
+  int64_t sr = a.class_split[1];
+  sr = sr < U ? sr : U;
+  sr = sr > 0 ? sr : 0;
+  *first = a.which ? sr : 0;
+  *end = a.which ? U : sr;
+}
+
+// Offsets of the rows [row0, row0 + rows_here) of the walk: s_tab[r] = table row, s_grad[r] =
+// element offset of the gradient row, s_old[r] = element offset of the old weight row in w_rows.
+__device__ __forceinline__ void resolve_listed(const ListedRows& a, int64_t row0, int rows_here,
+                                               int64_t* s_tab, int64_t* s_grad, int64_t* s_old) {
+  for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+    const int64_t p = a.list != nullptr ? a.list[row0 + r] : row0 + r;
+    s_tab[r] = a.row_index[p] & a.index_mask;
+    s_grad[r] = p * a.dim;
+    if (a.w_rows != nullptr) s_old[r] = static_cast<int64_t>(a.first_pos[p]) * a.dim;
+  }
+}
 
 template <int VEC>
 __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedArgs a) {
   typedef typename Vf<VEC>::type V;
-  __shared__ int64_t s_row[kRows];    // element offset of the row in w and s
-  __shared__ int64_t s_grad[kRows];   // element offset of the row in grad
-  __shared__ int64_t s_old[kRows];    // element offset of the old weight row in w_rows
-  int64_t first = 0, cnt;
-  if (a.list != nullptr) {
-    cnt = a.count[0];
-    cnt = cnt < a.max_count ? cnt : a.max_count;
-  } else {
-    int64_t U = a.num_unique[0];
-    U = U < a.max_count ? U : a.max_count;
-    int64_t sr = a.class_split[1];
-    sr = sr < U ? sr : U;
-    sr = sr > 0 ? sr : 0;
-    first = a.which ? sr : 0;
-    cnt = a.which ? U : sr;
-  }
-  const int cpr = static_cast<int>(a.dim / VEC);
+  __shared__ int64_t s_tab[kRows];
+  __shared__ int64_t s_grad[kRows];
+  __shared__ int64_t s_old[kRows];
+  int64_t first, cnt;
+  listed_range(a.r, &first, &cnt);
+  const int cpr = static_cast<int>(a.r.dim / VEC);
   for (int64_t row0 = first + static_cast<int64_t>(blockIdx.x) * kRows; row0 < cnt;
        row0 += static_cast<int64_t>(gridDim.x) * kRows) {
     const int64_t left = cnt - row0;
     const int rows_here = left < kRows ? static_cast<int>(left) : kRows;
-    for (int r = threadIdx.x; r < rows_here; r += kThreads) {
-      const int64_t p = a.list != nullptr ? a.list[row0 + r] : row0 + r;
-      s_row[r] = (a.row_index[p] & a.index_mask) * a.stride;
-      s_grad[r] = p * a.dim;
-      if (a.w_rows != nullptr) s_old[r] = static_cast<int64_t>(a.first_pos[p]) * a.dim;
-    }
+    resolve_listed(a.r, row0, rows_here, s_tab, s_grad, s_old);
     __syncthreads();
     const int total = rows_here * cpr;
     for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
@@ -192,11 +220,13 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
         if (c < total) {
           const int r = c / cpr;
           const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
-          sp[k] = reinterpret_cast<V*>(a.s + s_row[r] + col);
-          wp[k] = reinterpret_cast<V*>(a.w + s_row[r] + col);
-          g[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(a.grad + s_grad[r] + col));
+          const int64_t off = s_tab[r] * a.r.stride + col;
+          sp[k] = reinterpret_cast<V*>(a.s + off);
+          wp[k] = reinterpret_cast<V*>(a.w + off);
+          g[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(a.r.grad + s_grad[r] + col));
           s[k] = *sp[k];
-          w[k] = a.w_rows != nullptr ? *reinterpret_cast<const V*>(a.w_rows + s_old[r] + col) : *wp[k];
+          w[k] = a.r.w_rows != nullptr ? *reinterpret_cast<const V*>(a.r.w_rows + s_old[r] + col)
+                                       : *wp[k];
         }
       }
 #pragma unroll
@@ -208,6 +238,77 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
           const V w1 = w[k] - vdiv(a.lr * g[k], std_);
           *sp[k] = s1;
           *wp[k] = w1;
+        }
+      }
+    }
+    __syncthreads();   // the row offsets are rewritten by the next round
+  }
+}
+
+// SparseAdam over the same walk: the arithmetic of adam_kernel below, one table set per launch.
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void adam_listed_kernel(AdamListedArgs a) {
+  typedef typename Vf<VEC>::type V;
+  __shared__ int64_t s_tab[kRows];
+  __shared__ int64_t s_grad[kRows];
+  __shared__ int64_t s_old[kRows];
+  __shared__ float s_c1[kRows];
+  __shared__ float s_c2[kRows];
+  int64_t first, cnt;
+  listed_range(a.r, &first, &cnt);
+  const int cpr = static_cast<int>(a.r.dim / VEC);
+  for (int64_t row0 = first + static_cast<int64_t>(blockIdx.x) * kRows; row0 < cnt;
+       row0 += static_cast<int64_t>(gridDim.x) * kRows) {
+    const int64_t left = cnt - row0;
+    const int rows_here = left < kRows ? static_cast<int>(left) : kRows;
+    resolve_listed(a.r, row0, rows_here, s_tab, s_grad, s_old);
+    // thread r wrote s_tab[r] itself: the step counter and the bias corrections of its row
+    for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+      float* sp = a.step + s_tab[r];
+      const float step = *sp + 1.0f;
+      *sp = step;
+      s_c1[r] = 1.0f - powf(a.beta1, step);
+      s_c2[r] = 1.0f - powf(a.beta2, step);
+    }
+    __syncthreads();
+    const int total = rows_here * cpr;
+    for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
+      V g[kUnroll], m[kUnroll], v[kUnroll], w[kUnroll];
+      V* mp[kUnroll];
+      V* vp[kUnroll];
+      V* wp[kUnroll];
+      float c1[kUnroll], c2[kUnroll];
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        const int c = base + k * kThreads;
+        if (c < total) {
+          const int r = c / cpr;
+          const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
+          const int64_t off = s_tab[r] * a.r.stride + col;
+          mp[k] = reinterpret_cast<V*>(a.m + off);
+          vp[k] = reinterpret_cast<V*>(a.v + off);
+          wp[k] = reinterpret_cast<V*>(a.w + off);
+          g[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(a.r.grad + s_grad[r] + col));
+          m[k] = *mp[k];
+          v[k] = *vp[k];
+          w[k] = a.r.w_rows != nullptr ? *reinterpret_cast<const V*>(a.r.w_rows + s_old[r] + col)
+                                       : *wp[k];
+          c1[k] = s_c1[r];
+          c2[k] = s_c2[r];
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        const int c = base + k * kThreads;
+        if (c < total) {
+          const V m1 = a.beta1 * m[k] + a.one_minus_beta1 * g[k];
+          const V v1 = a.beta2 * v[k] + a.one_minus_beta2 * (g[k] * g[k]);
+          const V mc = vdiv(m1, V(c1[k]));
+          const V vc = vdiv(v1, V(c2[k]));
+          const V upd = vdiv(a.lr * mc, vsqrt(vc) + a.eps);
+          *mp[k] = m1;
+          *vp[k] = v1;
+          *wp[k] = w[k] - upd;
         }
       }
     }
@@ -295,22 +396,55 @@ int check_rows(const int64_t* uids, const float* grad, int64_t max_rows, int64_t
   return HADES_OK;
 }
 
-int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
-  float* w = a.w;
-  float* s = a.s;
-  const float* grad = a.grad;
-  const int64_t max_count = a.max_count, dim = a.dim, stride = a.stride;
+// grid of a listed walk: one block per kRows rows, capped; rows that cross the host link get a
+// narrow grid that strides over the list
+dim3 listed_grid(int64_t max_count, std::initializer_list<const void*> tables) {
   int64_t blocks = ceil_div(max_count, kRows);
   if (blocks > 16384) blocks = 16384;
-  // rows that cross the host link: a narrow grid that strides over the list
-  if ((is_host_memory(w) || is_host_memory(s)) && blocks > host_link_blocks(true))
-    blocks = host_link_blocks(true);
-  const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+  bool host = false;
+  for (const void* t : tables) host = host || is_host_memory(t);
+  if (host && blocks > host_link_blocks(true)) blocks = host_link_blocks(true);
+  return dim3(static_cast<unsigned>(blocks));
+}
+
+int check_listed(const ListedRows& r, bool class_form) {
+  HADES_REQUIRE(r.max_count >= 0 && r.dim >= 1, "the row count must be >= 0 and dim >= 1");
+  HADES_REQUIRE(r.stride >= r.dim, "stride must be 0 or >= dim");
+  HADES_REQUIRE(r.dim * kRows < (int64_t(1) << 30), "dim too large");
+  if (r.max_count == 0) return HADES_OK;
+  HADES_REQUIRE(r.row_index && r.grad, "null pointer argument");
+  if (class_form) {
+    HADES_REQUIRE(r.which == 0 || r.which == 1, "which must be 0 or 1");
+    HADES_REQUIRE(r.num_unique && r.class_split, "null pointer argument");
+    HADES_REQUIRE((r.w_rows == nullptr) == (r.first_pos == nullptr),
+                  "w_rows and first_pos go together");
+  } else {
+    HADES_REQUIRE(r.list && r.count, "null pointer argument");
+  }
+  return HADES_OK;
+}
+
+int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
+  const dim3 grid = listed_grid(a.r.max_count, {a.w, a.s}), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dim % 4 == 0 && stride % 4 == 0 && aligned16({grad, w, s, a.w_rows}))
+  if (a.r.dim % 4 == 0 && a.r.stride % 4 == 0 && aligned16({a.r.grad, a.w, a.s, a.r.w_rows}))
     HADES_LAUNCH((adagrad_listed_kernel<4>), grid, block, 0, st, a);
   else
     HADES_LAUNCH((adagrad_listed_kernel<1>), grid, block, 0, st, a);
+  return HADES_OK;
+}
+
+int launch_adam_listed(const ListedRows& r, float* w, float* step, float* m, float* v, float lr,
+                       double beta1, double beta2, float eps, void* stream) {
+  // 1 - beta is formed in double and rounded once, as in hades_adam_update
+  const AdamListedArgs a{r, w, step, m, v, lr, static_cast<float>(beta1), static_cast<float>(beta2),
+                         static_cast<float>(1.0 - beta1), static_cast<float>(1.0 - beta2), eps};
+  const dim3 grid = listed_grid(r.max_count, {w, step, m, v}), block(kThreads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (r.dim % 4 == 0 && r.stride % 4 == 0 && aligned16({r.grad, w, m, v, r.w_rows}))
+    HADES_LAUNCH((adam_listed_kernel<4>), grid, block, 0, st, a);
+  else
+    HADES_LAUNCH((adam_listed_kernel<1>), grid, block, 0, st, a);
   return HADES_OK;
 }
 
@@ -345,15 +479,13 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
 int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,
                                 const int64_t* count, int64_t max_count, int64_t dim, float* w,
                                 float* s, int64_t stride, float lr, float eps, void* stream) {
-  HADES_REQUIRE(max_count >= 0 && dim >= 1, "max_count must be >= 0 and dim >= 1");
-  HADES_REQUIRE(stride == 0 || stride >= dim, "stride must be 0 or >= dim");
-  HADES_REQUIRE(dim * kRows < (int64_t(1) << 30), "dim too large");
-  if (max_count == 0) return HADES_OK;
-  HADES_REQUIRE(row_index && grad && list && count && w && s, "null pointer argument");
-  if (stride == 0) stride = dim;
-  AdagradListedArgs a{row_index, grad, list, count, max_count, nullptr, nullptr, 0, int64_t(-1),
-                      nullptr, nullptr, dim, w, s, stride, lr, eps};
-  return launch_adagrad_listed(a, stream);
+  HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
+  const ListedRows r{row_index, grad, list, count, max_count, nullptr, nullptr, 0, int64_t(-1),
+                     nullptr, nullptr, dim, stride == 0 ? dim : stride};
+  const int rc = check_listed(r, false);
+  if (rc != HADES_OK || max_count == 0) return rc;
+  HADES_REQUIRE(w && s, "null pointer argument");
+  return launch_adagrad_listed(AdagradListedArgs{r, w, s, lr, eps}, stream);
 }
 
 int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
@@ -361,17 +493,41 @@ int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const in
                                int64_t max_rows, int64_t dim, float* w, float* s, int64_t stride,
                                const float* w_rows, const int32_t* first_pos, float lr, float eps,
                                void* stream) {
-  HADES_REQUIRE(max_rows >= 0 && dim >= 1, "max_rows must be >= 0 and dim >= 1");
-  HADES_REQUIRE(stride == 0 || stride >= dim, "stride must be 0 or >= dim");
-  HADES_REQUIRE(dim * kRows < (int64_t(1) << 30), "dim too large");
-  HADES_REQUIRE(which == 0 || which == 1, "which must be 0 or 1");
-  if (max_rows == 0) return HADES_OK;
-  HADES_REQUIRE(ukeys && grad && num_unique && class_split && w && s, "null pointer argument");
-  HADES_REQUIRE((w_rows == nullptr) == (first_pos == nullptr), "w_rows and first_pos go together");
-  if (stride == 0) stride = dim;
-  AdagradListedArgs a{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
-                      key_mask, w_rows, first_pos, dim, w, s, stride, lr, eps};
-  return launch_adagrad_listed(a, stream);
+  HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
+  const ListedRows r{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
+                     key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  const int rc = check_listed(r, true);
+  if (rc != HADES_OK || max_rows == 0) return rc;
+  HADES_REQUIRE(w && s, "null pointer argument");
+  return launch_adagrad_listed(AdagradListedArgs{r, w, s, lr, eps}, stream);
+}
+
+int hades_adam_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,
+                             const int64_t* count, int64_t max_count, int64_t dim, float* w,
+                             float* step, float* m, float* v, int64_t stride, float lr,
+                             double beta1, double beta2, float eps, void* stream) {
+  HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
+  const ListedRows r{row_index, grad, list, count, max_count, nullptr, nullptr, 0, int64_t(-1),
+                     nullptr, nullptr, dim, stride == 0 ? dim : stride};
+  const int rc = check_listed(r, false);
+  if (rc != HADES_OK || max_count == 0) return rc;
+  HADES_REQUIRE(w && step && m && v, "null pointer argument");
+  return launch_adam_listed(r, w, step, m, v, lr, beta1, beta2, eps, stream);
+}
+
+int hades_adam_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
+                            const int64_t* class_split, int which, int64_t key_mask,
+                            int64_t max_rows, int64_t dim, float* w, float* step, float* m,
+                            float* v, int64_t stride, const float* w_rows,
+                            const int32_t* first_pos, float lr, double beta1, double beta2,
+                            float eps, void* stream) {
+  HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
+  const ListedRows r{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
+                     key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  const int rc = check_listed(r, true);
+  if (rc != HADES_OK || max_rows == 0) return rc;
+  HADES_REQUIRE(w && step && m && v, "null pointer argument");
+  return launch_adam_listed(r, w, step, m, v, lr, beta1, beta2, eps, stream);
 }
 
 int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,

@@ -245,6 +245,35 @@ def adagrad_update_listed_(row_index, grad, pos_list, count, w, s, lr, eps):
               pos_list.numel(), dim, _ptr(w), _ptr(s), stride, float(lr), float(eps), _stream())
 
 
+def _adam_tables(tables, dim):
+    """Checks one (w, step, mem, power) table set of the per-class Adam forms; returns the row stride."""
+    w, step, m, v = tables
+    for name, t in (("w", w), ("mem", m), ("power", v)):
+        _dev_or_pinned(t, name, contiguous=False)
+        _check(t.dtype == torch.float32 and t.dim() == 2 and t.size(1) == dim, "%s: wrong dtype/width" % name)
+    _dev_or_pinned(step, "step")
+    _check(step.dtype == torch.float32 and step.dim() == 1 and step.numel() == w.size(0),
+           "step must be float32 with one entry per table row")
+    stride = _stride_of(w, dim)
+    _check(_stride_of(m, dim) == stride and _stride_of(v, dim) == stride,
+           "w, mem and power must have the same row stride")
+    return stride
+
+
+def adam_update_listed_(row_index, grad, pos_list, count, tables, lr, beta1, beta2, eps):
+    """SparseAdam (the arithmetic of adam_update_) over the rows named by the first count[0]
+    positions p of pos_list: g = grad[p]; r = row_index[p]; one Adam step on row r of
+    `tables` = (w, step, mem, power), one table set, device or pinned host."""
+    _i64(row_index, "row_index"); _i64(pos_list, "pos_list"); _i64(count, "count"); _dev(grad, "grad")
+    _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
+    dim = grad.size(1)
+    stride = _adam_tables(tables, dim)
+    w, step, m, v = tables
+    _lib.call("hades_adam_update_listed", _ptr(row_index), _ptr(grad), _ptr(pos_list), _ptr(count),
+              pos_list.numel(), dim, _ptr(w), _ptr(step), _ptr(m), _ptr(v), stride, float(lr),
+              float(beta1), float(beta2), float(eps), _stream())
+
+
 def split3_padded(ids, class_table, workspace=None):
     """Three-way split by the int8 class table (0 local, 1 remote-hot, 2 remote-cold) with the
     compacted position lists; no host synchronisation.  Returns (masks[3], pos[3], counts[3])."""
@@ -482,6 +511,26 @@ def adagrad_update_class_(plan, sums, which, w, s, lr, eps, fetched_rows=None):
     _lib.call("hades_adagrad_update_class", _ptr(plan.uids), _ptr(sums), _ptr(plan.num_unique),
               _ptr(plan.class_split), int(which), (1 << plan.key_bits) - 1, plan.uids.numel(), dim,
               _ptr(w), _ptr(s), stride, _opt(fetched_rows), _opt(fp), float(lr), float(eps), _stream())
+
+
+def adam_update_class_(plan, sums, which, tables, lr, beta1, beta2, eps, fetched_rows=None):
+    """SparseAdam over one class of a classed plan; rows and `fetched_rows` as in
+    adagrad_update_class_, `tables` = (w, step, mem, power) of that class."""
+    _dev(sums, "sums")
+    dim = sums.size(1)
+    stride = _adam_tables(tables, dim)
+    w, step, m, v = tables
+    fp = None
+    if fetched_rows is not None:
+        _dev(fetched_rows, "fetched_rows")
+        _check(plan.first_pos is not None, "the plan was made without first_pos")
+        _check(fetched_rows.dtype == torch.float32 and tuple(fetched_rows.shape) == (plan.n, dim),
+               "fetched_rows must be float32 [n, dim]")
+        fp = plan.first_pos
+    _lib.call("hades_adam_update_class", _ptr(plan.uids), _ptr(sums), _ptr(plan.num_unique),
+              _ptr(plan.class_split), int(which), (1 << plan.key_bits) - 1, plan.uids.numel(), dim,
+              _ptr(w), _ptr(step), _ptr(m), _ptr(v), stride, _opt(fetched_rows), _opt(fp),
+              float(lr), float(beta1), float(beta2), float(eps), _stream())
 
 
 def combine(idx, grad, id_bound=0, mode=COMBINE_FAST, workspace=None):

@@ -394,6 +394,18 @@ class SparseAdam(_SparseRowOptimizer):
         self.hot_m = torch.zeros_like(self.hot_w)
         self.hot_v = torch.zeros_like(self.hot_w)
 
+    def _tables(self, hot):
+        return ((self.hot_w, self.hot_step, self.hot_m, self.hot_v) if hot else
+                (self.cold_w, self.cold_step, self.cold_m, self.cold_v))
+
+    def _update_class(self, index, grad, pos, count, hot):
+        ops.adam_update_listed_(index, grad, pos, count, self._tables(hot), self.lr,
+                                self.betas[0], self.betas[1], self.eps)
+
+    def _update_keyed(self, plan, sums, which, fetched_rows=None):
+        ops.adam_update_class_(plan, sums, which, self._tables(bool(which)), self.lr,
+                               self.betas[0], self.betas[1], self.eps, fetched_rows=fetched_rows)
+
     def update(self, uids, grad, num_unique=None):
         ops.adam_update_(uids, grad, (self.hot_w, self.hot_step, self.hot_m, self.hot_v),
                          (self.cold_w, self.cold_step, self.cold_m, self.cold_v), self.hot_set,

@@ -384,6 +384,25 @@ int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num
                       float* cold_w, float* cold_step, float* cold_m, float* cold_v,
                       float lr, double beta1, double beta2, float eps, void* stream);
 
+/* The SparseAdam arithmetic of hades_adam_update over one half of a split, against one table
+ * set (the per-class form of python/EmbCache/sparse_optim.py:590-685 with the state gathers and
+ * scatters of python/EmbCache/cache.py:66-131 fused in): positions, row_index, list and count as
+ * in hades_adagrad_update_listed; step is float[rows of the table]; w, m and v have rows `stride`
+ * floats apart (0 = dim) and may be device or pinned host memory. */
+int hades_adam_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,
+                             const int64_t* count, int64_t max_count, int64_t dim, float* w,
+                             float* step, float* m, float* v, int64_t stride, float lr,
+                             double beta1, double beta2, float eps, void* stream);
+
+/* SparseAdam over one class of a class-ordered combine; arguments as in
+ * hades_adagrad_update_class, tables as in hades_adam_update_listed. */
+int hades_adam_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
+                            const int64_t* class_split, int which, int64_t key_mask,
+                            int64_t max_rows, int64_t dim, float* w, float* step, float* m,
+                            float* v, int64_t stride, const float* w_rows,
+                            const int32_t* first_pos, float lr, double beta1, double beta2,
+                            float eps, void* stream);
+
 /* Cold-gradient accumulator (delayed synchronisation): an open-addressing hash table in HBM,
  * int64 key -> fp32[dim] running sum and an int64 count.  Restates on the GPU the arithmetic of
  * EmbCacheServer._accumulate_gradients_cold_remote (python/EmbCache/server.py:546-562): per unique

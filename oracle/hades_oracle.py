@@ -278,6 +278,18 @@ def adagrad_listed(row_index, grad, pos_list, count, w, s, lr, eps):
     s[rows] = s1
 
 
+def adam_listed(row_index, grad, pos_list, count, w, step, m, v, lr, beta1, beta2, eps):
+    """adam_rows on the rows row_index[p] of (w, step, m, v) with gradient grad[p], p over the
+    first `count` positions of pos_list; in place (the per-class form of
+    python/EmbCache/sparse_optim.py:590-685)."""
+    pos = np.asarray(pos_list, dtype=np.int64)[: max(0, int(count))]
+    rows = np.asarray(row_index, dtype=np.int64)[pos]
+    if rows.size == 0:
+        return
+    w[rows], step[rows], m[rows], v[rows] = adam_rows(w[rows], step[rows], m[rows], v[rows],
+                                                      np.asarray(grad)[pos], lr, beta1, beta2, eps)
+
+
 def sparse_adagrad_step_split(cold_w, cold_s, hot_w, hot_s, sorted_hot, uids, g, lr, eps,
                               num_live=None):
     """sparse_adagrad_step done class by class; must equal sparse_adagrad_step."""
@@ -317,6 +329,30 @@ def keyed_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps, key_b
     slots = ukeys[split:] - thr
     w1, s1 = adagrad_rows(hot_w[slots], hot_s[slots], sums[split:], lr, eps)
     hot_w[slots], hot_s[slots] = w1, s1
+    return ukeys, sums, cnts, split
+
+
+def keyed_step_adam(cold, hot, sorted_hot, q, grad, lr, beta1, beta2, eps, key_bits,
+                    fetched_rows=None):
+    """keyed_step with the reference's SparseAdam arithmetic (adam_rows) in place of Adagrad.
+    `cold` and `hot` are (w, step, m, v) table sets, updated in place.  Must equal
+    combine_sequential on the ids followed by adam_rows on the gathered rows of each id.
+    Returns (ukeys, sums, cnts, first hot run)."""
+    keys = class_ordered_keys(q, sorted_hot, key_bits)
+    ukeys, sums, cnts = combine_sequential(keys, grad)
+    thr = np.int64(1) << np.int64(key_bits)
+    split = int(np.searchsorted(ukeys, thr, side="left"))
+    for tabs, rows, g, is_cold in ((cold, ukeys[:split], sums[:split], True),
+                                   (hot, ukeys[split:] - thr, sums[split:], False)):
+        if rows.size == 0:
+            continue
+        w, step, m, v = tabs
+        old = w[rows]
+        if is_cold and fetched_rows is not None:
+            first = np.array([np.flatnonzero(keys == k)[0] for k in rows], dtype=np.int64)
+            old = np.asarray(fetched_rows)[first]
+        w[rows], step[rows], m[rows], v[rows] = adam_rows(old, step[rows], m[rows], v[rows], g,
+                                                          lr, beta1, beta2, eps)
     return ukeys, sums, cnts, split
 
 

@@ -76,6 +76,20 @@ def test_argument_errors_of_the_split_schedule_entry_points():
     assert lib.hades_adagrad_update_class(one, one, one, one, 0, 255, 10, 8, one, one, 0, one, null,
                                           0.01, 1e-10, null) == 1                              # rows without positions
     assert b"go together" in lib.hades_last_error()
+    # listed / class Adam
+    assert lib.hades_adam_update_listed(one, one, one, one, 10, 8, one, one, one, one, 4, 0.01, 0.9, 0.999,
+                                        1e-8, null) == 1                                       # stride < dim
+    assert lib.hades_adam_update_listed(one, one, one, one, 10, 8, one, null, one, one, 0, 0.01, 0.9, 0.999,
+                                        1e-8, null) == 1                                       # step table
+    assert lib.hades_adam_update_listed(null, null, null, null, 0, 8, null, null, null, null, 0, 0.01, 0.9,
+                                        0.999, 1e-8, null) == 0
+    assert lib.hades_adam_update_class(one, one, one, one, 3, 255, 10, 8, one, one, one, one, 0, null, null,
+                                       0.01, 0.9, 0.999, 1e-8, null) == 1                      # which
+    assert lib.hades_adam_update_class(one, one, one, one, 1, 255, 10, 8, one, one, one, one, 0, null, one,
+                                       0.01, 0.9, 0.999, 1e-8, null) == 1
+    assert b"go together" in lib.hades_last_error()
+    assert lib.hades_adam_update_class(null, null, null, null, 0, 255, 0, 8, null, null, null, null, 0, null,
+                                       null, 0.01, 0.9, 0.999, 1e-8, null) == 0
     # lookup + split: key bits must leave room for the slots
     assert lib.hades_lookup_split(one, null, 10, one, 1 << 20, null, one, null, one, one, one, one, 8,
                                   one, 1 << 20, null) == 1

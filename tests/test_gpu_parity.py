@@ -1557,3 +1557,101 @@ def test_listed_gather_and_scatter_row_shapes(lib, dim, fdt, host):
         ops.fetch_listed(flat, dev(idx), dev(pos), cnt, o1)
         w1 = O.fetch_listed(flat.cpu().numpy(), idx, pos, pos.size - 7, np.zeros(n, NP_F[fdt]))
         assert np.array_equal(o1.cpu().numpy(), w1)
+
+
+def _adam_close(got, want, k, lr=0.01):
+    """tolerances of test_adam_update: weights to 1e-4 of one update, step exact, moments to rounding"""
+    if got.size == 0:
+        return got.shape == want.shape
+    if k == 0:
+        return np.abs(got - want).max() <= 1e-4 * lr
+    if k == 1:
+        return np.array_equal(got, want)
+    return np.allclose(got, want, rtol=1e-6, atol=1e-12)
+
+
+@pytest.mark.parametrize("N,D,H,n,hot_frac", [
+    (5000, 128, 500, 20_000, 0.9), (5000, 64, 500, 20_000, 1.0), (5000, 64, 500, 20_000, 0.0),
+    (5000, 7, 0, 3000, 0.0), (70_000, 128, 9000, 257, 0.5), (10, 4, 3, 0, 0.5),
+])
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_sparse_adam_on_the_split_and_keyed_schedules(lib, N, D, H, n, hot_frac, host_cold):
+    """SparseAdam class by class (hades_adam_update_listed through step_split,
+    hades_adam_update_class through forward_keyed / backward_keyed) against (1) the one-kernel
+    form on the same batch, whose arithmetic is the same instruction sequence: all eight tables
+    bit-equal in the deterministic-order mode, and (2) the oracle's per-class restatement of the
+    reference's SparseAdam.update (python/EmbCache/sparse_optim.py:590-685) to the tolerances of
+    test_adam_update."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdam
+    rng = np.random.default_rng(N + n + int(10 * hot_frac) + 7)
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, hot_frac)
+    if n > 1000:
+        q[: n // 8] = q[0]
+    kb = ops.key_bits_for(max(N, H, 2))
+
+    def make():
+        t = torch.from_numpy(cold.copy())
+        return SparseAdam(t.pin_memory() if host_cold else t.cuda(), torch.from_numpy(hot_ids), lr=0.01)
+
+    one, split, keyed = make(), make(), make()
+    ocold = (cold.copy(), np.zeros(N, np.float32), np.zeros_like(cold), np.zeros_like(cold))
+    ohot = (cold[hot_ids].copy(), np.zeros(H, np.float32), np.zeros((H, D), np.float32),
+            np.zeros((H, D), np.float32))
+    t_q = dev(q)
+    for it in range(3):
+        grad = (rng.standard_normal((n, D)) * 1e-2).astype(np.float32)
+        t_g = dev(grad)
+        one.step(t_q, t_g, mode=ops.COMBINE_EXACT)
+        split.step_split(t_q, t_g, mode=ops.COMBINE_EXACT)
+        rows, state = keyed.forward_keyed(t_q)
+        assert np.array_equal(rows.cpu().numpy(), O.cached_fetch(ocold[0], ohot[0], q, hot_ids))
+        keyed.backward_keyed(state, t_g, mode=ops.COMBINE_EXACT)
+        torch.cuda.synchronize()
+        O.keyed_step_adam(ocold, ohot, hot_ids, q, grad, 0.01, 0.9, 0.999, 1e-8, kb)
+        # the oracle's weights drift from the device's by the tolerance of each step: restart it
+        # from the device's tables so that every step is checked on its own
+        for k, name in enumerate(("w", "step", "m", "v")):
+            for tabs, o, hot in ((ocold, one, False), (ohot, one, True)):
+                got = getattr(o, ("hot_" if hot else "cold_") + name).cpu().numpy()
+                assert _adam_close(got, tabs[k], k), (it, name, hot)
+                tabs[k][...] = got
+    for name in ("w", "step", "m", "v"):
+        for pre in ("hot_", "cold_"):
+            a = getattr(one, pre + name).cpu()
+            assert torch.equal(a, getattr(split, pre + name).cpu()), pre + name
+            assert torch.equal(a, getattr(keyed, pre + name).cpu()), pre + name
+
+
+def test_sparse_adam_keyed_with_the_forward_rows(lib):
+    """backward_keyed(fetched_rows=...) with SparseAdam: untouched rows give the plain result bit
+    for bit; rows altered on purpose move the cold weights by exactly the alteration."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdam
+    rng = np.random.default_rng(99)
+    N, D, H, n = 20_000, 64, 2000, 30_000
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, 0.6)
+    grad = (rng.standard_normal((n, D)) * 1e-2).astype(np.float32)
+
+    def make():
+        return SparseAdam(torch.from_numpy(cold.copy()).pin_memory(), torch.from_numpy(hot_ids))
+
+    plain, reuse, altered = make(), make(), make()
+    t_q, t_g = dev(q), dev(grad)
+    rows, st = plain.forward_keyed(t_q)
+    plain.backward_keyed(st, t_g, mode=ops.COMBINE_EXACT)
+    rows2, st2 = reuse.forward_keyed(t_q)
+    reuse.backward_keyed(st2, t_g, mode=ops.COMBINE_EXACT, fetched_rows=rows2)
+    rows3, st3 = altered.forward_keyed(t_q)
+    altered.backward_keyed(st3, t_g, mode=ops.COMBINE_EXACT, fetched_rows=rows3 + 0.25)
+    torch.cuda.synchronize()
+    for name in ("w", "step", "m", "v"):
+        for pre in ("hot_", "cold_"):
+            assert torch.equal(getattr(plain, pre + name).cpu(), getattr(reuse, pre + name).cpu())
+            if pre + name != "cold_w":
+                assert torch.equal(getattr(plain, pre + name).cpu(), getattr(altered, pre + name).cpu())
+    touched = np.unique(q[O.lookup_sorted(q, hot_ids) < 0])
+    diff = altered.cold_w.numpy() - plain.cold_w.numpy()
+    assert np.allclose(diff[touched], 0.25, atol=1e-6)
+    mask = np.ones(N, bool); mask[touched] = False
+    assert np.array_equal(diff[mask], np.zeros_like(diff[mask]))

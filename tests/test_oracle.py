@@ -645,3 +645,43 @@ def test_keyed_step_equals_combine_then_update_on_the_ids():
                  fetched_rows=O.cached_fetch(c[0], c[2], q, hot_ids))
     for x, y in zip(b, c):
         assert np.array_equal(x, y)
+
+
+def test_keyed_step_adam_equals_combine_then_adam_on_the_ids():
+    """keyed_step_adam (class-ordered keys, per-class tables) must give what the reference's flow
+    gives on the ids: unique + index_add (only_unique_grads, python/EmbCache/sparse_optim.py:132-139)
+    and then adam_rows on the gathered rows of each distinct id (:590-685), whichever table holds
+    the row.  Also adam_listed class by class."""
+    rng = np.random.default_rng(5)
+    N, D, H, n = 400, 8, 60, 1500
+    hot_ids = np.sort(rng.choice(N, H, replace=False)).astype(np.int64)
+    w0 = rng.standard_normal((N, D)).astype(np.float32)
+    q = rng.integers(0, N, n).astype(np.int64)
+    kb = 9
+    cold = (w0.copy(), np.zeros(N, np.float32), np.zeros_like(w0), np.zeros_like(w0))
+    hot = tuple(x[hot_ids].copy() for x in cold)
+    full = tuple(x.copy() for x in cold)                  # one table, no cache: the plain flow
+    lcold = tuple(x.copy() for x in cold)
+    lhot = tuple(x.copy() for x in hot)
+    for it in range(3):
+        grad = rng.standard_normal((n, D)).astype(np.float32)
+        ukeys, sums, cnts, split = O.keyed_step_adam(cold, hot, hot_ids, q, grad, 0.01, 0.9, 0.999, 1e-8, kb)
+        uids, usum, ucnt = O.combine_sequential(q, grad)
+        res = O.adam_rows(full[0][uids], full[1][uids], full[2][uids], full[3][uids], usum,
+                          0.01, 0.9, 0.999, 1e-8)
+        for k in range(4):
+            full[k][uids] = res[k]
+        # the listed form on the distinct ids
+        loc, hot_pos, cold_pos = O.lookup_split(uids, hot_ids)
+        O.adam_listed(loc, usum, hot_pos, hot_pos.size, *lhot, 0.01, 0.9, 0.999, 1e-8)
+        O.adam_listed(uids, usum, cold_pos, cold_pos.size, *lcold, 0.01, 0.9, 0.999, 1e-8)
+        assert split == (O.lookup_sorted(uids, hot_ids) < 0).sum()
+    is_hot = np.zeros(N, bool); is_hot[hot_ids] = True
+    for k in range(4):
+        merged = cold[k].copy(); merged[hot_ids] = hot[k]
+        assert np.array_equal(merged, full[k])
+        lm = lcold[k].copy(); lm[hot_ids] = lhot[k]
+        assert np.array_equal(lm, full[k])
+        # the cold table's rows of hot ids were never touched
+        init = (w0, np.zeros(N, np.float32), np.zeros_like(w0), np.zeros_like(w0))[k]
+        assert np.array_equal(cold[k][is_hot], init[is_hot])
