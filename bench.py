@@ -58,6 +58,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours", "random-rows"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
+    ap.add_argument("--optimizer", default="adagrad", choices=["adagrad", "adam"],
+                    help="row update of the step: sparse Adagrad (the configurations' optimizer) or "
+                         "the reference's SparseAdam (cfg2 / cfg3 / cfg5 steps only)")
     ap.add_argument("--schedule", default=None, choices=["serial", "keyed", "split", "overlap", "graph"],
                     help="serial: every kernel of the step on one stream, hot and cold rows in the "
                          "same kernels (default when the whole table is in HBM); keyed: one lookup + "
@@ -112,10 +115,11 @@ class Workload:
     """Tables, hot set and pre-generated batches of one configuration, resident on the device
     (cold table in pinned host memory for cfg3)."""
 
-    def __init__(self, name, nbatches, device):
+    def __init__(self, name, nbatches, device, optimizer="adagrad"):
         import torch
         from hades_amd import synth
-        from hades_amd.sparse_optim import SparseAdagrad
+        from hades_amd.sparse_optim import SparseAdagrad, SparseAdam
+        self.optimizer = optimizer
         cfg = synth.CONFIGS[name]
         self.name, self.cfg = name, cfg
         N, D, H = cfg["num_rows"], cfg["dim"], cfg["num_hot"]
@@ -138,8 +142,12 @@ class Workload:
         # The benchmark box refuses a page-locked allocation that would hold weights and state
         # together (113.7 GB in one piece: hipHostMalloc says out of memory; 56.8 GB is granted),
         # and 288 GB of HBM have the room.
-        self.opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=device,
-                                 state_on_device=self.host_cold)
+        if optimizer == "adam":      # its cold step / mem / power tables stay in HBM likewise
+            self.opt = SparseAdam(table, hot_ids, lr=0.01, betas=(0.9, 0.999), eps=1e-8, device=device,
+                                  state_on_device=self.host_cold)
+        else:
+            self.opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=device,
+                                     state_on_device=self.host_cold)
         log("sampling %d batches of %d ids" % (nbatches, self.n))
         sampler = synth.ZipfSampler(N, cfg["zipf_s"], device)
         self.ids, self.grads = [], []
@@ -160,7 +168,7 @@ class Workload:
         return ("%s: %d x %d fp32 table (%s), hot %d rows in HBM, %d ids/step zipf s=%.2f%s" %
                 (self.name, self.N, self.D,
                  "cold weights in pinned host memory read and written zero-copy; deviation: cold "
-                 "Adagrad state in HBM, the box refuses the 113.7 GB page-locked allocation that "
+                 "optimizer state in HBM, the box refuses the 113.7 GB page-locked allocation that "
                  "would hold weights and state" if self.host_cold
                  else "all in HBM", self.H, self.n, self.cfg["zipf_s"],
                  ", %d trainer batches concatenated" % self.trainers if self.trainers > 1 else ""))
@@ -281,7 +289,20 @@ def parity_gate(wl, step_fn, rows=20_000):
     sums64 = torch.zeros((uniq.numel(), wl.D), dtype=torch.float64, device=q.device)
     sums64.index_add_(0, inv, g.double())
     w0, _ = table_rows(opt.cold_w, opt.hot_w, uniq)
-    s0, _ = table_rows(opt.cold_s, opt.hot_s, uniq)
+    adam = wl.optimizer == "adam"
+    if adam:
+        m0, loc_u = table_rows(opt.cold_m, opt.hot_m, uniq)
+        v0, _ = table_rows(opt.cold_v, opt.hot_v, uniq)
+
+        def steps_of():
+            hit = loc_u >= 0
+            st = opt.cold_step[uniq].clone()
+            if hot.numel():
+                st[hit] = opt.hot_step[loc_u[hit]]
+            return st
+        st0 = steps_of()
+    else:
+        s0, _ = table_rows(opt.cold_s, opt.hot_s, uniq)
 
     rows_out, (uids, sums, cnts, nu) = step_fn(q, g, ops.COMBINE_EXACT)
     torch.cuda.synchronize()
@@ -299,17 +320,34 @@ def parity_gate(wl, step_fn, rows=20_000):
 
     e_sum = close(sums[:u], sums64, "summed gradients")
     gs = sums[:u]
-    s1 = s0 + gs * gs
-    w1 = w0 - (0.01 * gs) / (s1.sqrt() + 1e-10)
     w_got, _ = table_rows(opt.cold_w, opt.hot_w, uniq)
-    s_got, _ = table_rows(opt.cold_s, opt.hot_s, uniq)
-    e_w = close(w_got, w1, "updated weights")
-    e_s = close(s_got, s1, "updated Adagrad state")
+    if adam:
+        # the reference's float32 arithmetic (python/EmbCache/sparse_optim.py:632-657,681) in torch
+        b1, b2 = opt.betas
+        st1 = st0 + 1
+        m1 = b1 * m0 + (1.0 - b1) * gs
+        v1 = b2 * v0 + (1.0 - b2) * (gs * gs)
+        c1 = (1.0 - torch.pow(torch.tensor(b1, device=q.device), st1)).unsqueeze(1)
+        c2 = (1.0 - torch.pow(torch.tensor(b2, device=q.device), st1)).unsqueeze(1)
+        w1 = w0 - 0.01 * (m1 / c1) / (torch.sqrt(v1 / c2) + opt.eps)
+        m_got, _ = table_rows(opt.cold_m, opt.hot_m, uniq)
+        v_got, _ = table_rows(opt.cold_v, opt.hot_v, uniq)
+        assert torch.equal(steps_of(), st1), "parity gate: Adam step counters differ"
+        errs = {"sums": e_sum, "weights": close(w_got, w1, "updated weights"),
+                "mem": close(m_got, m1, "updated Adam mem"), "power": close(v_got, v1, "updated Adam power")}
+        form = "SparseAdam closed form in float32, first step of every row"
+    else:
+        s1 = s0 + gs * gs
+        w1 = w0 - (0.01 * gs) / (s1.sqrt() + 1e-10)
+        s_got, _ = table_rows(opt.cold_s, opt.hot_s, uniq)
+        errs = {"sums": e_sum, "weights": close(w_got, w1, "updated weights"),
+                "state": close(s_got, s1, "updated Adagrad state")}
+        form = "Adagrad closed form"
     return {"rows": m, "distinct": u, "mode": "exact",
-            "bit_exact": ["lookup slots", "fetched rows", "distinct ids", "counts"],
-            "max_rel_err": {"sums": e_sum, "weights": e_w, "state": e_s}, "tolerance": 1e-5,
-            "against": "torch device ops (searchsorted, indexing, unique + float64 index_add_, "
-                       "Adagrad closed form)"}
+            "bit_exact": ["lookup slots", "fetched rows", "distinct ids", "counts"] +
+                         (["Adam step counters"] if adam else []),
+            "max_rel_err": errs, "tolerance": 1e-5,
+            "against": "torch device ops (searchsorted, indexing, unique + float64 index_add_, %s)" % form}
 
 
 def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows=False):
@@ -317,7 +355,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
     from hades_amd import ops
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    wl = Workload(workload, args.batches, dev)
+    wl = Workload(workload, args.batches, dev, args.optimizer)
     opt = wl.opt
     mode = ops.COMBINE_FAST if args.mode == "fast" else ops.COMBINE_EXACT
     nb = len(wl.ids)
@@ -427,20 +465,21 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
     sampled = [i for i in range(K) if i % every == 0]
     seg_name = "seg_chunk_kernel" if args.mode == "fast" else "seg_exact_kernel + seg_exact_long_kernel"
     if split or keyed:
-        upd = "hades_adagrad_update_class" if keyed else "hades_adagrad_update_listed"
+        oname = args.optimizer
+        upd = "hades_%s_update_class" % oname if keyed else "hades_%s_update_listed" % oname
         knames = {"hot_fetch": "row_move_listed_kernel<gather> over the hot class (hades_fetch_listed)",
                   "cold_fetch": "row_move_listed_kernel<gather> over the cold class (hades_fetch_listed)",
                   "seg_sum": seg_name + (" over the hot class (hades_combine_apply_class)" if keyed
                                          else " (hades_combine_apply)"),
-                  "hot_update": "adagrad_listed_kernel over the hot class (%s)" % upd,
-                  "cold_update": "adagrad_listed_kernel over the cold class (%s)" % upd}
+                  "hot_update": "%s_listed_kernel over the hot class (%s)" % (oname, upd),
+                  "cold_update": "%s_listed_kernel over the cold class (%s)" % (oname, upd)}
         hook_of = {"seg_sum": ops.KERNEL_SEG_SUM}
     else:
         knames = {"fetch": "row_move_kernel<AddrFetchSorted> (hades_cached_fetch)",
                   "seg_sum": seg_name + " (hades_combine_apply)",
-                  "update": "adagrad_kernel (hades_adagrad_update)"}
+                  "update": "%s_kernel (hades_%s_update)" % (args.optimizer, args.optimizer)}
         hook_of = {"fetch": ops.KERNEL_CACHED_FETCH, "seg_sum": ops.KERNEL_SEG_SUM,
-                   "update": ops.KERNEL_ADAGRAD}
+                   "update": ops.KERNEL_ADAM if args.optimizer == "adam" else ops.KERNEL_ADAGRAD}
     kev = {i: {k: new_events(2) for k in knames} for i in sampled}
     step_ev = new_events(K + 1)
     phase_ev = [new_events(4) for _ in range(K)]
@@ -551,13 +590,17 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
     # fetch 16 + 8D per query row; segmented sum n(8+4D) read + U*4D written; Adagrad 8 + 20D per
     # distinct row.  A cold row moves 4D bytes over the host link in the fetch and 4D each way in
     # the update (weights; the cold Adagrad state sits in HBM).
-    row_f, row_u = 16 + 8 * D, 8 + 20 * D
+    # (SparseAdam: 16 + 28D - the id, the step counter both ways, and g, mem, power, w read,
+    # mem, power, w written.)
+    row_f, row_u = 16 + 8 * D, (16 + 28 * D) if args.optimizer == "adam" else (8 + 20 * D)
     alg_bytes = {"fetch": n * row_f, "combine": n * (8 + 4 * D) + U * (16 + 4 * D), "update": U * row_u}
     kbytes = {"fetch": n * row_f, "update": U * row_u,
               "seg_sum": (n_hot * (8 + 4 * D) + U_hot * 4 * D) if keyed else (n * (8 + 4 * D) + U * 4 * D),
               "hot_fetch": n_hot * row_f, "cold_fetch": n_cold * row_f,
               "hot_update": U_hot * row_u, "cold_update": U_cold * row_u}
     traffic = measured_traffic(workload, args.mode)
+    if args.optimizer != "adagrad":     # the committed counters are those of the Adagrad kernels
+        traffic = {k: v for k, v in traffic.items() if "update" not in k}
     kernels = {}
     for k, name in knames.items():
         if not kernel_ms[k]:
@@ -1138,6 +1181,14 @@ def main():
     if args.workload == "random-rows":
         run_random_rows(args)
         return
+    if args.optimizer != "adagrad":
+        if args.workload == "cfg1":
+            print("cfg1 is the CPU reference case: it runs with the configurations' Adagrad only",
+                  file=sys.stderr)
+            sys.exit(2)
+        # the secondary runs and the CPU baseline are those of the configurations' optimizer
+        args.no_secondary = True
+        args.no_cpu_baseline = True
     res = run_gpu(args, args.workload, args.schedule, reuse_rows=args.reuse_rows)
     ms_per_step = res.pop("ms_per_step")
     n = res.pop("n")
@@ -1158,7 +1209,9 @@ def main():
         "config": {"workload": res.pop("workload") + (
                        "; cold update reuses the rows fetched by the same step" if args.reuse_rows else ""),
                    "combine_mode": args.mode,
-                   "optimizer": "sparse Adagrad lr=0.01 eps=1e-10",
+                   "optimizer": ("SparseAdam lr=0.01 betas=(0.9, 0.999) eps=1e-8 (the reference's "
+                                 "optimizer; the configurations name Adagrad)" if args.optimizer == "adam"
+                                 else "sparse Adagrad lr=0.01 eps=1e-10"),
                    "schedule": {"serial": "one stream, hot and cold rows in the same kernels",
                                 "split": "lookup + hot/cold partition; hot rows on the main stream, "
                                          "cold rows on a second stream of the same priority",

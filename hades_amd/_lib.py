@@ -25,6 +25,7 @@ _L = c_int64
 # name -> argument types; every function returns int unless listed in _RESTYPE
 KERNEL_NONE, KERNEL_CACHED_FETCH, KERNEL_SEG_SUM, KERNEL_ADAGRAD, KERNEL_RADIX_PASS = 0, 1, 2, 3, 4
 KERNEL_HASH_ACCUMULATE = 5
+KERNEL_ADAM = 6
 
 _SIGNATURES = {
     "hades_profile_kernel": [c_int, _P, _P],

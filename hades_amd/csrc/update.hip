@@ -552,9 +552,9 @@ int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num
   const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dim % 4 == 0 && aligned16({grad, hot_w, hot_m, hot_v, cold_w, cold_m, cold_v}))
-    HADES_LAUNCH((adam_kernel<4>), grid, block, 0, st, a);
+    HADES_LAUNCH_TIMED(HADES_KERNEL_ADAM, st, (adam_kernel<4>), grid, block, 0, st, a);
   else
-    HADES_LAUNCH((adam_kernel<1>), grid, block, 0, st, a);
+    HADES_LAUNCH_TIMED(HADES_KERNEL_ADAM, st, (adam_kernel<1>), grid, block, 0, st, a);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }

@@ -79,6 +79,7 @@ KERNEL_SEG_SUM = _lib.KERNEL_SEG_SUM
 KERNEL_ADAGRAD = _lib.KERNEL_ADAGRAD
 KERNEL_RADIX_PASS = _lib.KERNEL_RADIX_PASS
 KERNEL_HASH_ACCUMULATE = _lib.KERNEL_HASH_ACCUMULATE
+KERNEL_ADAM = _lib.KERNEL_ADAM
 
 
 def profile_kernel(kernel_id, start=None, stop=None):

@@ -65,7 +65,8 @@ int hades_version(void);
 #define HADES_KERNEL_ADAGRAD 3      /* hades_adagrad_update */
 #define HADES_KERNEL_RADIX_PASS 4   /* scatter passes of the sort in hades_combine (the pair keeps the last pass) */
 #define HADES_KERNEL_HASH_ACCUMULATE 5 /* hades_hash_accumulate */
-#define HADES_KERNEL_LAST 5
+#define HADES_KERNEL_ADAM 6         /* hades_adam_update */
+#define HADES_KERNEL_LAST 6
 int hades_profile_kernel(int kernel_id, void* start_event, void* stop_event);
 
 /* ------------------------------------------------------------------------- */
