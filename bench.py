@@ -1,7 +1,7 @@
 """Benchmark of the embedding-cache hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]      the headline workload (cfg3) + cfg2 nested
-    python bench.py --workload cfg2|cfg3|cfg5 [--mode fast|exact] [--schedule serial|keyed|split|overlap|graph]
+    python bench.py --workload cfg2|cfg3|cfg5 [--mode fast|exact] [--schedule serial|keyed|pipelined|split|overlap|graph]
     python bench.py --workload cfg4          cold-gradient accumulator with delayed write-back
     python bench.py --workload cfg4 --flush-rule staleness    the cache server's own per-row rule
     python bench.py --workload neighbours    pre-exchange bucketing, index cache, cold-data cache
@@ -61,7 +61,7 @@ def parse_args():
     ap.add_argument("--optimizer", default="adagrad", choices=["adagrad", "adam"],
                     help="row update of the step: sparse Adagrad (the configurations' optimizer) or "
                          "the reference's SparseAdam (cfg2 / cfg3 / cfg5 steps only)")
-    ap.add_argument("--schedule", default=None, choices=["serial", "keyed", "split", "overlap", "graph"],
+    ap.add_argument("--schedule", default=None, choices=["serial", "keyed", "pipelined", "split", "overlap", "graph"],
                     help="serial: every kernel of the step on one stream, hot and cold rows in the "
                          "same kernels (default when the whole table is in HBM); keyed: one lookup + "
                          "hot/cold partition per batch, hot rows on one stream, cold rows on "
@@ -182,7 +182,8 @@ def link_probe(dev, nbytes=256 << 20, reps=4):
     h2 = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
     d1 = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     d2 = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    from hades_amd.sparse_optim import side_stream     # no further streams: see side_stream
+    s1, s2 = side_stream(dev, 0), side_stream(dev, 1)
 
     def h2d():
         with torch.cuda.stream(s1):
@@ -224,7 +225,8 @@ def link_kernel_probe(wl, reps=3):
     rows = wl.rows_out
     ops.fetch_listed(opt.cold_w, q, cold_pos, cnt, rows)
     src = rows.clone()
-    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    from hades_amd.sparse_optim import side_stream
+    s1, s2 = side_stream(opt.device, 0), side_stream(opt.device, 1)
     mb = n_cold * wl.D * 4 / 1e6
 
     def gather():
@@ -364,7 +366,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
     if schedule is None:
         schedule = "keyed" if wl.host_cold else "serial"
     split = schedule == "split"
-    keyed = schedule == "keyed"
+    pipelined = schedule == "pipelined"
+    keyed = schedule == "keyed" or pipelined     # pipelined: the keyed kernels, two batches in flight
     overlap = schedule == "overlap"
 
     def new_events(count):
@@ -423,12 +426,57 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         if events: events[3].record()
         return rows, res
 
+    # pipelined schedule: step i = the forward half of batch i+1 started on side streams
+    # (prefetch_keyed), the backward half of batch i, then the completion of batch i+1's rows
+    # (hot gather behind the hot update, refresh of the cold rows that update wrote).  `pipe`
+    # carries batch i's rows and plan from step to step; a step whose batch is not the one in
+    # flight runs that batch's forward half first (only ever extra work).
+    pipe = {"i": None}
+    row_bufs = [wl.rows_out, torch.empty_like(wl.rows_out)] if pipelined else None
+
+    def prime(i):
+        rows, st = opt.forward_keyed(wl.ids[i % nb], out=row_bufs[i % 2], slot=i % 2)
+        pipe.update(i=i, rows=rows, state=st)
+
+    def pipe_step(i, cmode, events=None, timing=None):
+        if pipe["i"] != i:
+            prime(i)
+        rows, st = pipe["rows"], pipe["state"]
+        if events: events[0].record()
+        nxt = opt.prefetch_keyed(wl.ids[(i + 1) % nb], slot=(i + 1) % 2, out=row_bufs[(i + 1) % 2],
+                                 timing=timing)
+        if events: events[1].record()
+        if events: events[2].record()
+        res = opt.backward_keyed(st, wl.grads[i % nb], cmode, timing=timing,
+                                 fetched_rows=rows if reuse_rows else None, join=False)
+        rows2, st2 = opt.finish_prefetch(nxt, after=st, timing=timing)
+        if events: events[3].record()
+        pipe.update(i=i + 1, rows=rows2, state=st2)
+        return rows, res
+
     def step(i, events=None, timing=None):
-        run_step(wl.ids[i % nb], wl.grads[i % nb], mode, events, timing)
+        if pipelined:
+            pipe_step(i, mode, events, timing)
+        else:
+            run_step(wl.ids[i % nb], wl.grads[i % nb], mode, events, timing)
 
     def gate_step(q, g, m):
         """one step for the parity gate: rows and the distinct rows in id order"""
-        rows, res = run_step(q, g, m)
+        if pipelined:
+            # batch (q, g) through the pipelined calls, with the same ids prefetched as the next
+            # batch: every cold row of that next batch is written by this batch's update, so its
+            # rows are right only if the refresh works - checked against the one-kernel fetch
+            rows, st = opt.forward_keyed(q, out=row_bufs[0][:q.numel()], slot=0)
+            rows = rows.clone()
+            nxt = opt.prefetch_keyed(q, slot=1, out=row_bufs[1][:q.numel()])
+            res = opt.backward_keyed(st, g, m, fetched_rows=rows if reuse_rows else None, join=False)
+            rows2, _ = opt.finish_prefetch(nxt, after=st)
+            torch.cuda.synchronize()
+            want2 = ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_set)
+            assert torch.equal(rows2, want2), "parity gate: rows prefetched across an update differ"
+            pipe["i"] = None
+        else:
+            rows, res = run_step(q, g, m)
         if keyed:
             ukeys, sums, cnts, nu, _ = res
             ids = opt.distinct_ids_of(ukeys, nu)
@@ -473,6 +521,9 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
                                          else " (hades_combine_apply)"),
                   "hot_update": "%s_listed_kernel over the hot class (%s)" % (oname, upd),
                   "cold_update": "%s_listed_kernel over the cold class (%s)" % (oname, upd)}
+        if pipelined:
+            knames["cold_refresh"] = ("row_move_listed_kernel<gather, filter>: the next batch's cold rows "
+                                      "that this batch's update wrote, read again (hades_fetch_listed_in_set)")
         hook_of = {"seg_sum": ops.KERNEL_SEG_SUM}
     else:
         knames = {"fetch": "row_move_kernel<AddrFetchSorted> (hades_cached_fetch)",
@@ -499,7 +550,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
             armed[i] = [hk]
         ops.profile_kernel(0)
         graphs = []
-        side = torch.cuda.Stream()
+        from hades_amd.sparse_optim import side_stream
+        side = side_stream(dev, 0)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for b in range(nb):
@@ -522,6 +574,9 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         # Timed region: exactly K steps.  One event record per step marks the step boundary
         # (3-4 us of GPU time each, inside the measured time); the kernel brackets are taken in
         # every `event_every`-th step only.
+        if pipelined:       # batch 0's forward half: the pipeline is full when the clock starts
+            prime(0)
+            torch.cuda.synchronize()
         t0 = time.perf_counter()
         step_ev[0].record()
         for j_i, i in enumerate(range(K)):
@@ -555,13 +610,15 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         opt.one_stream = True
         aev = [{k: new_events(2) for k in knames} for _ in range(3)]
         for j in range(3):
-            tim = {k: aev[j][k] for k in knames if k not in hook_of}
+            tim = {k: aev[j][k] for k in knames if k not in hook_of and k != "cold_refresh"}
             ops.profile_kernel(hook_of["seg_sum"], aev[j]["seg_sum"][0], aev[j]["seg_sum"][1])
-            step(j, timing=tim)
+            run_step(wl.ids[j % nb], wl.grads[j % nb], mode, None, tim)   # one batch at a time
         ops.profile_kernel(0)
         torch.cuda.synchronize()
         opt.one_stream = False
-        alone_ms = {k: sum(aev[j][k][0].elapsed_time(aev[j][k][1]) for j in range(3)) / 3 for k in knames}
+        pipe["i"] = None
+        alone_ms = {k: sum(aev[j][k][0].elapsed_time(aev[j][k][1]) for j in range(3)) / 3
+                    for k in knames if k != "cold_refresh"}
 
     # phases: a second, untimed pass with four event records per step on the main stream
     for i in range(K):
@@ -606,6 +663,10 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         if not kernel_ms[k]:
             continue
         ms = sum(kernel_ms[k]) / len(kernel_ms[k])
+        if k not in kbytes:     # no byte model: the time only
+            kernels[k] = {"kernel": name, "us": round(ms * 1e3, 2), "launches_timed": len(kernel_ms[k]),
+                          "bound": "latency"}
+            continue
         gbs = kbytes[k] / (ms * 1e-3) / 1e9
         entry = {"kernel": name, "us": round(ms * 1e3, 2), "launches_timed": len(kernel_ms[k]),
                  "bytes_per_launch": int(kbytes[k]), "GB/s": round(gbs, 1)}
@@ -657,7 +718,12 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
             roofline["hot_traffic_all_row_kernels"]["alone_note"] = (
                 "the same kernels in three untimed steps with both classes on one stream "
                 "(nothing on the host link beside them)")
-    if keyed:       # the sums are interleaved with the updates: one backward phase
+    if pipelined:   # the forward half runs on side streams: the main stream sees one phase
+        tot = sum(phase_ms.values())
+        phase_ms = {"backward of batch i + completion of batch i+1 (main stream)": tot}
+        phase_bytes = {next(iter(phase_ms)): sum(alg_bytes.values())}
+        phases = tuple(phase_ms)
+    elif keyed:     # the sums are interleaved with the updates: one backward phase
         phase_ms = {"fetch": phase_ms["fetch"], "combine+update": phase_ms["combine"] + phase_ms["update"]}
         phase_bytes = {"fetch": alg_bytes["fetch"], "combine+update": alg_bytes["combine"] + alg_bytes["update"]}
         phases = tuple(phase_ms)
@@ -683,7 +749,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
                           ("; fetch = the forward half (lookup, partition, both gathers, sort of the "
                            "keys beside the cold gather); combine is inside update = the backward "
                            "half (cold sums, cold update beside hot sums and hot update)"
-                           if keyed else ""),
+                           if keyed and not pipelined else ""),
            "step_alg_GB": round(total_bytes / 1e9, 4),
            "step_GB/s": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
            "step_frac_hbm": round(total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -1219,6 +1285,13 @@ def main():
                                          "main stream, cold rows on a second stream of the same "
                                          "priority; combine over class-ordered keys: the cold class "
                                          "is summed first and its update overlaps the hot class",
+                                "pipelined": "the keyed kernels with two batches in flight: the next "
+                                             "batch's lookup, partition, cold gather and key sort run on "
+                                             "side streams while this batch's cold update writes the host "
+                                             "table; afterwards the cold rows that update wrote are read "
+                                             "again, so every batch gets the rows and leaves the tables of "
+                                             "the one-batch-at-a-time order, bit for bit (the trainer must "
+                                             "know a batch's ids one step ahead)",
                                 "overlap": "one stream + the sort of the step's ids on a side stream, "
                                            "concurrent with its fetch",
                                 "graph": "one stream, every step replayed from a HIP graph captured "
@@ -1243,6 +1316,22 @@ def main():
                         "flight per table; opt-in: backward_keyed(fetched_rows=...))",
                 "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
                 "step_us": sec["step_us"], "phases": sec["phases"], "pcie": sec["pcie"],
+                "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
+                            for k, v in sec["kernels"].items()},
+                "parity_gate": sec["parity_gate"]}
+        if schedule == "keyed" and not args.reuse_rows:
+            log("secondary: cfg3 with two batches in flight (pipelined schedule, fetched rows reused)")
+            sec = run_gpu(args, "cfg3", "pipelined", with_gate=True, with_link=False, reuse_rows=True)
+            line["secondary"]["cfg3_pipelined"] = {
+                "what": "the headline workload with the next batch's forward half (lookup, partition, "
+                        "cold gather, key sort) running on side streams while this batch's cold update "
+                        "writes the host table, so that the link carries reads and writes at once; the "
+                        "cold rows that update wrote are read again afterwards, and every batch gets the "
+                        "rows and leaves the tables of the one-batch-at-a-time order, bit for bit.  Needs "
+                        "the ids of a batch one step ahead (prefetch_keyed / finish_prefetch) and, for the "
+                        "reuse of the fetched rows, one writer per table row",
+                "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
+                "step_us": sec["step_us"], "pcie": sec["pcie"],
                 "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
                             for k, v in sec["kernels"].items()},
                 "parity_gate": sec["parity_gate"]}

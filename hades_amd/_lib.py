@@ -54,6 +54,7 @@ _SIGNATURES = {
     "hades_split3_compact": [_P, c_int, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t, _P],
     "hades_lookup_split": [_P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, c_int, _P, c_size_t, _P],
     "hades_fetch_listed": [_P, _L, _P, _P, _P, _L, _P, _L, c_int, _P],
+    "hades_fetch_listed_in_set": [_P, _L, _P, _P, _P, _L, _P, _P, _L, _P, _L, c_int, _P],
     "hades_set_listed": [_P, _P, _L, _P, _P, _P, _L, _L, c_int, _P],
     "hades_adagrad_update_listed": [_P, _P, _P, _P, _L, _L, _P, _P, _L, c_float, c_float, _P],
     "hades_cached_fetch": [_P, _P, _P, _L, _P, _L, _P, _P, _P, _L, c_int, _P],

@@ -167,31 +167,68 @@ struct ListedArgs {
   const char* batch_ro;        // SCATTER source
   char* batch_rw;              // GATHER destination
   int64_t row_bytes;
+  // FILTER: only the positions whose table row is a member of this ascending set are moved
+  const int64_t* only_in;      // [only_in_max]
+  const int64_t* only_in_count;  // [1]
+  int64_t only_in_max;
 };
 
-template <typename Vec, bool GATHER>
+template <typename Vec, bool GATHER, bool FILTER>
 __global__ __launch_bounds__(kThreads) void row_move_listed_kernel(ListedArgs a, int chunks_per_row,
                                                                   int shift) {
+  static_assert(kRowsPerBlock <= kWave, "the filter compacts a block's rows inside one wave");
   __shared__ const char* s_src[kRowsPerBlock];
   __shared__ char* s_dst[kRowsPerBlock];
+  __shared__ int s_kept;
   int64_t cnt = a.count[0];
   cnt = cnt < a.max_count ? cnt : a.max_count;
+  int64_t set_n = 0;
+  if (FILTER) {
+    set_n = a.only_in_count[0];
+    set_n = set_n < a.only_in_max ? set_n : a.only_in_max;
+    if (set_n <= 0) return;
+  }
   for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock; row0 < cnt;
        row0 += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
     const int64_t left = cnt - row0;
-    const int rows_here = left < kRowsPerBlock ? static_cast<int>(left) : kRowsPerBlock;
-    for (int r = threadIdx.x; r < rows_here; r += kThreads) {
-      const int64_t p = a.list[row0 + r];
-      const int64_t t = a.index[p] * a.table_stride_bytes;
-      if (GATHER) {
-        s_src[r] = a.table_ro + t;
-        s_dst[r] = a.batch_rw + p * a.row_bytes;
-      } else {
-        s_src[r] = a.batch_ro + p * a.row_bytes;
-        s_dst[r] = a.table_rw + t;
+    int rows_here = left < kRowsPerBlock ? static_cast<int>(left) : kRowsPerBlock;
+    if (FILTER) {
+      // wave 0: one lane per row; the member rows are packed to the front of the row list
+      if (threadIdx.x < kWave) {
+        const int r = threadIdx.x;
+        int64_t p = 0, row = 0;
+        bool member = false;
+        if (r < rows_here) {
+          p = a.list[row0 + r];
+          row = a.index[p];
+          const int64_t pos = upper_bound_dev<int64_t>(a.only_in, set_n, row);
+          member = pos > 0 && a.only_in[pos - 1] == row;
+        }
+        const uint64_t mask = __ballot(member);
+        if (member) {
+          const int slot = __popcll(mask & ((uint64_t(1) << r) - 1));
+          const int64_t t = row * a.table_stride_bytes;
+          s_src[slot] = GATHER ? a.table_ro + t : a.batch_ro + p * a.row_bytes;
+          s_dst[slot] = GATHER ? a.batch_rw + p * a.row_bytes : a.table_rw + t;
+        }
+        if (r == 0) s_kept = __popcll(mask);
       }
+      __syncthreads();
+      rows_here = s_kept;
+    } else {
+      for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+        const int64_t p = a.list[row0 + r];
+        const int64_t t = a.index[p] * a.table_stride_bytes;
+        if (GATHER) {
+          s_src[r] = a.table_ro + t;
+          s_dst[r] = a.batch_rw + p * a.row_bytes;
+        } else {
+          s_src[r] = a.batch_ro + p * a.row_bytes;
+          s_dst[r] = a.table_rw + t;
+        }
+      }
+      __syncthreads();
     }
-    __syncthreads();
     const int total = rows_here * chunks_per_row;
     for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
       Vec v[kUnroll];
@@ -218,7 +255,7 @@ __global__ __launch_bounds__(kThreads) void row_move_listed_kernel(ListedArgs a,
 
 constexpr int64_t kMaxListedBlocks = 16384;
 
-template <bool GATHER>
+template <bool GATHER, bool FILTER = false>
 int launch_listed(const ListedArgs& a, int vec, hipStream_t stream) {
   const int64_t cpr64 = a.row_bytes / vec;
   HADES_REQUIRE(cpr64 * kRowsPerBlock < (int64_t(1) << 30), "row of %lld bytes is too large",
@@ -229,14 +266,19 @@ int launch_listed(const ListedArgs& a, int vec, hipStream_t stream) {
   if (blocks > kMaxListedBlocks) blocks = kMaxListedBlocks;
   // rows that cross the host link: a narrow grid that strides over the list
   const void* table = GATHER ? static_cast<const void*>(a.table_ro) : a.table_rw;
-  if (is_host_memory(table) && blocks > host_link_blocks(false)) blocks = host_link_blocks(false);
+  // (a filtered walk is mostly set look-ups in HBM and moves few rows: it keeps the wide grid)
+  if (!FILTER && is_host_memory(table) && blocks > host_link_blocks(false))
+    blocks = host_link_blocks(false);
   dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
   if (vec == 16) {
-    HADES_LAUNCH((row_move_listed_kernel<u32x4, GATHER>), grid, block, 0, stream, a, cpr, shift);
+    HADES_LAUNCH((row_move_listed_kernel<u32x4, GATHER, FILTER>), grid, block, 0, stream, a, cpr,
+                 shift);
   } else if (vec == 8) {
-    HADES_LAUNCH((row_move_listed_kernel<u32x2, GATHER>), grid, block, 0, stream, a, cpr, shift);
+    HADES_LAUNCH((row_move_listed_kernel<u32x2, GATHER, FILTER>), grid, block, 0, stream, a, cpr,
+                 shift);
   } else {
-    HADES_LAUNCH((row_move_listed_kernel<uint32_t, GATHER>), grid, block, 0, stream, a, cpr, shift);
+    HADES_LAUNCH((row_move_listed_kernel<uint32_t, GATHER, FILTER>), grid, block, 0, stream, a, cpr,
+                 shift);
   }
   return HADES_OK;
 }
@@ -424,8 +466,28 @@ int hades_fetch_listed(const void* src, int64_t src_stride, const int64_t* src_i
   int vec = pick_vec(row_bytes, {src, dst});
   while (vec > 4 && stride_bytes % vec != 0) vec >>= 1;
   ListedArgs a{(const char*)src, nullptr, stride_bytes, src_index, list, count, max_count,
-               nullptr, (char*)dst, row_bytes};
+               nullptr, (char*)dst, row_bytes, nullptr, nullptr, 0};
   return launch_listed<true>(a, vec, static_cast<hipStream_t>(stream));
+}
+
+int hades_fetch_listed_in_set(const void* src, int64_t src_stride, const int64_t* src_index,
+                              const int64_t* list, const int64_t* count, int64_t max_count,
+                              const int64_t* sorted_set, const int64_t* set_count, int64_t set_max,
+                              void* dst, int64_t dim, int dtype, void* stream) {
+  HADES_REQUIRE(max_count >= 0 && dim >= 1, "max_count must be >= 0 and dim >= 1");
+  HADES_REQUIRE(set_max >= 0, "set_max must be >= 0");
+  HADES_REQUIRE(elem_size(dtype) != 0, "Type can only be float or double (code %d)", dtype);
+  HADES_REQUIRE(src_stride == 0 || src_stride >= dim, "src_stride must be 0 or >= dim");
+  if (max_count == 0 || set_max == 0) return HADES_OK;
+  HADES_REQUIRE(src && src_index && list && count && sorted_set && set_count && dst,
+                "null pointer argument");
+  const int64_t row_bytes = dim * elem_size(dtype);
+  const int64_t stride_bytes = (src_stride ? src_stride : dim) * elem_size(dtype);
+  int vec = pick_vec(row_bytes, {src, dst});
+  while (vec > 4 && stride_bytes % vec != 0) vec >>= 1;
+  ListedArgs a{(const char*)src, nullptr, stride_bytes, src_index, list, count, max_count,
+               nullptr, (char*)dst, row_bytes, sorted_set, set_count, set_max};
+  return launch_listed<true, true>(a, vec, static_cast<hipStream_t>(stream));
 }
 
 int hades_set_listed(const void* src, void* dst, int64_t dst_stride, const int64_t* dst_index,
@@ -441,7 +503,7 @@ int hades_set_listed(const void* src, void* dst, int64_t dst_stride, const int64
   int vec = pick_vec(row_bytes, {src, dst});
   while (vec > 4 && stride_bytes % vec != 0) vec >>= 1;
   ListedArgs a{nullptr, (char*)dst, stride_bytes, dst_index, list, count, max_count,
-               (const char*)src, nullptr, row_bytes};
+               (const char*)src, nullptr, row_bytes, nullptr, nullptr, 0};
   return launch_listed<false>(a, vec, static_cast<hipStream_t>(stream));
 }
 

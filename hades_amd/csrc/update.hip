@@ -396,14 +396,20 @@ int check_rows(const int64_t* uids, const float* grad, int64_t max_rows, int64_t
   return HADES_OK;
 }
 
-// grid of a listed walk: one block per kRows rows, capped; rows that cross the host link get a
-// narrow grid that strides over the list
-dim3 listed_grid(int64_t max_count, std::initializer_list<const void*> tables) {
+// Grid of a listed walk.  Device tables: one block per kRows rows, capped.  Rows that cross the
+// host link: a narrow grid that strides over the list - 128 blocks when the kernel reads and
+// writes over the link, 32 when it only writes there (`host_reads` false: stores are posted, so
+// few waves saturate the link, and every further store in flight only queues up in front of the
+// HBM traffic of the kernels on other streams: the segmented sum beside a write-only update of
+// 128 blocks took 690 us, beside one of 32 blocks 155 us, and the update itself as long).
+dim3 listed_grid(int64_t max_count, bool host_writes, bool host_reads) {
   int64_t blocks = ceil_div(max_count, kRows);
   if (blocks > 16384) blocks = 16384;
-  bool host = false;
-  for (const void* t : tables) host = host || is_host_memory(t);
-  if (host && blocks > host_link_blocks(true)) blocks = host_link_blocks(true);
+  if (host_writes || host_reads) {
+    int64_t cap = host_link_blocks(true);
+    if (!host_reads && cap > 32 && getenv("HADES_HOST_LINK_BLOCKS_RW") == nullptr) cap = 32;
+    if (blocks > cap) blocks = cap;
+  }
   return dim3(static_cast<unsigned>(blocks));
 }
 
@@ -425,7 +431,9 @@ int check_listed(const ListedRows& r, bool class_form) {
 }
 
 int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
-  const dim3 grid = listed_grid(a.r.max_count, {a.w, a.s}), block(kThreads);
+  const bool w_host = is_host_memory(a.w), s_host = is_host_memory(a.s);
+  const dim3 grid = listed_grid(a.r.max_count, w_host || s_host,
+                                s_host || (w_host && a.r.w_rows == nullptr)), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (a.r.dim % 4 == 0 && a.r.stride % 4 == 0 && aligned16({a.r.grad, a.w, a.s, a.r.w_rows}))
     HADES_LAUNCH((adagrad_listed_kernel<4>), grid, block, 0, st, a);
@@ -439,7 +447,10 @@ int launch_adam_listed(const ListedRows& r, float* w, float* step, float* m, flo
   // 1 - beta is formed in double and rounded once, as in hades_adam_update
   const AdamListedArgs a{r, w, step, m, v, lr, static_cast<float>(beta1), static_cast<float>(beta2),
                          static_cast<float>(1.0 - beta1), static_cast<float>(1.0 - beta2), eps};
-  const dim3 grid = listed_grid(r.max_count, {w, step, m, v}), block(kThreads);
+  const bool w_host = is_host_memory(w);
+  const bool state_host = is_host_memory(step) || is_host_memory(m) || is_host_memory(v);
+  const dim3 grid = listed_grid(r.max_count, w_host || state_host,
+                                state_host || (w_host && r.w_rows == nullptr)), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (r.dim % 4 == 0 && r.stride % 4 == 0 && aligned16({r.grad, w, m, v, r.w_rows}))
     HADES_LAUNCH((adam_listed_kernel<4>), grid, block, 0, st, a);

@@ -207,15 +207,24 @@ def _stride_of(table, dim):
     return table.stride(0)
 
 
-def fetch_listed(table, index, pos_list, count, out):
+def fetch_listed(table, index, pos_list, count, out, only_in=None, only_in_count=None):
     """out[p] = table[index[p]] for the first count[0] positions p of pos_list (device-side count:
-    no host synchronisation).  `table` may be pinned host memory and may be a row-strided view."""
+    no host synchronisation).  `table` may be pinned host memory and may be a row-strided view.
+    With `only_in` (ascending int64 ids) and `only_in_count` (int64[1] on the device) only the
+    positions whose table row is among the first only_in_count[0] entries of only_in are fetched:
+    the refresh of rows that were gathered ahead of an update of exactly those rows."""
     _i64(index, "index"); _i64(pos_list, "pos_list"); _i64(count, "count")
     _dev_or_pinned(table, "table", contiguous=False); _dev(out, "out")
     dim = 1 if out.dim() == 1 else out.size(1)
     _check(table.dtype == out.dtype, "table and out differ in dtype")
-    _lib.call("hades_fetch_listed", _ptr(table), _stride_of(table, dim), _ptr(index), _ptr(pos_list),
-              _ptr(count), pos_list.numel(), _ptr(out), dim, _dcode(out), _stream())
+    if only_in is None:
+        _lib.call("hades_fetch_listed", _ptr(table), _stride_of(table, dim), _ptr(index), _ptr(pos_list),
+                  _ptr(count), pos_list.numel(), _ptr(out), dim, _dcode(out), _stream())
+        return out
+    _i64(only_in, "only_in"); _i64(only_in_count, "only_in_count")
+    _lib.call("hades_fetch_listed_in_set", _ptr(table), _stride_of(table, dim), _ptr(index),
+              _ptr(pos_list), _ptr(count), pos_list.numel(), _ptr(only_in), _ptr(only_in_count),
+              only_in.numel(), _ptr(out), dim, _dcode(out), _stream())
     return out
 
 

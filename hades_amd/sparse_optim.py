@@ -51,6 +51,21 @@ def unique_grads(idx, grad, cnt=None, id_bound=0, mode=ops.COMBINE_FAST):
     return uids[:u], sums
 
 
+_side_streams = {}
+
+
+def side_stream(device, k):
+    """The k-th (0, 1, 2) side stream of this module on `device`, created once per process and
+    shared by every optimizer: HIP serves a process's streams from a handful of hardware queues
+    (four by default), and streams that share a queue run one after the other, so a process
+    that wants its cold, prefetch and sort streams to overlap with its main stream must not
+    create a fresh set per optimizer."""
+    key = (torch.device(device).index or 0, int(k))
+    if key not in _side_streams:
+        _side_streams[key] = torch.cuda.Stream(device=device)
+    return _side_streams[key]
+
+
 class _SparseRowOptimizer:
     """State shared by the two optimizers: weights and state as (hot, cold) pairs keyed by the
     ascending hot-ID set.  `weight_cold` is [N, D] on the device or pinned on the host."""
@@ -115,7 +130,7 @@ class _SparseRowOptimizer:
                    torch.empty(1, dtype=torch.int64, device=self.device))
         if stream is None:
             if self._side is None:
-                self._side = torch.cuda.Stream(device=self.device)
+                self._side = side_stream(self.device, 2)
             stream = self._side
         # everything queued so far (the ids, and the previous step that used the workspace) first
         stream.wait_stream(cur)
@@ -138,7 +153,7 @@ class _SparseRowOptimizer:
 
     def _split_state(self):
         if getattr(self, "_cold_stream", None) is None:
-            self._cold_stream = torch.cuda.Stream(device=self.device)
+            self._cold_stream = side_stream(self.device, 0)
             self._split_bufs = {}
             self._split_ws = ops.Workspace(self.device)
             self._cold_done = None
@@ -228,7 +243,7 @@ class _SparseRowOptimizer:
             self.join()
 
     # ---- the keyed step: one lookup per query serves the gather, the combine and the update ----
-    def forward_keyed(self, ids, out=None, timing=None, bufs=None):
+    def forward_keyed(self, ids, out=None, timing=None, bufs=None, slot=None):
         """Forward half of a training step on the split schedule.  One lookup gives every query
         its slot, its class list and a class-ordered sort key; the hot rows are gathered on the
         current stream and the cold rows on the cold stream; meanwhile the keys are sorted (the
@@ -240,10 +255,10 @@ class _SparseRowOptimizer:
         if out is None:
             out = torch.empty((n, self.dim), dtype=self.hot_w.dtype, device=self.device)
         kb = ops.key_bits_for(max(self.num_rows, self.hot_ids.numel(), 2))
-        if bufs is None:
-            bufs = self._keyed_bufs(n)
+        if bufs is None:      # slot: see prefetch_keyed (the first batch of a pipelined run)
+            bufs = self._keyed_bufs(n, slot)
         loc, hot_pos, cold_pos, counts = ops.lookup_split(
-            ids, self.hot_set, workspace=self._split_ws, out=bufs["split"],
+            ids, self.hot_set, workspace=bufs.get("split_ws", self._split_ws), out=bufs["split"],
             sort_keys=bufs["keys"], key_bits=kb)
         hot_pos, cold_pos = hot_pos[:n], cold_pos[:n]
         split_done = torch.cuda.Event()
@@ -257,14 +272,18 @@ class _SparseRowOptimizer:
         if self.hot_ids.numel():
             self._timed(timing, "hot_fetch", cur,
                         lambda: ops.fetch_listed(self.hot_w, loc, hot_pos, counts[0:1], out))
-        plan = ops.combine_plan_classed(bufs["keys"][:n], self.dim, kb, workspace=self._ws,
+        plan = ops.combine_plan_classed(bufs["keys"][:n], self.dim, kb, workspace=bufs.get("ws", self._ws),
                                         out=(bufs["ukeys"][:n], bufs["nu"], bufs["class_split"]),
                                         first_pos=bufs["first_pos"][:n])
         self.join()
         return out, (plan, bufs)
 
-    def _keyed_bufs(self, n):
-        b = getattr(self, "_kbufs", None)
+    def _keyed_bufs(self, n, slot=None):
+        """Buffers of one keyed step.  slot = None: the optimizer's single set, with the shared
+        workspaces (one batch in flight).  slot = 0 / 1: one of two sets that also own their
+        workspaces, for the pipelined schedule where two batches are in flight."""
+        sets = self.__dict__.setdefault("_kbufs", {})
+        b = sets.get(slot)
         if b is None or b["keys"].numel() < n:
             dev = self.device
             i64 = lambda k: torch.empty(k, dtype=torch.int64, device=dev)
@@ -272,10 +291,83 @@ class _SparseRowOptimizer:
                  "nu": i64(1), "class_split": i64(2),
                  "first_pos": torch.empty(n, dtype=torch.int32, device=dev),
                  "sums": torch.empty((n, self.dim), dtype=torch.float32, device=dev), "cnts": i64(n)}
-            self._kbufs = b
+            if slot is not None:
+                b["ws"], b["split_ws"] = ops.Workspace(dev), ops.Workspace(dev)
+            sets[slot] = b
         return b
 
-    def backward_keyed(self, state, grad, mode=ops.COMBINE_FAST, timing=None, fetched_rows=None):
+    # ---- the pipelined keyed step: the next batch's cold rows cross the host link while the
+    # ---- current batch's cold update writes the table ------------------------------------------
+    # The link carries reads and writes at the same time, and a keyed step uses one direction at a
+    # time for most of its length (gather: reads; update with fetched_rows: writes).  A trainer
+    # that has the ids of batch i+1 before the backward half of batch i (the reference's sampler
+    # runs ahead of the step) calls
+    #     p = opt.prefetch_keyed(ids_next, slot=(i + 1) % 2, out=rows_next)
+    #     opt.backward_keyed(state_i, grads_i, fetched_rows=rows_i, join=False)
+    #     rows_next, state_next = opt.finish_prefetch(p, after=state_i)
+    # and gets, bit for bit, the rows and tables of the one-batch-at-a-time order: the rows that
+    # batch i's update wrote (its distinct cold ids; usually a handful of the next batch's) are
+    # read again after that update, the hot rows are gathered after the hot update as before.
+    def prefetch_keyed(self, ids, slot, out=None, timing=None):
+        """Starts the forward half of the NEXT batch on side streams: lookup + partition + cold
+        gather on one, the sort of the class-ordered keys on another.  Nothing of it is visible to
+        the caller's stream until finish_prefetch.  `slot` (0 or 1) alternates from batch to
+        batch; `out` must not be the rows buffer of the batch whose backward half is pending."""
+        self._split_state()
+        if getattr(self, "_pre_stream", None) is None:
+            self._pre_stream = side_stream(self.device, 1)
+            self._sort_stream = side_stream(self.device, 2)
+        cur, pre, srt = torch.cuda.current_stream(), self._pre_stream, self._sort_stream
+        n = ids.numel()
+        if out is None:
+            out = torch.empty((n, self.dim), dtype=self.hot_w.dtype, device=self.device)
+        kb = ops.key_bits_for(max(self.num_rows, self.hot_ids.numel(), 2))
+        bufs = self._keyed_bufs(n, slot)
+        pre.wait_stream(cur)      # the ids, and everything that last used this slot's buffers
+        with torch.cuda.stream(pre):
+            loc, hot_pos, cold_pos, counts = ops.lookup_split(
+                ids, self.hot_set, workspace=bufs["split_ws"], out=bufs["split"],
+                sort_keys=bufs["keys"], key_bits=kb)
+            looked_up = torch.cuda.Event()
+            looked_up.record(pre)
+            self._timed(timing, "cold_fetch", pre,
+                        lambda: ops.fetch_listed(self.cold_w, ids, cold_pos[:n], counts[1:2], out))
+            gathered = torch.cuda.Event()
+            gathered.record(pre)
+        srt.wait_event(looked_up)
+        with torch.cuda.stream(srt):
+            plan = ops.combine_plan_classed(bufs["keys"][:n], self.dim, kb, workspace=bufs["ws"],
+                                            out=(bufs["ukeys"][:n], bufs["nu"], bufs["class_split"]),
+                                            first_pos=bufs["first_pos"][:n])
+            planned = torch.cuda.Event()
+            planned.record(srt)
+        return {"ids": ids, "out": out, "plan": plan, "bufs": bufs, "loc": loc, "hot_pos": hot_pos[:n],
+                "cold_pos": cold_pos[:n], "counts": counts, "looked_up": looked_up,
+                "gathered": gathered, "planned": planned}
+
+    def finish_prefetch(self, p, after=None, timing=None):
+        """Completes a prefetched forward half on the current stream, after the backward half of
+        the batch before it (`after` = that batch's state, or None if there was none) has been
+        queued: gathers the hot rows (behind the hot update), waits for the cold update, re-reads
+        the cold rows that update wrote, and returns (rows, state) like forward_keyed."""
+        cur = torch.cuda.current_stream()
+        ids, out, counts = p["ids"], p["out"], p["counts"]
+        cur.wait_event(p["looked_up"])
+        if self.hot_ids.numel():
+            self._timed(timing, "hot_fetch", cur,
+                        lambda: ops.fetch_listed(self.hot_w, p["loc"], p["hot_pos"], counts[0:1], out))
+        self.join()                         # the cold update of the batch before
+        cur.wait_event(p["gathered"])
+        if after is not None:
+            prev = after[0]
+            self._timed(timing, "cold_refresh", cur,
+                        lambda: ops.fetch_listed(self.cold_w, ids, p["cold_pos"], counts[1:2], out,
+                                                 only_in=prev.uids, only_in_count=prev.class_split[1:2]))
+        cur.wait_event(p["planned"])
+        return out, (p["plan"], p["bufs"])
+
+    def backward_keyed(self, state, grad, mode=ops.COMBINE_FAST, timing=None, fetched_rows=None,
+                       join=True):
         """Backward half: segmented sums of the cold class, whose update then starts on the cold
         stream while the hot class is summed and updated on the current stream; joins at the end.
         Returns (ukeys, sums, cnts, num_unique, class_split): the distinct rows in class order -
@@ -304,7 +396,8 @@ class _SparseRowOptimizer:
                     lambda: ops.combine_apply_class(plan, grad, 1, mode, out=out))
         if self.hot_ids.numel():
             self._timed(timing, "hot_update", cur, lambda: self._update_keyed(plan, out[0], 1))
-        self.join()
+        if join:        # join=False: finish_prefetch (or join()) waits for the cold update later
+            self.join()
         return plan.uids, out[0], out[1], plan.num_unique, plan.class_split
 
     def _update_keyed(self, plan, sums, which, fetched_rows=None):

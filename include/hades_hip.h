@@ -256,6 +256,19 @@ int hades_set_listed(const void* src, void* dst, int64_t dst_stride, const int64
                      const int64_t* list, const int64_t* count, int64_t max_count, int64_t dim,
                      int dtype, void* stream);
 
+/* hades_fetch_listed restricted to the positions whose table row src_index[p] is a member of the
+ * ascending set sorted_set[0 .. min(set_count[0], set_max)); the other positions of dst are left as
+ * they are.  It refreshes rows that were gathered ahead of an update: a trainer that knows the ids
+ * of its next batch (the reference's data loader hands them out ahead of the step,
+ * python/EmbCache/dist_emb.py:276-288 keeps them in its trace) gathers that batch's cold rows
+ * while the current batch's update is still writing the table, and afterwards re-reads exactly
+ * the rows that update wrote - sorted_set = the update's distinct cold ids - so that the batch
+ * sees what a gather after the update would have seen. */
+int hades_fetch_listed_in_set(const void* src, int64_t src_stride, const int64_t* src_index,
+                              const int64_t* list, const int64_t* count, int64_t max_count,
+                              const int64_t* sorted_set, const int64_t* set_count, int64_t set_max,
+                              void* dst, int64_t dim, int dtype, void* stream);
+
 /* combine: sort + dedup + segment-sum of duplicate-ID gradient rows; the arithmetic of
  * only_unique_grads (python/EmbCache/sparse_optim.py:132-139), which is also the
  * local-aggregation reduction (:310) over concatenated trainer batches.

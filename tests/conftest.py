@@ -102,3 +102,21 @@ def cuda_device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def _release_cached_memory(request):
+    """After every GPU test: hand torch's cached page-locked host blocks and device blocks back.
+    The host allocator never releases by itself, and the sum of page-locked memory that one
+    process may hold is limited on the GPU boxes (a later pin_memory allocation is then refused)."""
+    yield
+    if request.node.get_closest_marker("gpu") is None:
+        return
+    import gc
+    import torch
+    if torch.cuda.is_available():
+        gc.collect()
+        torch.cuda.synchronize()
+        if hasattr(torch._C, "_host_emptyCache"):
+            torch._C._host_emptyCache()
+        torch.cuda.empty_cache()

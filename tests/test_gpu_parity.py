@@ -1655,3 +1655,117 @@ def test_sparse_adam_keyed_with_the_forward_rows(lib):
     assert np.allclose(diff[touched], 0.25, atol=1e-6)
     mask = np.ones(N, bool); mask[touched] = False
     assert np.array_equal(diff[mask], np.zeros_like(diff[mask]))
+
+
+@pytest.mark.parametrize("host", [False, True])
+def test_fetch_listed_restricted_to_a_set(lib, host):
+    """hades_fetch_listed_in_set: only positions whose table row is in the ascending set are
+    fetched; every other row of the output keeps its value; set count and list count are read
+    on the device; an empty set moves nothing."""
+    _, ops = lib
+    rng = np.random.default_rng(31)
+    N, D, n = 5000, 96, 4000
+    table = rng.standard_normal((N, D)).astype(np.float32)
+    t = torch.from_numpy(table)
+    t = t.pin_memory() if host else t.cuda()
+    idx = rng.integers(0, N, n).astype(np.int64)
+    pos = rng.permutation(n)[: n - 300].astype(np.int64)
+    members = np.sort(rng.choice(N, 700, replace=False)).astype(np.int64)
+    padded = np.concatenate([members, np.arange(N, N + 50)])       # entries past the count: ignored
+    for live, set_live in ((pos.size, members.size), (pos.size - 11, 123), (pos.size, 0), (0, members.size)):
+        out = torch.full((n, D), -7.0, dtype=torch.float32, device="cuda")
+        ops.fetch_listed(t, dev(idx), dev(pos), torch.tensor([live], device="cuda"), out,
+                         only_in=dev(padded), only_in_count=torch.tensor([set_live], device="cuda"))
+        want = np.full((n, D), -7.0, np.float32)
+        p = pos[:live]
+        keep = p[np.isin(idx[p], members[:set_live])]
+        want[keep] = table[idx[keep]]
+        assert np.array_equal(out.cpu().numpy(), want)
+        assert live == 0 or set_live == 0 or keep.size > 0
+
+
+@pytest.mark.parametrize("N,D,H,n,hot_frac", [
+    (3000, 64, 300, 5000, 0.5),             # small cold table: most cold rows of a batch were just updated
+    (200_000, 128, 20_000, 60_000, 0.8),    # a few refreshed rows among many
+    (5000, 32, 0, 4000, 0.0),               # no hot set
+    (5000, 32, 500, 4000, 1.0),             # no cold rows
+])
+@pytest.mark.parametrize("host_cold", [False, True])
+@pytest.mark.parametrize("kind", ["adagrad", "adam"])
+def test_pipelined_keyed_steps_equal_one_batch_at_a_time(lib, N, D, H, n, hot_frac, host_cold, kind):
+    """prefetch_keyed / backward_keyed(join=False) / finish_prefetch over six different batches:
+    the rows every batch receives and all tables at the end equal, bit for bit, those of the same
+    optimizer run one batch at a time (forward_keyed, backward_keyed) - which the tests above pin
+    to the oracle - and, for Adagrad, the oracle's own sequence of keyed steps.  Both with the
+    cold update reading the table and with it taking the old rows from the fetched ones."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad, SparseAdam
+    rng = np.random.default_rng(N + n + 17)
+    cold, hot_ids, q0 = _split_case(rng, N, D, H, n, hot_frac)
+    steps = 6
+    is_hot_row = np.zeros(N, bool)
+    is_hot_row[hot_ids] = True
+    cold_ids = np.flatnonzero(~is_hot_row).astype(np.int64)
+
+    def draw():
+        m = rng.random(n) < hot_frac
+        if H == 0:
+            m[:] = False
+        if cold_ids.size == 0:
+            m[:] = True
+        hq = hot_ids[rng.integers(0, max(H, 1), n)] if H else np.zeros(n, np.int64)
+        cq = cold_ids[rng.integers(0, max(cold_ids.size, 1), n)] if cold_ids.size else np.zeros(n, np.int64)
+        return np.where(m, hq, cq).astype(np.int64)
+
+    qs = [q0] + [draw() for _ in range(steps - 1)]
+    grads = [(rng.standard_normal((n, D)) * 1e-2).astype(np.float32) for _ in range(steps)]
+    kb = ops.key_bits_for(max(N, H, 2))
+
+    def make():
+        t = torch.from_numpy(cold.copy())
+        t = t.pin_memory() if host_cold else t.cuda()
+        if kind == "adam":
+            return SparseAdam(t, torch.from_numpy(hot_ids))
+        return SparseAdagrad(t, torch.from_numpy(hot_ids), lr=0.01, eps=1e-10)
+
+    def tables(o):
+        names = ("w", "step", "m", "v") if kind == "adam" else ("w", "s")
+        return [getattr(o, pre + nm).cpu() for pre in ("cold_", "hot_") for nm in names]
+
+    t_q = [dev(x) for x in qs]
+    t_g = [dev(x) for x in grads]
+    for reuse in (False, True):
+        seq, pipe = make(), make()
+        seq_rows = []
+        for k in range(steps):
+            rows, st = seq.forward_keyed(t_q[k])
+            seq_rows.append(rows.clone())
+            seq.backward_keyed(st, t_g[k], mode=ops.COMBINE_EXACT, fetched_rows=rows if reuse else None)
+        bufs = [torch.empty((n, D), dtype=torch.float32, device="cuda") for _ in range(2)]
+        rows, st = pipe.forward_keyed(t_q[0], out=bufs[0], slot=0)
+        refreshed = 0
+        for k in range(steps):
+            assert torch.equal(rows, seq_rows[k]), (reuse, k)
+            nxt = None
+            if k + 1 < steps:
+                nxt = pipe.prefetch_keyed(t_q[k + 1], slot=(k + 1) % 2, out=bufs[(k + 1) % 2])
+            pipe.backward_keyed(st, t_g[k], mode=ops.COMBINE_EXACT, fetched_rows=rows if reuse else None,
+                                join=nxt is None)
+            if nxt is not None:
+                prev_cold = np.unique(qs[k][~np.isin(qs[k], hot_ids)])
+                refreshed += int(np.isin(qs[k + 1], prev_cold).sum())
+                rows, st = pipe.finish_prefetch(nxt, after=st)
+        torch.cuda.synchronize()
+        for a, b in zip(tables(seq), tables(pipe)):
+            assert torch.equal(a, b), reuse
+        if hot_frac < 1.0:
+            assert refreshed > 0            # the case does exercise the refresh
+        if kind == "adagrad" and not reuse:
+            cw, cs = cold.copy(), np.zeros_like(cold)
+            hw, hs = cold[hot_ids].copy(), np.zeros((H, D), np.float32)
+            for k in range(steps):
+                assert np.array_equal(seq_rows[k].cpu().numpy(), O.cached_fetch(cw, hw, qs[k], hot_ids))
+                O.keyed_step(cw, cs, hw, hs, hot_ids, qs[k], grads[k], 0.01, 1e-10, kb)
+            got = tables(pipe)
+            assert np.array_equal(got[0].numpy(), cw) and np.array_equal(got[1].numpy(), cs)
+            assert np.array_equal(got[2].numpy(), hw) and np.array_equal(got[3].numpy(), hs)
