@@ -70,7 +70,10 @@ inline uintptr_t align_of_ptr(const void* p) { return reinterpret_cast<uintptr_t
 // true if `p` is host memory that kernels reach over the host link (hipHostMalloc / registered)
 bool is_host_memory(const void* p);
 // blocks to launch for a kernel whose table rows cross the host link (see core.hip)
-int64_t host_link_blocks(bool read_and_write);
+// what a kernel does over the host link: copies rows one way, updates rows in place (reads and
+// writes at once), or only writes them (the old rows come from device memory)
+enum HostLinkUse { kLinkCopy = 0, kLinkReadWrite = 1, kLinkWriteOnly = 2 };
+int64_t host_link_blocks(HostLinkUse use);
 
 // Carve aligned sub-buffers out of a caller-provided workspace.
 struct Carver {

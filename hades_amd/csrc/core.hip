@@ -35,14 +35,22 @@ bool is_host_memory(const void* p) {
 // it parks hundreds of thousands of slow requests in the memory pipeline, and every HBM kernel
 // that runs beside it on another stream slows down to the link's pace.
 // Measured on 76 K rows of 512 bytes: a gather reaches the link's read rate (55 GB/s) from 32 to
-// 128 blocks; an update, which has reads and writes in flight, peaks at 128 (42.6 GB/s each way).
-int64_t host_link_blocks(bool read_and_write) {
-  const char* e = getenv(read_and_write ? "HADES_HOST_LINK_BLOCKS_RW" : "HADES_HOST_LINK_BLOCKS");
-  if (e != nullptr) {                                  // tuning override
+// 128 blocks, 53 GB/s with 16; an update that has reads and writes in flight peaks at 128
+// (42.6 GB/s each way); an update that only writes (stores are posted: its waves never wait for
+// the link) saturates it from 32 blocks, and every further store in flight only queues up in front
+// of the HBM traffic of other streams (the segmented sum beside a write-only update of 128 blocks
+// took 690 us, beside one of 32 blocks 155 us, the update itself as long either way).
+// HADES_HOST_LINK_BLOCKS / _RW / _WO override the three widths for tuning.
+int64_t host_link_blocks(HostLinkUse use) {
+  static const char* const names[] = {"HADES_HOST_LINK_BLOCKS", "HADES_HOST_LINK_BLOCKS_RW",
+                                      "HADES_HOST_LINK_BLOCKS_WO"};
+  static const int64_t defaults[] = {16, 128, 32};
+  const char* e = getenv(names[use]);
+  if (e != nullptr) {
     const long v = atol(e);
     if (v >= 1) return v;
   }
-  return read_and_write ? 128 : 16;
+  return defaults[use];
 }
 
 }  // namespace hades

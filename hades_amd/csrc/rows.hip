@@ -267,8 +267,8 @@ int launch_listed(const ListedArgs& a, int vec, hipStream_t stream) {
   // rows that cross the host link: a narrow grid that strides over the list
   const void* table = GATHER ? static_cast<const void*>(a.table_ro) : a.table_rw;
   // (a filtered walk is mostly set look-ups in HBM and moves few rows: it keeps the wide grid)
-  if (!FILTER && is_host_memory(table) && blocks > host_link_blocks(false))
-    blocks = host_link_blocks(false);
+  if (!FILTER && is_host_memory(table) && blocks > host_link_blocks(kLinkCopy))
+    blocks = host_link_blocks(kLinkCopy);
   dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
   if (vec == 16) {
     HADES_LAUNCH((row_move_listed_kernel<u32x4, GATHER, FILTER>), grid, block, 0, stream, a, cpr,

@@ -397,17 +397,13 @@ int check_rows(const int64_t* uids, const float* grad, int64_t max_rows, int64_t
 }
 
 // Grid of a listed walk.  Device tables: one block per kRows rows, capped.  Rows that cross the
-// host link: a narrow grid that strides over the list - 128 blocks when the kernel reads and
-// writes over the link, 32 when it only writes there (`host_reads` false: stores are posted, so
-// few waves saturate the link, and every further store in flight only queues up in front of the
-// HBM traffic of the kernels on other streams: the segmented sum beside a write-only update of
-// 128 blocks took 690 us, beside one of 32 blocks 155 us, and the update itself as long).
+// host link: a narrow grid that strides over the list (host_link_blocks: wider when the kernel
+// reads and writes over the link than when it only writes there).
 dim3 listed_grid(int64_t max_count, bool host_writes, bool host_reads) {
   int64_t blocks = ceil_div(max_count, kRows);
   if (blocks > 16384) blocks = 16384;
   if (host_writes || host_reads) {
-    int64_t cap = host_link_blocks(true);
-    if (!host_reads && cap > 32 && getenv("HADES_HOST_LINK_BLOCKS_RW") == nullptr) cap = 32;
+    const int64_t cap = host_link_blocks(host_reads ? kLinkReadWrite : kLinkWriteOnly);
     if (blocks > cap) blocks = cap;
   }
   return dim3(static_cast<unsigned>(blocks));

@@ -85,6 +85,7 @@ class _SparseRowOptimizer:
         self.hot_w = self._gather_hot(weight_cold)
         self._ws = ops.Workspace(self.device)
         self._side = None
+        self._kbufs = {}            # buffer sets of the keyed steps, by slot
 
     def _gather_hot(self, cold):
         """Hot copy of the rows named by hot_ids; a pinned host table is read zero-copy by the
@@ -282,7 +283,7 @@ class _SparseRowOptimizer:
         """Buffers of one keyed step.  slot = None: the optimizer's single set, with the shared
         workspaces (one batch in flight).  slot = 0 / 1: one of two sets that also own their
         workspaces, for the pipelined schedule where two batches are in flight."""
-        sets = self.__dict__.setdefault("_kbufs", {})
+        sets = self._kbufs
         b = sets.get(slot)
         if b is None or b["keys"].numel() < n:
             dev = self.device
