@@ -907,6 +907,15 @@ def run_cfg4(args):
     assert int(acc.status.item()) == 0, "accumulator overflow"
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     K = args.steps
+    # the accumulate kernel undisturbed: every - 1 further steps (none of them flushes) with no
+    # write-back in flight
+    aev = [new_events(2) for _ in range(every - 1)]
+    for j in range(every - 1):
+        ops.profile_kernel(ops.KERNEL_HASH_ACCUMULATE, aev[j][0], aev[j][1])
+        step(j)
+    ops.profile_kernel(0)
+    torch.cuda.synchronize()
+    alone_ms = sum(a.elapsed_time(b) for a, b in aev) / max(1, len(aev))
     flush_steps = [i for i in range(K) if (i + 1) % every == 0]
     comb_ms = sum(ev[i][0].elapsed_time(ev[i][1]) for i in range(K)) / K
     acc_ms = sum(ev[i][1].elapsed_time(ev[i][2]) for i in range(K)) / K
@@ -931,10 +940,18 @@ def run_cfg4(args):
     # 8 B count and 4D accumulator read-modify-write (2 x 4D)
     kbytes = U * (16 + 4 * D + 8 + 16 + 8 * D)
     achieved = kbytes / (kern_ms * 1e-3) / 1e9
+    alone = kbytes / (alone_ms * 1e-3) / 1e9
     line["roofline"] = {"bound": "hbm", "kernel": "hash_accumulate_kernel (hades_hash_accumulate)",
                         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                        "kernel_us": round(kern_ms * 1e3, 2), "bytes_per_launch": int(kbytes)}
+                        "kernel_us": round(kern_ms * 1e3, 2), "bytes_per_launch": int(kbytes),
+                        "kernel_us_alone": round(alone_ms * 1e3, 2), "GB/s_alone": round(alone, 1),
+                        "frac_alone": round(alone / HBM_PEAK_GBS, 4),
+                        "note": "kernel_us: the launches of the timed steps, which run beside the "
+                                "write-back of the previous flush when that is on the side stream "
+                                "(HBM kernels slow down while requests to host memory are in flight); "
+                                "alone: %d further steps after the timed region with nothing on the "
+                                "host link" % (every - 1)}
     if flush_steps:
         fl_ms = sum(ev[i][2].elapsed_time(ev[i][3]) for i in flush_steps) / len(flush_steps)
         if overlapped:
