@@ -1020,6 +1020,7 @@ def run_cfg4_staleness(args):
                 torch.empty(n, dtype=torch.int64, device=dev),
                 torch.empty(1, dtype=torch.int64, device=dev))
     fetched = torch.empty((n, D), dtype=torch.float32, device=dev)
+    m_cnt = torch.zeros(1, dtype=torch.int64, device=dev)
     log("workload ready")
     stats = {"miss": 0, "hit": 0, "flushed": 0}
 
@@ -1031,12 +1032,12 @@ def run_cfg4_staleness(args):
         locs = cache.accumulate_gradients_cold_remote(uids, sums)          # cached ids: delayed
         _, hit_pos, miss_pos = ops.split(locs)
         if miss_pos.numel():
-            m_ids = uids[miss_pos]
-            m_sums = sums[miss_pos]
-            ops.adagrad_update_(m_ids, m_sums, None, None, cold_w, cold_s, None, 0.01, 1e-10)
-            rows = fetched[:m_ids.numel()]
-            E.cudaFetch2(cold_w, m_ids, rows)                              # the rows a trainer pulled
-            cache.update_cache(m_ids, rows)
+            # the update hands back the new rows (w_out), which are the rows a trainer would pull
+            # next: no third crossing of the link to fetch them for the cache
+            m_cnt.fill_(miss_pos.numel())
+            ops.adagrad_update_listed_(uids, sums, miss_pos, m_cnt, cold_w, cold_s, 0.01, 1e-10,
+                                       w_out=fetched[:u])
+            cache.update_cache(uids[miss_pos], fetched[:u][miss_pos])
         f_ids, f_grads, f_cnts, f_num = cache.staled_gradients_remote_padded(slots)
         ops.adagrad_update_(f_ids, f_grads, None, None, cold_w, cold_s, None, 0.01, 1e-10,
                             num_unique=f_num)
@@ -1058,9 +1059,9 @@ def run_cfg4_staleness(args):
         step(warm + args.steps + i, count=True)
     K = args.steps
     miss, hit, flushed = (stats[k] / K for k in ("miss", "hit", "flushed"))
-    # rows over the host link: uncached ids are read, written and fetched once more for the cache;
-    # flushed rows are read and written
-    host_rows = miss * 3 + flushed * 2
+    # rows over the host link: uncached ids are read and written (the update also returns the new
+    # rows for the cache); flushed rows are read and written
+    host_rows = miss * 2 + flushed * 2
     line = {
         "metric": "cold gradient rows/s (combine + cold-data cache with the staleness rule + write-back)",
         "value": round(n / (ms_per_step * 1e-3), 1), "unit": "rows/s", "n_gpus": 1, "steps": K,

@@ -56,7 +56,7 @@ _SIGNATURES = {
     "hades_fetch_listed": [_P, _L, _P, _P, _P, _L, _P, _L, c_int, _P],
     "hades_fetch_listed_in_set": [_P, _L, _P, _P, _P, _L, _P, _P, _L, _P, _L, c_int, _P],
     "hades_set_listed": [_P, _P, _L, _P, _P, _P, _L, _L, c_int, _P],
-    "hades_adagrad_update_listed": [_P, _P, _P, _P, _L, _L, _P, _P, _L, c_float, c_float, _P],
+    "hades_adagrad_update_listed": [_P, _P, _P, _P, _L, _L, _P, _P, _L, _P, c_float, c_float, _P],
     "hades_cached_fetch": [_P, _P, _P, _L, _P, _L, _P, _P, _P, _L, c_int, _P],
     "hades_cached_fetch_loc": [_P, _P, _P, _P, _L, _P, _L, c_int, _P],
     "hades_cached_set": [_P, _P, _P, _P, _L, _P, _L, _P, _L, c_int, _P],

@@ -153,6 +153,7 @@ struct AdagradListedArgs {
   ListedRows r;
   float* w;
   float* s;
+  float* w_out;             // optional: the new weight row of position p also goes to row p of w_out
   float lr, eps;
 };
 
@@ -238,6 +239,11 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
           const V w1 = w[k] - vdiv(a.lr * g[k], std_);
           *sp[k] = s1;
           *wp[k] = w1;
+          if (a.w_out != nullptr) {
+            const int r = c / cpr;
+            const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
+            *reinterpret_cast<V*>(a.w_out + s_grad[r] + col) = w1;
+          }
         }
       }
     }
@@ -431,7 +437,7 @@ int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
   const dim3 grid = listed_grid(a.r.max_count, w_host || s_host,
                                 s_host || (w_host && a.r.w_rows == nullptr)), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (a.r.dim % 4 == 0 && a.r.stride % 4 == 0 && aligned16({a.r.grad, a.w, a.s, a.r.w_rows}))
+  if (a.r.dim % 4 == 0 && a.r.stride % 4 == 0 && aligned16({a.r.grad, a.w, a.s, a.r.w_rows, a.w_out}))
     HADES_LAUNCH((adagrad_listed_kernel<4>), grid, block, 0, st, a);
   else
     HADES_LAUNCH((adagrad_listed_kernel<1>), grid, block, 0, st, a);
@@ -485,14 +491,15 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
 
 int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,
                                 const int64_t* count, int64_t max_count, int64_t dim, float* w,
-                                float* s, int64_t stride, float lr, float eps, void* stream) {
+                                float* s, int64_t stride, float* w_out, float lr, float eps,
+                                void* stream) {
   HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
   const ListedRows r{row_index, grad, list, count, max_count, nullptr, nullptr, 0, int64_t(-1),
                      nullptr, nullptr, dim, stride == 0 ? dim : stride};
   const int rc = check_listed(r, false);
   if (rc != HADES_OK || max_count == 0) return rc;
   HADES_REQUIRE(w && s, "null pointer argument");
-  return launch_adagrad_listed(AdagradListedArgs{r, w, s, lr, eps}, stream);
+  return launch_adagrad_listed(AdagradListedArgs{r, w, s, w_out, lr, eps}, stream);
 }
 
 int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
@@ -506,7 +513,7 @@ int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const in
   const int rc = check_listed(r, true);
   if (rc != HADES_OK || max_rows == 0) return rc;
   HADES_REQUIRE(w && s, "null pointer argument");
-  return launch_adagrad_listed(AdagradListedArgs{r, w, s, lr, eps}, stream);
+  return launch_adagrad_listed(AdagradListedArgs{r, w, s, nullptr, lr, eps}, stream);
 }
 
 int hades_adam_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,

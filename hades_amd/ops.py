@@ -238,11 +238,12 @@ def set_listed(src, table, index, pos_list, count):
               _ptr(pos_list), _ptr(count), pos_list.numel(), dim, _dcode(src), _stream())
 
 
-def adagrad_update_listed_(row_index, grad, pos_list, count, w, s, lr, eps):
+def adagrad_update_listed_(row_index, grad, pos_list, count, w, s, lr, eps, w_out=None):
     """Sparse Adagrad over the rows named by the first count[0] positions p of pos_list:
     g = grad[p]; r = row_index[p]; s[r] += g*g; w[r] -= lr * g / (sqrt(s[r]) + eps).  w and s are
     one table pair (device or pinned host) with the same row stride; they may be the two halves of
-    one interleaved table."""
+    one interleaved table.  `w_out` (float32 [positions, D] on the device) also receives the new
+    weight row of every position."""
     _i64(row_index, "row_index"); _i64(pos_list, "pos_list"); _i64(count, "count"); _dev(grad, "grad")
     _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
     dim = grad.size(1)
@@ -251,8 +252,13 @@ def adagrad_update_listed_(row_index, grad, pos_list, count, w, s, lr, eps):
         _check(t.dtype == torch.float32 and t.dim() == 2 and t.size(1) == dim, "%s: wrong dtype/width" % name)
     stride = _stride_of(w, dim)
     _check(_stride_of(s, dim) == stride, "w and s must have the same row stride")
+    if w_out is not None:
+        _dev(w_out, "w_out")
+        _check(w_out.dtype == torch.float32 and tuple(w_out.shape) == tuple(grad.shape),
+               "w_out must be float32 of grad's shape")
     _lib.call("hades_adagrad_update_listed", _ptr(row_index), _ptr(grad), _ptr(pos_list), _ptr(count),
-              pos_list.numel(), dim, _ptr(w), _ptr(s), stride, float(lr), float(eps), _stream())
+              pos_list.numel(), dim, _ptr(w), _ptr(s), stride, _opt(w_out), float(lr), float(eps),
+              _stream())
 
 
 def _adam_tables(tables, dim):

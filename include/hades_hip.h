@@ -365,10 +365,15 @@ int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* 
  * batch, list/count one of the two lists hades_lookup_split made of its distinct ids.  w and s may
  * be device or pinned host memory; rows lie `stride` floats apart (0 = dim), so the weight and
  * state row of an id may be stored next to each other (s = w + dim, stride = 2*dim): one burst
- * over the host link per cold row and direction instead of two. */
+ * over the host link per cold row and direction instead of two.
+ * w_out (optional, float[positions, dim], device): the new weight row of position p is also
+ * written to row p of w_out, for a caller that wants the updated rows at hand (the cold-data cache
+ * takes in the rows it just applied, python/EmbCache/server.py:499-544) without reading them back
+ * over the link. */
 int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,
                                 const int64_t* count, int64_t max_count, int64_t dim, float* w,
-                                float* s, int64_t stride, float lr, float eps, void* stream);
+                                float* s, int64_t stride, float* w_out, float lr, float eps,
+                                void* stream);
 
 /* The same arithmetic over one class of a class-ordered combine: the rows u of (ukeys, grad) in
  * [0, class_split[1]) for which = 0 or [class_split[1], num_unique[0]) for which = 1; the table row

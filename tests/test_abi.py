@@ -68,9 +68,9 @@ def test_argument_errors_of_the_split_schedule_entry_points():
     assert lib.hades_set_listed(one, one, 3, one, one, one, 10, 8, _lib.F32, null) == 1
     assert lib.hades_set_listed(null, null, 0, null, null, null, 0, 8, _lib.F32, null) == 0
     # listed / class Adagrad
-    assert lib.hades_adagrad_update_listed(one, one, one, one, 10, 8, one, one, 4, 0.01, 1e-10, null) == 1
-    assert lib.hades_adagrad_update_listed(one, one, one, null, 10, 8, one, one, 0, 0.01, 1e-10, null) == 1
-    assert lib.hades_adagrad_update_listed(null, null, null, null, 0, 8, null, null, 0, 0.01, 1e-10, null) == 0
+    assert lib.hades_adagrad_update_listed(one, one, one, one, 10, 8, one, one, 4, null, 0.01, 1e-10, null) == 1
+    assert lib.hades_adagrad_update_listed(one, one, one, null, 10, 8, one, one, 0, null, 0.01, 1e-10, null) == 1
+    assert lib.hades_adagrad_update_listed(null, null, null, null, 0, 8, null, null, 0, null, 0.01, 1e-10, null) == 0
     assert lib.hades_adagrad_update_class(one, one, one, one, 2, 255, 10, 8, one, one, 0, null, null,
                                           0.01, 1e-10, null) == 1                              # which
     assert lib.hades_adagrad_update_class(one, one, one, one, 0, 255, 10, 8, one, one, 0, one, null,

@@ -1769,3 +1769,31 @@ def test_pipelined_keyed_steps_equal_one_batch_at_a_time(lib, N, D, H, n, hot_fr
             got = tables(pipe)
             assert np.array_equal(got[0].numpy(), cw) and np.array_equal(got[1].numpy(), cs)
             assert np.array_equal(got[2].numpy(), hw) and np.array_equal(got[3].numpy(), hs)
+
+
+@pytest.mark.parametrize("host", [False, True])
+def test_listed_adagrad_also_returns_the_new_rows(lib, host):
+    """hades_adagrad_update_listed with w_out: tables as without it (bit-equal to the oracle), and
+    row p of w_out = the new weight row of position p for the listed positions, untouched elsewhere."""
+    _, ops = lib
+    rng = np.random.default_rng(77)
+    N, D, n = 4000, 96, 3000
+    w0 = rng.standard_normal((N, D)).astype(np.float32)
+    s0 = np.abs(rng.standard_normal((N, D))).astype(np.float32)
+    idx = rng.permutation(N)[:n].astype(np.int64)            # distinct rows
+    grad = (rng.standard_normal((n, D)) * 1e-2).astype(np.float32)
+    pos = rng.permutation(n)[: n - 200].astype(np.int64)
+    live = pos.size - 13
+    t_w = torch.from_numpy(w0.copy()); t_s = torch.from_numpy(s0.copy())
+    t_w = t_w.pin_memory() if host else t_w.cuda()
+    t_s = t_s.cuda()
+    out = torch.full((n, D), 5.0, dtype=torch.float32, device="cuda")
+    ops.adagrad_update_listed_(dev(idx), dev(grad), dev(pos), torch.tensor([live], device="cuda"),
+                               t_w, t_s, 0.01, 1e-10, w_out=out)
+    torch.cuda.synchronize()
+    w, st = w0.copy(), s0.copy()
+    O.adagrad_listed(idx, grad, pos, live, w, st, 0.01, 1e-10)
+    assert np.array_equal(t_w.cpu().numpy(), w) and np.array_equal(t_s.cpu().numpy(), st)
+    want = np.full((n, D), 5.0, np.float32)
+    want[pos[:live]] = w[idx[pos[:live]]]
+    assert np.array_equal(out.cpu().numpy(), want)
