@@ -377,7 +377,10 @@ class _SparseRowOptimizer:
         `fetched_rows` = the rows forward_keyed returned for this batch: the cold update then takes
         the old weights from them instead of reading the cold table a second time (half the
         host-link traffic of the update).  The caller vouches that nothing has written the table
-        since that forward pass - true for a trainer with one batch in flight."""
+        since that forward pass - true for a trainer with one batch in flight.
+
+        join=False returns without making the current stream wait for the cold update; the caller
+        then calls finish_prefetch(...) or join() before it reads the cold table on that stream."""
         plan, bufs = state
         cold = self._split_state()
         cur = torch.cuda.current_stream()
