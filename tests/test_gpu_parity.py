@@ -1797,3 +1797,39 @@ def test_listed_adagrad_also_returns_the_new_rows(lib, host):
     want = np.full((n, D), 5.0, np.float32)
     want[pos[:live]] = w[idx[pos[:live]]]
     assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_pipelined_keyed_steps_with_batches_of_different_sizes(lib):
+    """The pipelined calls with a different number of ids in every batch (the buffer sets are sized
+    by the largest so far; an empty batch in the middle): rows and tables as one batch at a time."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad
+    rng = np.random.default_rng(2024)
+    N, D, H = 4000, 64, 400
+    cold, hot_ids, _ = _split_case(rng, N, D, H, 10, 0.5)
+    sizes = [3000, 1200, 5000, 0, 2500, 64, 5000]
+    qs = [rng.integers(0, N, m).astype(np.int64) for m in sizes]
+    grads = [(rng.standard_normal((m, D)) * 1e-2).astype(np.float32) for m in sizes]
+
+    def make():
+        return SparseAdagrad(torch.from_numpy(cold.copy()).pin_memory(), torch.from_numpy(hot_ids))
+
+    seq, pipe = make(), make()
+    seq_rows = []
+    for q, g in zip(qs, grads):
+        rows, st = seq.forward_keyed(dev(q))
+        seq_rows.append(rows.clone())
+        seq.backward_keyed(st, dev(g), mode=ops.COMBINE_EXACT, fetched_rows=rows)
+    bufs = [torch.empty((max(sizes), D), dtype=torch.float32, device="cuda") for _ in range(2)]
+    rows, st = pipe.forward_keyed(dev(qs[0]), out=bufs[0][:sizes[0]], slot=0)
+    for k in range(len(sizes)):
+        assert torch.equal(rows, seq_rows[k]), k
+        nxt = None
+        if k + 1 < len(sizes):
+            nxt = pipe.prefetch_keyed(dev(qs[k + 1]), slot=(k + 1) % 2, out=bufs[(k + 1) % 2][:sizes[k + 1]])
+        pipe.backward_keyed(st, dev(grads[k]), mode=ops.COMBINE_EXACT, fetched_rows=rows, join=nxt is None)
+        if nxt is not None:
+            rows, st = pipe.finish_prefetch(nxt, after=st)
+    torch.cuda.synchronize()
+    for name in ("cold_w", "cold_s", "hot_w", "hot_s"):
+        assert torch.equal(getattr(seq, name).cpu(), getattr(pipe, name).cpu()), name
