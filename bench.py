@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]      the headline workload (cfg3) + cfg2 nested
     python bench.py --workload cfg2|cfg3|cfg5 [--mode fast|exact] [--schedule serial|keyed|pipelined|split|overlap|graph]
+                    [--reuse-rows] [--optimizer adagrad|adam]
     python bench.py --workload cfg4          cold-gradient accumulator with delayed write-back
     python bench.py --workload cfg4 --flush-rule staleness    the cache server's own per-row rule
     python bench.py --workload neighbours    pre-exchange bucketing, index cache, cold-data cache
