@@ -1833,3 +1833,24 @@ def test_pipelined_keyed_steps_with_batches_of_different_sizes(lib):
     torch.cuda.synchronize()
     for name in ("cold_w", "cold_s", "hot_w", "hot_s"):
         assert torch.equal(getattr(seq, name).cpu(), getattr(pipe, name).cpu()), name
+
+
+def test_prefetch_without_a_batch_before_it(lib):
+    """prefetch_keyed + finish_prefetch(after=None) as the first call of a run gives what
+    forward_keyed gives, and the backward half that follows leaves the same tables."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad
+    rng = np.random.default_rng(5)
+    N, D, H, n = 6000, 32, 600, 5000
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, 0.6)
+    grad = (rng.standard_normal((n, D)) * 1e-2).astype(np.float32)
+    a = SparseAdagrad(torch.from_numpy(cold.copy()).pin_memory(), torch.from_numpy(hot_ids))
+    b = SparseAdagrad(torch.from_numpy(cold.copy()).pin_memory(), torch.from_numpy(hot_ids))
+    rows_a, st_a = a.forward_keyed(dev(q))
+    rows_b, st_b = b.finish_prefetch(b.prefetch_keyed(dev(q), slot=0))
+    assert torch.equal(rows_a, rows_b)
+    a.backward_keyed(st_a, dev(grad), mode=ops.COMBINE_EXACT)
+    b.backward_keyed(st_b, dev(grad), mode=ops.COMBINE_EXACT, fetched_rows=rows_b)
+    torch.cuda.synchronize()
+    for name in ("cold_w", "cold_s", "hot_w", "hot_s"):
+        assert torch.equal(getattr(a, name).cpu(), getattr(b, name).cpu()), name
