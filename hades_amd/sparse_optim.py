@@ -287,6 +287,10 @@ class _SparseRowOptimizer:
         b = sets.get(slot)
         if b is None or b["keys"].numel() < n:
             dev = self.device
+            if b is not None:
+                # a larger batch: the old set may still be read on a side stream, and the caching
+                # allocator hands freed blocks back without asking the side streams
+                torch.cuda.synchronize(dev)
             i64 = lambda k: torch.empty(k, dtype=torch.int64, device=dev)
             b = {"split": (i64(n), i64(n), i64(n), i64(2)), "keys": i64(n), "ukeys": i64(n),
                  "nu": i64(1), "class_split": i64(2),
