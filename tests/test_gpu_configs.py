@@ -163,6 +163,70 @@ def test_cfg3_full_size_fetch_and_update(cuda_device, schedule):
     assert np.array_equal(ow, base) and not os_.any()
 
 
+def test_cfg3_full_size_keyed_and_pipelined(cuda_device):
+    """cfg3 at full size on the schedules the benchmark times: batch A through forward_keyed;
+    batch B prefetched on the side streams while A's backward half runs (its cold update takes
+    the old rows from the fetched ones); B's rows completed by finish_prefetch.  A's rows equal
+    plain indexing of the tables before the step; the weight and state rows of sampled distinct
+    ids of A (hot, cold, ids beyond 2^31 elements) equal the oracle's Adagrad on their old rows
+    and summed gradients; B's whole batch of rows equals plain indexing of the tables AFTER A's
+    update - among them the cold rows that A's update wrote while B's gather was under way."""
+    from hades_amd import ops, synth
+    from hades_amd.sparse_optim import SparseAdagrad
+    cfg = synth.CONFIGS["cfg3"]
+    N, D, H, n = cfg["num_rows"], cfg["dim"], cfg["num_hot"], cfg["batch"]
+    dev = cuda_device
+    table = _alloc_or_skip(lambda: torch.empty((N, D), dtype=torch.float32, pin_memory=True),
+                           "cfg3 needs a 56.8 GB page-locked table")
+    synth.fill_normal_(table, 0.01, 1237)
+    hot_ids = synth.hot_ids(N, H, dev)
+    opt = _alloc_or_skip(lambda: SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=dev,
+                                               state_on_device=True), "cfg3 needs 70 GB of HBM")
+    opt.hot_w += 1.0
+    sampler = synth.ZipfSampler(N, cfg["zipf_s"], dev)
+    qa = synth.make_ids(sampler, N, n, 1237_000)
+    qb = synth.make_ids(sampler, N, n, 1237_001)
+    del sampler
+    # make sure B asks for cold rows that A updates: a few thousand of A's cold ids go into B
+    pa = torch.searchsorted(hot_ids, qa, right=True)
+    a_cold = qa[~((pa > 0) & (hot_ids[(pa - 1).clamp(min=0)] == qa))]
+    qb[:3000] = a_cold[:3000]
+    g = synth.make_grads(n, D, 1237_500, dev)
+
+    def plain_rows(q):
+        p = torch.searchsorted(hot_ids, q, right=True)
+        hit = (p > 0) & (hot_ids[(p - 1).clamp(min=0)] == q)
+        want = _rows_of(opt.cold_w, q)
+        want[hit] = opt.hot_w[(p - 1)[hit]]
+        return want
+
+    want_a = plain_rows(qa)
+    uq = torch.unique(qa)
+    gen = torch.Generator().manual_seed(7)
+    pick = torch.randperm(uq.numel(), generator=gen)[:5000].to(dev)
+    sample = torch.unique(torch.cat([uq[pick], uq[-1000:], a_cold[:500]]))
+    w0, s0, s_hit = _table_rows(opt, sample)
+    assert 0 < int(s_hit.sum()) < sample.numel()
+    rows_a, st_a = opt.forward_keyed(qa, slot=0)
+    torch.cuda.synchronize()
+    assert torch.equal(rows_a, want_a)
+    del want_a
+    nxt = opt.prefetch_keyed(qb, slot=1)
+    ukeys, sums, cnts, nu, split = opt.backward_keyed(st_a, g, mode=ops.COMBINE_EXACT,
+                                                      fetched_rows=rows_a, join=False)
+    rows_b, st_b = opt.finish_prefetch(nxt, after=st_a)
+    torch.cuda.synchronize()
+    U = int(nu.item())
+    assert U == uq.numel() and int(cnts[:U].sum()) == n
+    ids = opt.distinct_ids_of(ukeys, nu)
+    order = torch.argsort(ids)
+    assert torch.equal(ids[order], uq)
+    w1, s1 = _sampled_update_check(opt, ids[order], sums[:U][order], U, (w0, s0), sample)
+    gw, gs, _ = _table_rows(opt, sample)
+    assert np.array_equal(gw, w1) and np.array_equal(gs, s1)
+    assert torch.equal(rows_b, plain_rows(qb))
+
+
 def test_cfg5_full_size_local_aggregation_and_update(cuda_device):
     """Four 256 K batches over a 244 M x 64 table in HBM (62.5 GB plus as much Adagrad state):
     combine of the concatenation, then the update; sampled rows against the oracle, the rest of a
