@@ -737,10 +737,16 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
     total_bytes = sum(alg_bytes.values())
     res = {"workload": wl.describe(), "schedule": schedule, "n": n,
            "ms_per_step": ms_per_step,
-           "step_us": {"mean": round(ms_per_step * 1e3, 1), "median": round(pct(step_ms, 50) * 1e3, 1),
+           "step_us": {"mean": round(ms_per_step * 1e3, 1),
+                       "mean_by_events": round(sum(step_ms) / len(step_ms) * 1e3, 1),
+                       "max": round(max(step_ms) * 1e3, 1),
+                       "slow_steps": [(i, round(t * 1e3, 1)) for i, t in enumerate(step_ms)
+                                      if t > 1.3 * pct(step_ms, 50)],
+                       "median": round(pct(step_ms, 50) * 1e3, 1),
                        "p10": round(pct(step_ms, 10) * 1e3, 1), "p90": round(pct(step_ms, 90) * 1e3, 1),
-                       "note": "mean: wall clock over the K timed steps; median/p10/p90: the same "
-                               "steps by HIP events at the step boundaries"},
+                       "note": "mean: wall clock over the K timed steps; the rest: the same steps by HIP "
+                               "events at the step boundaries (slow_steps: index and time of those "
+                               "above 1.3 x the median)"},
            "roofline": roofline, "kernels": kernels,
            "phases": per_phase,
            "phases_note": "from a second, untimed pass with four event records per step (each adds "
