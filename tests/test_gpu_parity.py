@@ -1854,3 +1854,33 @@ def test_prefetch_without_a_batch_before_it(lib):
     torch.cuda.synchronize()
     for name in ("cold_w", "cold_s", "hot_w", "hot_s"):
         assert torch.equal(getattr(a, name).cpu(), getattr(b, name).cpu()), name
+
+
+def test_listed_adam_partial_count_and_strided_tables(lib):
+    """hades_adam_update_listed over a position list with a device-side count, on tables whose
+    rows are views of one [N, 3, D] block (weights, mem, power of a row next to each other):
+    listed rows follow the oracle's adam_listed, every other row and the step counters of
+    untouched rows stay as they were."""
+    _, ops = lib
+    rng = np.random.default_rng(88)
+    N, D, n = 3000, 48, 2000
+    block = (rng.standard_normal((N, 3, D)) * 0.1).astype(np.float32)
+    block[:, 2] = np.abs(block[:, 2])                         # power >= 0
+    step0 = rng.integers(0, 5, N).astype(np.float32)
+    t_block = torch.from_numpy(block.copy()).cuda()
+    t_step = torch.from_numpy(step0.copy()).cuda()
+    idx = rng.permutation(N)[:n].astype(np.int64)
+    grad = (rng.standard_normal((n, D)) * 1e-2).astype(np.float32)
+    pos = rng.permutation(n)[: n - 300].astype(np.int64)
+    live = pos.size - 21
+    ops.adam_update_listed_(dev(idx), dev(grad), dev(pos), torch.tensor([live], device="cuda"),
+                            (t_block[:, 0], t_step, t_block[:, 1], t_block[:, 2]), 0.01, 0.9, 0.999, 1e-8)
+    torch.cuda.synchronize()
+    w, m, v, st = block[:, 0].copy(), block[:, 1].copy(), block[:, 2].copy(), step0.copy()
+    O.adam_listed(idx, grad, pos, live, w, st, m, v, 0.01, 0.9, 0.999, 1e-8)
+    got = t_block.cpu().numpy()
+    touched = np.zeros(N, bool); touched[idx[pos[:live]]] = True
+    assert np.array_equal(t_step.cpu().numpy(), st)
+    assert np.array_equal(got[~touched], block[~touched])
+    assert np.abs(got[:, 0] - w).max() <= 1e-4 * 0.01                       # as in test_adam_update
+    assert np.allclose(got[:, 1], m, rtol=1e-6, atol=1e-12) and np.allclose(got[:, 2], v, rtol=1e-6, atol=1e-12)
