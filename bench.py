@@ -985,10 +985,8 @@ def run_cfg4_staleness(args):
     hotness, count threshold 16) in front of the pinned-host table.  Per step: combine the batch;
     gradients of cached ids accumulate in their slots; the other ids are applied to the host
     table at once and their rows enter the cache; rows that are due leave the cache and are
-    applied.  One host synchronisation per step (the number of uncached ids sizes the row fetch).
-    Prints its own JSON line."""
+    applied.  No host synchronisation inside a step.  Prints its own JSON line."""
     import torch
-    import hades_amd.EmbCacheLib as E
     from hades_amd import ops, synth
     from hades_amd.cold_cache import ColdDataCache
     dev = torch.device("cuda:0")
@@ -1027,29 +1025,36 @@ def run_cfg4_staleness(args):
                 torch.empty(n, dtype=torch.int64, device=dev),
                 torch.empty(1, dtype=torch.int64, device=dev))
     fetched = torch.empty((n, D), dtype=torch.float32, device=dev)
-    m_cnt = torch.zeros(1, dtype=torch.int64, device=dev)
     log("workload ready")
     stats = {"miss": 0, "hit": 0, "flushed": 0}
 
+    positions = torch.arange(n, dtype=torch.int64, device=dev)
+    minus_one = torch.full((n,), -1, dtype=torch.int64, device=dev)
+    zero = torch.zeros(n, dtype=torch.int64, device=dev)
+    split_ws = ops.Workspace(dev)
+
     def step(i, count=False):
+        """No host synchronisation: the number of distinct ids stays on the device, the entries
+        past it are given the id -1 (no cache line: every cache operator answers -1 for them and
+        leaves them alone), and the uncached ids go through position lists with device counts."""
         q, g = ids[i], grads[i % ng]
         uids, sums, cnts, nu = ops.combine_padded(q, g, id_bound=N, workspace=ws, out=comb_out)
-        u = int(nu.item())
-        uids, sums = uids[:u], sums[:u]
-        locs = cache.accumulate_gradients_cold_remote(uids, sums)          # cached ids: delayed
-        _, hit_pos, miss_pos = ops.split(locs)
-        if miss_pos.numel():
-            # the update hands back the new rows (w_out), which are the rows a trainer would pull
-            # next: no third crossing of the link to fetch them for the cache
-            m_cnt.fill_(miss_pos.numel())
-            ops.adagrad_update_listed_(uids, sums, miss_pos, m_cnt, cold_w, cold_s, 0.01, 1e-10,
-                                       w_out=fetched[:u])
-            cache.update_cache(uids[miss_pos], fetched[:u][miss_pos])
+        live = positions < nu
+        live_ids = torch.where(live, uids, minus_one)
+        locs = cache.accumulate_gradients_cold_remote(live_ids, sums)      # cached ids: delayed
+        miss = live & (locs < 0)
+        _, _, miss_pos, counts = ops.split_padded(torch.where(miss, minus_one, zero), workspace=split_ws)
+        # the uncached ids are applied at once; the update hands back the new rows (w_out), which
+        # are the rows a trainer would pull next: no third crossing of the link for the cache
+        ops.adagrad_update_listed_(uids, sums, miss_pos, counts[1:2], cold_w, cold_s, 0.01, 1e-10,
+                                   w_out=fetched)
+        cache.update_cache(torch.where(miss, uids, minus_one), fetched)
         f_ids, f_grads, f_cnts, f_num = cache.staled_gradients_remote_padded(slots)
         ops.adagrad_update_(f_ids, f_grads, None, None, cold_w, cold_s, None, 0.01, 1e-10,
                             num_unique=f_num)
         if count:
-            stats["miss"] += int(miss_pos.numel()); stats["hit"] += int(hit_pos.numel())
+            m = int(counts[1].item())
+            stats["miss"] += m; stats["hit"] += int(nu.item()) - m
             stats["flushed"] += int(f_num.item())
 
     for i in range(warm):

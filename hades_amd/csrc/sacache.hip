@@ -131,11 +131,11 @@ __global__ __launch_bounds__(kThreads) void sac_walk_kernel(
   const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (j >= n) return;
   const uint32_t ln = sorted_line[j];
-  if (j > 0 && sorted_line[j - 1] == ln) return;  // not the first id of its line
-  if (static_cast<int64_t>(ln) >= lines) {       // ids without a line (negative)
-    for (int64_t k = j; k < n && sorted_line[k] == ln; ++k) locs[perm[k]] = -1;
-    return;
+  if (static_cast<int64_t>(ln) >= lines) {       // ids without a line (negative; e.g. the padding
+    locs[perm[j]] = -1;                          // of a batch whose length lives on the device):
+    return;                                      // every thread answers for its own entry
   }
+  if (j > 0 && sorted_line[j - 1] == ln) return;  // not the first id of its line
   Line l;
   load_line(line_ids, line_age, ln, l);
   for (int64_t k = j; k < n && sorted_line[k] == ln; ++k) {

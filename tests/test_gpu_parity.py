@@ -1884,3 +1884,46 @@ def test_listed_adam_partial_count_and_strided_tables(lib):
     assert np.array_equal(got[~touched], block[~touched])
     assert np.abs(got[:, 0] - w).max() <= 1e-4 * 0.01                       # as in test_adam_update
     assert np.allclose(got[:, 1], m, rtol=1e-6, atol=1e-12) and np.allclose(got[:, 2], v, rtol=1e-6, atol=1e-12)
+
+
+def test_cold_data_cache_with_padding_entries(lib):
+    """Batches padded with the id -1 (the entries past a device-side length): the index cache
+    and the cold-data cache answer -1 for them and evolve exactly as with the compacted batch -
+    locs of the real ids, line contents, ages, slot arrays and the flushed rows."""
+    _, ops = lib
+    from hades_amd.cold_cache import ColdDataCache
+    rng = np.random.default_rng(321)
+    N, D, slots = 50_000, 32, 4096
+    hotness = torch.from_numpy(rng.random(N).astype(np.float32) * 3).cuda()
+    a = ColdDataCache(slots, D, hotness, cnt_threshold=4)
+    b = ColdDataCache(slots, D, hotness, cnt_threshold=4)
+    for it in range(6):
+        m = 3000
+        ids = rng.permutation(N)[:m].astype(np.int64)
+        rows = rng.standard_normal((m, D)).astype(np.float32)
+        grads = rng.standard_normal((m, D)).astype(np.float32)
+        # the padded form: the real entries scattered over 2.5 x as many positions, -1 elsewhere
+        P = 7500
+        where = np.sort(rng.permutation(P)[:m])
+        pid = np.full(P, -1, np.int64); pid[where] = ids
+        prow = rng.standard_normal((P, D)).astype(np.float32); prow[where] = rows
+        pgrad = rng.standard_normal((P, D)).astype(np.float32); pgrad[where] = grads
+        la = a.accumulate_gradients_cold_remote(dev(ids), dev(grads))
+        lb = b.accumulate_gradients_cold_remote(dev(pid), dev(pgrad))
+        assert np.array_equal(lb.cpu().numpy()[where], la.cpu().numpy())
+        assert (np.delete(lb.cpu().numpy(), where) == -1).all()
+        miss = la.cpu().numpy() < 0
+        ua = a.update_cache(dev(ids[miss]), dev(rows[miss]))
+        pid2 = np.full(P, -1, np.int64); pid2[where[miss]] = ids[miss]
+        ub = b.update_cache(dev(pid2), dev(prow))
+        assert np.array_equal(ub.cpu().numpy()[where[miss]], ua.cpu().numpy())
+        fa = a.staled_gradients_remote_padded(slots)
+        fb = b.staled_gradients_remote_padded(slots)
+        k = int(fa[3].item())
+        assert k == int(fb[3].item())
+        for x, y in zip(fa[:3], fb[:3]):
+            assert torch.equal(x[:k], y[:k])
+    torch.cuda.synchronize()
+    for name in ("emb_cache_buff", "grad_cache_buff", "grad_cnt_cache_buff", "grad_idx_cache_buff"):
+        assert torch.equal(getattr(a, name), getattr(b, name)), name
+    assert torch.equal(a.index.line_ids, b.index.line_ids) and torch.equal(a.index.line_age, b.index.line_age)
