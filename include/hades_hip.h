@@ -474,7 +474,8 @@ int hades_bucket_by_owner(const int64_t* ids, int64_t n, const int64_t* range_pa
  * src/pybind.cc:17-36).  State is two caller-owned device arrays:
  *   line_ids int64[lines * 8]  (-1 = empty entry),  line_age int32[lines * 8]  (LRU ages);
  * an id lives in line id % lines and its loc is line * 8 + entry.  Negative ids are never cached
- * (loc -1).  Batches are handled in input order line by line, which is what the reference's
+ * (loc -1, nothing changes): a batch whose length is only known on the device can be padded with
+ * -1 and passed at its capacity.  Batches are handled in input order line by line, which is what the reference's
  * loops give with one OpenMP thread.
  *   init          constructor + _init_cache (cache.h:41-48, cache_line.h:13-18)
  *   add           _add (cache.h:51-91): loc of each id after insertion, -1 if its line has no victim
