@@ -26,6 +26,7 @@ _L = c_int64
 KERNEL_NONE, KERNEL_CACHED_FETCH, KERNEL_SEG_SUM, KERNEL_ADAGRAD, KERNEL_RADIX_PASS = 0, 1, 2, 3, 4
 KERNEL_HASH_ACCUMULATE = 5
 KERNEL_ADAM = 6
+ABI_VERSION = 120      # HADES_ABI_VERSION of include/hades_hip.h
 
 _SIGNATURES = {
     "hades_profile_kernel": [c_int, _P, _P],
@@ -123,6 +124,10 @@ def load():
     lib.hades_last_error.argtypes = []
     lib.hades_version.restype = c_int
     lib.hades_version.argtypes = []
+    if lib.hades_version() != ABI_VERSION:
+        raise RuntimeError("%s was built from other sources (interface version %d, this binding "
+                           "expects %d): rebuild it with `python -m hades_amd.build`"
+                           % (LIB_PATH, lib.hades_version(), ABI_VERSION))
     for name, argtypes in _SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = c_int

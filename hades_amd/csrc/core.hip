@@ -61,7 +61,7 @@ extern "C" {
 
 const char* hades_last_error(void) { return g_last_error.c_str(); }
 
-int hades_version(void) { return 100; }
+int hades_version(void) { return HADES_ABI_VERSION; }
 
 int hades_profile_kernel(int kernel_id, void* start_event, void* stop_event) {
   HADES_REQUIRE(kernel_id >= 0 && kernel_id <= HADES_KERNEL_LAST, "unknown kernel id %d", kernel_id);

@@ -53,6 +53,9 @@ extern "C" {
 #define HADES_COMBINE_EXACT 1 /* strictly sequential sum in occurrence order: bit-equal to CPU index_add_ */
 
 const char* hades_last_error(void);
+/* Version of this interface; raised whenever a signature changes, so that a binding can refuse a
+ * library built from other sources. */
+#define HADES_ABI_VERSION 120
 int hades_version(void);
 
 /* Kernel timing hook (no counterpart in the reference, whose scripts time whole calls from the

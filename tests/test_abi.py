@@ -117,3 +117,13 @@ def test_workspace_queries():
     assert 0 < a < b
     assert _lib.query("hades_split_compact_workspace_bytes", 1_000_000) >= 1_000_000
     assert _lib.query("hades_hash_flush_workspace_bytes", 1 << 22, 1 << 22) > (1 << 22) * 8
+
+
+def test_interface_version_agrees_between_header_binding_and_library():
+    """HADES_ABI_VERSION of the header, the number the Python binding expects and what the built
+    library reports are one number: a library built from other sources is refused at load."""
+    import re
+    from hades_amd import _lib
+    header = open(os.path.join(ROOT, "include", "hades_hip.h")).read()
+    v = int(re.search(r"#define HADES_ABI_VERSION (\d+)", header).group(1))
+    assert v == _lib.ABI_VERSION == _lib.load().hades_version()
