@@ -146,3 +146,22 @@ def test_split_schedule_objects_need_no_gpu_to_import():
     from hades_amd import sparse_optim
     for name in ("fetch_split", "update_split", "step_split", "forward_keyed", "backward_keyed", "join"):
         assert callable(getattr(sparse_optim.SparseAdagrad, name))
+
+
+def test_bench_percentile_and_committed_traffic_summaries():
+    """bench.py's percentile helper, and the HBM-traffic figures it reads from the committed
+    counter summaries: every workload it nests in the default run has its kernels' lines, and
+    each figure lies within a factor of two of the kernel's algorithmic bytes at that workload."""
+    import bench
+    assert bench.pct([3.0, 1.0, 2.0], 50) == 2.0 and bench.pct([1.0, 2.0], 50) == 1.5
+    assert bench.pct([5.0], 90) == 5.0 and bench.pct([0.0, 10.0], 10) == 1.0
+    t3 = bench.measured_traffic("cfg3", "fast")
+    assert set(t3) >= {"hot_fetch", "seg_sum", "hot_update"}
+    n_hot, u_hot, D = 923_828, 243_433, 128
+    alg = {"hot_fetch": n_hot * (16 + 8 * D), "seg_sum": n_hot * (8 + 4 * D) + u_hot * 4 * D,
+           "hot_update": u_hot * (8 + 20 * D)}
+    for k, a in alg.items():
+        assert 0.5 * a < t3[k] < 2 * a, (k, t3[k], a)
+    t2 = bench.measured_traffic("cfg2", "fast")
+    assert set(t2) >= {"fetch", "seg_sum", "update"}
+    assert bench.measured_traffic("cfg2", "exact") == {} and bench.measured_traffic("no-such", "fast") == {}
