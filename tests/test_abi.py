@@ -76,6 +76,12 @@ def test_argument_errors_of_the_split_schedule_entry_points():
     assert lib.hades_adagrad_update_class(one, one, one, one, 0, 255, 10, 8, one, one, 0, one, null,
                                           0.01, 1e-10, null) == 1                              # rows without positions
     assert b"go together" in lib.hades_last_error()
+    # listed gather restricted to a set
+    assert lib.hades_fetch_listed_in_set(one, 4, one, one, one, 10, one, one, 5, one, 8, _lib.F32, null) == 1   # stride < dim
+    assert lib.hades_fetch_listed_in_set(one, 0, one, one, one, 10, null, one, 5, one, 8, _lib.F32, null) == 1  # set is null
+    assert lib.hades_fetch_listed_in_set(one, 0, one, one, one, 10, one, one, -1, one, 8, _lib.F32, null) == 1  # set_max
+    assert lib.hades_fetch_listed_in_set(null, 0, null, null, null, 10, null, null, 0, null, 8, _lib.F32, null) == 0  # empty set
+    assert lib.hades_fetch_listed_in_set(null, 0, null, null, null, 0, null, null, 5, null, 8, _lib.F32, null) == 0   # empty list
     # listed / class Adam
     assert lib.hades_adam_update_listed(one, one, one, one, 10, 8, one, one, one, one, 4, 0.01, 0.9, 0.999,
                                         1e-8, null) == 1                                       # stride < dim
