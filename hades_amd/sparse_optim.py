@@ -203,6 +203,9 @@ class _SparseRowOptimizer:
         split_done = torch.cuda.Event()
         split_done.record(cur)
         cold.wait_event(split_done)
+        if cold != cur:       # memory of the caller's stream, used on another one
+            out.record_stream(cold)
+            ids.record_stream(cold)
         with torch.cuda.stream(cold):
             self._timed(timing, "cold_fetch", cold,
                         lambda: ops.fetch_listed(self.cold_w, ids, cold_pos, counts[1:2], out))
@@ -265,6 +268,9 @@ class _SparseRowOptimizer:
         split_done = torch.cuda.Event()
         split_done.record(cur)
         cold.wait_event(split_done)
+        if cold != cur:       # memory of the caller's stream, used on another one
+            out.record_stream(cold)
+            ids.record_stream(cold)
         with torch.cuda.stream(cold):
             self._timed(timing, "cold_fetch", cold,
                         lambda: ops.fetch_listed(self.cold_w, ids, cold_pos, counts[1:2], out))
@@ -329,6 +335,8 @@ class _SparseRowOptimizer:
         kb = ops.key_bits_for(max(self.num_rows, self.hot_ids.numel(), 2))
         bufs = self._keyed_bufs(n, slot)
         pre.wait_stream(cur)      # the ids, and everything that last used this slot's buffers
+        out.record_stream(pre)    # memory of the caller's stream, used on another one
+        ids.record_stream(pre)
         with torch.cuda.stream(pre):
             loc, hot_pos, cold_pos, counts = ops.lookup_split(
                 ids, self.hot_set, workspace=bufs["split_ws"], out=bufs["split"],
@@ -395,6 +403,8 @@ class _SparseRowOptimizer:
         cold_summed = torch.cuda.Event()
         cold_summed.record(cur)
         cold.wait_event(cold_summed)
+        if fetched_rows is not None and cold != cur:
+            fetched_rows.record_stream(cold)
         with torch.cuda.stream(cold):
             self._timed(timing, "cold_update", cold,
                         lambda: self._update_keyed(plan, out[0], 0, fetched_rows))
