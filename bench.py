@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]      the headline workload (cfg3) + cfg2 nested
     python bench.py --workload cfg2|cfg3|cfg5 [--mode fast|exact] [--schedule serial|keyed|pipelined|split|overlap|graph]
-                    [--reuse-rows] [--optimizer adagrad|adam]
+                    [--no-reuse-rows] [--optimizer adagrad|adam]
     python bench.py --workload cfg4          cold-gradient accumulator with delayed write-back
     python bench.py --workload cfg4 --flush-rule staleness    the cache server's own per-row rule
     python bench.py --workload neighbours    pre-exchange bucketing, index cache, cold-data cache
@@ -72,10 +72,14 @@ def parse_args():
                          "ids; overlap: serial with the sort of "
                          "the ids on a side stream next to the fetch; graph: serial, every step the "
                          "replay of a HIP graph captured once per batch")
-    ap.add_argument("--reuse-rows", action="store_true",
-                    help="keyed schedule only: the cold update takes the old weight rows from the "
-                         "rows the step's own fetch brought in instead of reading the host table "
-                         "again (valid with one batch in flight per table)")
+    ap.add_argument("--no-reuse-rows", dest="reuse_rows", action="store_false",
+                    help="keyed / pipelined schedules: make the cold update read the old weight rows "
+                         "from the host table again.  By default it takes them from the rows the "
+                         "step's own fetch brought in whenever the optimizer can tell that nothing "
+                         "has written the table in between (backward_keyed's guarded default)")
+    ap.add_argument("--allow-fallback", action="store_true",
+                    help="if the host refuses cfg3's page-locked table, measure cfg2 instead and say "
+                         "so in config.fallback (without this flag such a run exits non-zero)")
     ap.add_argument("--flush-rule", default="every8", choices=["every8", "staleness"],
                     help="cfg4 only: write the accumulated cold gradients back every 8 steps (hash "
                          "accumulator), or per row by the cache server's staleness rule (cold-data "
@@ -353,7 +357,7 @@ def parity_gate(wl, step_fn, rows=20_000):
             "against": "torch device ops (searchsorted, indexing, unique + float64 index_add_, %s)" % form}
 
 
-def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows=False):
+def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows=True):
     import torch
     from hades_amd import ops
     dev = torch.device("cuda:0")
@@ -378,6 +382,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         return evs
 
     uids_o, sums_o, cnts_o, nu_o = wl.comb_out
+    reused = {"yes": 0, "no": 0}    # backward halves that took / did not take the forward rows
 
     def run_step(q, g, cmode, events=None, timing=None):
         """fetch -> combine -> update of one batch.
@@ -403,7 +408,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
             if events: events[1].record()
             if events: events[2].record()
             res = opt.backward_keyed(state, g, cmode, timing=timing,
-                                     fetched_rows=rows if reuse_rows else None)
+                                     fetched_rows="auto" if reuse_rows else None)
+            reused["yes" if state[0].reused_rows else "no"] += 1
         elif split:
             opt.fetch_split(q, out=rows, join=False, timing=timing)
             plan = ops.combine_plan(q, D, id_bound=N, workspace=opt._ws, out=out_ids)
@@ -449,7 +455,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         if events: events[1].record()
         if events: events[2].record()
         res = opt.backward_keyed(st, wl.grads[i % nb], cmode, timing=timing,
-                                 fetched_rows=rows if reuse_rows else None, join=False)
+                                 fetched_rows="auto" if reuse_rows else None, join=False)
+        reused["yes" if st[0].reused_rows else "no"] += 1
         rows2, st2 = opt.finish_prefetch(nxt, after=st, timing=timing)
         if events: events[3].record()
         pipe.update(i=i + 1, rows=rows2, state=st2)
@@ -470,7 +477,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
             rows, st = opt.forward_keyed(q, out=row_bufs[0][:q.numel()], slot=0)
             rows = rows.clone()
             nxt = opt.prefetch_keyed(q, slot=1, out=row_bufs[1][:q.numel()])
-            res = opt.backward_keyed(st, g, m, fetched_rows=rows if reuse_rows else None, join=False)
+            res = opt.backward_keyed(st, g, m, fetched_rows="auto" if reuse_rows else None, join=False)
             rows2, _ = opt.finish_prefetch(nxt, after=st)
             torch.cuda.synchronize()
             want2 = ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_set)
@@ -701,7 +708,15 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
                 (mk["launches_timed"], K) if schedule != "graph" else "eager steps before the timed region",
                 "timing": "HIP events recorded on the launch stream right before and after the "
                           "launch: the kernel plus about 3 us of dispatch latency",
-                "bytes_per_launch": mk["bytes_per_launch"]}
+                "bytes_per_launch": mk["bytes_per_launch"],
+                # achieved / frac price the kernel on its ALGORITHMIC bytes; where queries repeat,
+                # part of those bytes is served by L2, so the rate of bytes that reached HBM
+                # (counter traffic over the same time) is stated beside it and is the lower one
+                "achieved_is": "algorithmic bytes per launch / kernel time",
+                "traffic_GB/s": mk.get("traffic_GB/s"), "traffic_frac": mk.get("traffic_frac")}
+    if wl.host_cold:
+        roofline["step_bound"] = ("the step as a whole is bound by the host link, not by HBM: see "
+                                  "`pcie` (this object is the HBM kernel that moves the most bytes)")
     if split or keyed:
         hot_b = sum(kbytes[k] for k in ("hot_fetch", "seg_sum", "hot_update"))
         hot_ms = sum(kernels[k]["us"] for k in ("hot_fetch", "seg_sum", "hot_update")) / 1e3
@@ -787,19 +802,28 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
                 u["frac_kernel_probe_both_ways"] = round(u_gbs / link["kernels"]["both_ways_each_GB/s"], 4)
                 f["frac_kernel_probe_gather"] = round(f_gbs / link["kernels"]["gather_GB/s"], 4)
         pcie["fetch_host_to_device"] = f
-        if reuse_rows and keyed:
+        write_only = keyed and reuse_rows and reused["no"] == 0 and reused["yes"] > 0
+        if write_only:
             pcie["update_device_to_host_only"] = u
             pcie["update_note"] = ("the cold update takes the old weights from the rows this step's "
-                                   "fetch brought in: it only writes over the link")
+                                   "fetch brought in (backward_keyed's guarded default: the optimizer "
+                                   "saw no write to the table between the two halves in any of the "
+                                   "%d backward halves of this run): it only writes over the link"
+                                   % reused["yes"])
         else:
             pcie["update_each_way_at_once"] = u
         pcie["achieved"] = round(min(f_gbs, u_gbs), 2)
         pcie["frac"] = round(min(f_gbs, u_gbs) / PCIE_PEAK_GBS, 4)
-        pcie["note"] = ("%s; %s; achieved/frac = the lower of the two" % (
+        pcie["legs"] = {"fetch_host_to_device": round(f_gbs / PCIE_PEAK_GBS, 4),
+                        ("update_device_to_host_only" if write_only else "update_each_way_at_once"):
+                            round(u_gbs / PCIE_PEAK_GBS, 4)}
+        pcie["note"] = ("%s; %s; achieved/frac = the lower of the two legs" % (
             timing_note, "the update only writes the cold weight rows (4D bytes per distinct cold row)"
-            if (reuse_rows and keyed) else
+            if write_only else
             "the update reads and writes the cold weight rows (4D bytes each way per distinct cold row)"))
         res["pcie"] = pcie
+    if keyed:
+        res["backward_halves_that_reused_the_forward_rows"] = dict(reused)
     del wl, opt
     torch.cuda.empty_cache()
     return res
@@ -1326,13 +1350,18 @@ def main():
         msg = str(err).splitlines()[0][:300] if str(err) else type(err).__name__
         if args.workload != "cfg3" or "memory" not in msg.lower():
             raise
+        if not args.allow_fallback:
+            print("bench.py: cfg3 could not be set up on this host (%s).  Nothing was measured; "
+                  "--allow-fallback measures cfg2 instead and labels the line so." % msg,
+                  file=sys.stderr)
+            sys.exit(3)
         log("cfg3 could not be set up (%s): falling back to cfg2" % msg)
         import gc
         import torch
         gc.collect()
         torch.cuda.empty_cache()
         fallback = "cfg3 could not be allocated on this host (%s); this line is cfg2" % msg
-        args.workload, args.schedule, args.reuse_rows = "cfg2", None, False
+        args.workload, args.schedule = "cfg2", None
         res = run_gpu(args, "cfg2", None)
     ms_per_step = res.pop("ms_per_step")
     n = res.pop("n")
@@ -1351,7 +1380,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": res.pop("workload") + (
-                       "; cold update reuses the rows fetched by the same step" if args.reuse_rows else ""),
+                       "; the cold update re-reads the table (--no-reuse-rows)"
+                       if (schedule in ("keyed", "pipelined") and not args.reuse_rows) else ""),
                    "combine_mode": args.mode,
                    "optimizer": ("SparseAdam lr=0.01 betas=(0.9, 0.999) eps=1e-8 (the reference's "
                                  "optimizer; the configurations name Adagrad)" if args.optimizer == "adam"
@@ -1386,20 +1416,20 @@ def main():
             "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
             "step_us": sec["step_us"], "step_frac_hbm": sec["step_frac_hbm"],
             "roofline": sec["roofline"], "kernels": sec["kernels"], "phases": sec["phases"]}}
-        if schedule == "keyed" and not args.reuse_rows:
-            log("secondary: cfg3 again with the cold update reusing the fetched rows")
-            sec = run_gpu(args, "cfg3", "keyed", with_gate=True, with_link=False, reuse_rows=True)
-            line["secondary"]["cfg3_reuse_fetched_rows"] = {
-                "what": "the headline workload and schedule, but the cold update takes the old weight "
-                        "rows from the rows the step's own fetch brought in instead of reading the "
-                        "host table a second time (bit-identical results; valid with one batch in "
-                        "flight per table; opt-in: backward_keyed(fetched_rows=...))",
+        if schedule == "keyed" and args.reuse_rows:
+            log("secondary: cfg3 again with the cold update re-reading the host table")
+            sec = run_gpu(args, "cfg3", "keyed", with_gate=True, with_link=False, reuse_rows=False)
+            line["secondary"]["cfg3_table_reread"] = {
+                "what": "the headline workload and schedule, but the cold update reads the old weight "
+                        "rows from the host table a second time (backward_keyed(fetched_rows=None), or "
+                        "an optimizer constructed with reuse_fetched_rows=False): what a table with "
+                        "writers the optimizer cannot see has to do.  Bit-identical results",
                 "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
                 "step_us": sec["step_us"], "phases": sec["phases"], "pcie": sec["pcie"],
                 "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
                             for k, v in sec["kernels"].items()},
                 "parity_gate": sec["parity_gate"]}
-        if schedule == "keyed" and not args.reuse_rows:
+        if schedule == "keyed" and args.reuse_rows:
             log("secondary: cfg3 with two batches in flight (pipelined schedule, fetched rows reused)")
             sec = run_gpu(args, "cfg3", "pipelined", with_gate=True, with_link=False, reuse_rows=True)
             line["secondary"]["cfg3_pipelined"] = {

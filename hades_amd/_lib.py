@@ -26,10 +26,11 @@ _L = c_int64
 KERNEL_NONE, KERNEL_CACHED_FETCH, KERNEL_SEG_SUM, KERNEL_ADAGRAD, KERNEL_RADIX_PASS = 0, 1, 2, 3, 4
 KERNEL_HASH_ACCUMULATE = 5
 KERNEL_ADAM = 6
-ABI_VERSION = 120      # HADES_ABI_VERSION of include/hades_hip.h
+ABI_VERSION = 130      # HADES_ABI_VERSION of include/hades_hip.h
 
 _SIGNATURES = {
     "hades_profile_kernel": [c_int, _P, _P],
+    "hades_set_host_link_blocks": [c_int, _L],
     "hades_pin": [_P, c_size_t],
     "hades_unpin": [_P],
     "hades_host_alloc": [ctypes.POINTER(c_void_p), c_size_t],
@@ -93,6 +94,7 @@ _SIGNATURES = {
                               _L, _P, c_size_t, _P],
 }
 _SIZE_QUERIES = {
+    "hades_get_host_link_blocks": [c_int],
     "hades_split_compact_workspace_bytes": [_L],
     "hades_hot_index_bytes": [_L],
     "hades_combine_workspace_bytes": [_L, _L],

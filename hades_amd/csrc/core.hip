@@ -3,6 +3,8 @@
 
 #include <stdlib.h>
 
+#include <atomic>
+#include <mutex>
 #include <string>
 
 namespace hades {
@@ -20,14 +22,47 @@ int set_error(int code, const char* fmt, ...) {
   return code;
 }
 
+// Whether a table lives in host memory decides nothing but the width of the grid that walks it,
+// and the answer for a given base pointer does not change while the allocation lives.  The
+// runtime query costs a few microseconds and a step asks it for the same handful of tables six
+// or more times, so answers are kept in a small table keyed by the pointer.  hades_host_free and
+// hades_unpin drop their pointer; an entry that outlives a foreign free can at worst pick the
+// other grid width for whatever is allocated there next.
+namespace {
+constexpr int kPtrCache = 64;
+struct PtrCacheEntry {
+  const void* ptr = nullptr;
+  bool host = false;
+};
+std::mutex g_ptr_mu;
+PtrCacheEntry g_ptr_cache[kPtrCache];
+int g_ptr_next = 0;
+}  // namespace
+
+void forget_pointer(const void* p) {
+  std::lock_guard<std::mutex> lock(g_ptr_mu);
+  for (auto& e : g_ptr_cache)
+    if (e.ptr == p) e.ptr = nullptr;
+}
+
 bool is_host_memory(const void* p) {
   if (p == nullptr) return false;
+  {
+    std::lock_guard<std::mutex> lock(g_ptr_mu);
+    for (const auto& e : g_ptr_cache)
+      if (e.ptr == p) return e.host;
+  }
   hipPointerAttribute_t attr;
+  bool host = false;
   if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
     (void)hipGetLastError();   // an ordinary pointer the runtime does not know: not ours to read
-    return false;
+  } else {
+    host = attr.type == hipMemoryTypeHost;
   }
-  return attr.type == hipMemoryTypeHost;
+  std::lock_guard<std::mutex> lock(g_ptr_mu);
+  g_ptr_cache[g_ptr_next] = PtrCacheEntry{p, host};
+  g_ptr_next = (g_ptr_next + 1) % kPtrCache;
+  return host;
 }
 
 // A kernel that reads or writes rows over the host link needs only enough loads in flight to
@@ -40,17 +75,26 @@ bool is_host_memory(const void* p) {
 // the link) saturates it from 32 blocks, and every further store in flight only queues up in front
 // of the HBM traffic of other streams (the segmented sum beside a write-only update of 128 blocks
 // took 690 us, beside one of 32 blocks 155 us, the update itself as long either way).
-// HADES_HOST_LINK_BLOCKS / _RW / _WO override the three widths for tuning.
+// HADES_HOST_LINK_BLOCKS / _RW / _WO (read once, at the first use) and
+// hades_set_host_link_blocks() override the three widths for tuning.
+namespace {
+std::atomic<int64_t> g_link_blocks[3] = {{0}, {0}, {0}};   // 0: not set yet
+}  // namespace
+
 int64_t host_link_blocks(HostLinkUse use) {
   static const char* const names[] = {"HADES_HOST_LINK_BLOCKS", "HADES_HOST_LINK_BLOCKS_RW",
                                       "HADES_HOST_LINK_BLOCKS_WO"};
   static const int64_t defaults[] = {16, 128, 32};
+  int64_t v = g_link_blocks[use].load(std::memory_order_relaxed);
+  if (v > 0) return v;
+  v = defaults[use];
   const char* e = getenv(names[use]);
   if (e != nullptr) {
-    const long v = atol(e);
-    if (v >= 1) return v;
+    const long ev = atol(e);
+    if (ev >= 1) v = ev;
   }
-  return defaults[use];
+  g_link_blocks[use].store(v, std::memory_order_relaxed);
+  return v;
 }
 
 }  // namespace hades
@@ -79,8 +123,21 @@ int hades_pin(void* host_ptr, size_t bytes) {
   return HADES_OK;
 }
 
+int hades_set_host_link_blocks(int use, int64_t blocks) {
+  HADES_REQUIRE(use >= 0 && use <= 2, "use must be 0 (copy), 1 (read and write) or 2 (write only)");
+  HADES_REQUIRE(blocks >= 0 && blocks <= 65536, "blocks must be in [0, 65536]");
+  g_link_blocks[use].store(blocks, std::memory_order_relaxed);   // 0: back to the default
+  return HADES_OK;
+}
+
+int64_t hades_get_host_link_blocks(int use) {
+  if (use < 0 || use > 2) return 0;
+  return host_link_blocks(static_cast<HostLinkUse>(use));
+}
+
 int hades_unpin(void* host_ptr) {
   HADES_REQUIRE(host_ptr != nullptr, "hades_unpin: null pointer");
+  forget_pointer(host_ptr);
   HADES_HIP_TRY(hipHostUnregister(host_ptr));
   return HADES_OK;
 }
@@ -102,6 +159,7 @@ int hades_host_alloc(void** out_ptr, size_t bytes) {
 
 int hades_host_free(void* ptr) {
   if (!ptr) return HADES_OK;
+  forget_pointer(ptr);
   HADES_HIP_TRY(hipHostFree(ptr));
   return HADES_OK;
 }

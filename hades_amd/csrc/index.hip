@@ -522,6 +522,9 @@ int hades_lookup_split(const int64_t* q, const int64_t* num_live, int64_t n,
   HADES_REQUIRE(sort_keys == nullptr || (key_bits >= 1 && key_bits <= 61 &&
                                          num_hot <= (int64_t(1) << key_bits)),
                 "key_bits must be in [1, 61] and leave room for every hot slot");
+  // entries past num_live[0] get neither a slot nor a key, and the classed combine sorts all n keys
+  HADES_REQUIRE(num_live == nullptr || sort_keys == nullptr,
+                "num_live and sort_keys cannot be combined: sort keys are written for whole batches only");
   HADES_REQUIRE(n == 0 || (q && loc), "null pointer argument");
   HADES_REQUIRE(num_hot == 0 || sorted_hot, "sorted_hot is null but num_hot > 0");
   CompactOut out{{hot_mask, nullptr, nullptr}, {hot_pos, cold_pos, nullptr}};

@@ -93,6 +93,19 @@ def profile_kernel(kernel_id, start=None, stop=None):
               ctypes.c_void_p(stop.cuda_event))
 
 
+LINK_COPY, LINK_READ_WRITE, LINK_WRITE_ONLY = 0, 1, 2
+
+
+def set_host_link_blocks(use, blocks):
+    """Width (workgroups) of the kernels whose table rows cross the host link: use = LINK_COPY
+    (gather / scatter), LINK_READ_WRITE (update that reads and writes host rows) or
+    LINK_WRITE_ONLY (update that only writes them); blocks = 0 restores the default.  Returns the
+    width that was in force.  Process-wide; for tuning and measurement."""
+    old = _lib.query("hades_get_host_link_blocks", int(use))
+    _lib.call("hades_set_host_link_blocks", int(use), int(blocks))
+    return old
+
+
 # ---- the hot set and lookup -----------------------------------------------------
 class HotSet:
     """The ascending, duplicate-free hot ids on the device together with the bucket index that

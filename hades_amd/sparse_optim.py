@@ -7,6 +7,10 @@ Mirrors the reference's python/EmbCache/sparse_optim.py for one GPU: `only_uniqu
 an EmbCache-style (hot, cold) table pair.  The cross-trainer all-to-all of the reference
 (:19-129, 267-341) is not part of this build.
 """
+import os
+import warnings
+import weakref
+
 import torch
 
 from . import EmbCacheLib, ops
@@ -62,16 +66,50 @@ def side_stream(device, k):
     create a fresh set per optimizer."""
     key = (torch.device(device).index or 0, int(k))
     if key not in _side_streams:
+        _check_hw_queues()
         _side_streams[key] = torch.cuda.Stream(device=device)
     return _side_streams[key]
+
+
+_hw_queues_checked = False
+
+
+def _check_hw_queues():
+    """The schedules here are built for HIP's default of four hardware queues per process (the
+    caller's stream and three side streams).  A process that ran them with GPU_MAX_HW_QUEUES=8
+    died with a segmentation fault when copies were first issued on the side streams; the cause
+    is not known, so a raised limit is reported instead of being used silently."""
+    global _hw_queues_checked
+    if _hw_queues_checked:
+        return
+    _hw_queues_checked = True
+    v = os.environ.get("GPU_MAX_HW_QUEUES")
+    try:
+        if v is not None and int(v) > 4:
+            warnings.warn("GPU_MAX_HW_QUEUES=%s: hades_amd's multi-stream schedules are validated with "
+                          "the default of 4 hardware queues only; a run with 8 ended in a segmentation "
+                          "fault of unknown cause.  Unset the variable." % v, RuntimeWarning, stacklevel=3)
+    except ValueError:
+        pass
 
 
 class _SparseRowOptimizer:
     """State shared by the two optimizers: weights and state as (hot, cold) pairs keyed by the
     ascending hot-ID set.  `weight_cold` is [N, D] on the device or pinned on the host."""
 
-    def __init__(self, weight_cold, hot_ids, lr, device="cuda", state_on_device=False):
+    def __init__(self, weight_cold, hot_ids, lr, device="cuda", state_on_device=False,
+                 reuse_fetched_rows=True):
         self.device = torch.device(device)
+        # backward_keyed may take the old cold weights from the rows forward_keyed fetched instead
+        # of reading the cold table a second time.  That is right only while nothing has written
+        # the table in between: every update this optimizer issues bumps `_epoch`, the forward
+        # state carries the epoch (and torch's version counters of the table and of the rows), and
+        # the backward half reuses the rows only if all of them are unchanged.  Writers this
+        # object cannot see (another optimizer or a raw kernel on the same table) either call
+        # note_table_write() or construct with reuse_fetched_rows=False.
+        self.reuse_fetched_rows = bool(reuse_fetched_rows)
+        self._epoch = 0
+        self._rows_writer = {}      # storage address -> plan of the forward half that last wrote it
         # cold optimizer state normally lives where the cold weights live; with state_on_device
         # it is kept in HBM even when the weights are a pinned host table (288 GB of HBM hold the
         # state of tables whose weights are served from the host)
@@ -114,6 +152,45 @@ class _SparseRowOptimizer:
             m = min(step, flat.numel() - i)
             flat[i:i + m].copy_(zeros[:m])
         return t
+
+    def note_table_write(self):
+        """Tells the optimizer that its tables were written by something it did not launch (a raw
+        kernel, another object sharing the tables): rows fetched before this call are no longer
+        trusted as the old weights of a later backward_keyed."""
+        self._epoch += 1
+
+    def _table_stamp(self):
+        """What must be unchanged between a forward fetch and the reuse of its rows: this
+        optimizer's own update count and torch's in-place version counter of the cold table."""
+        return (self._epoch, self.cold_w._version)
+
+    def _stamp_forward(self, plan, rows, stamp=None):
+        plan.rows = rows
+        plan.rows_version = rows._version
+        plan.table_stamp = self._table_stamp() if stamp is None else stamp
+        # a later forward half that writes into the same storage (through raw pointers: no version
+        # bump) takes the rows away from this plan
+        dead = [k for k, r in self._rows_writer.items() if r() is None]
+        for k in dead:
+            del self._rows_writer[k]
+        self._rows_writer[rows.untyped_storage().data_ptr()] = weakref.ref(plan)
+
+    def _rows_to_reuse(self, plan, fetched_rows):
+        """The rows the cold update may take its old weights from, or None (read the table).
+        fetched_rows: "auto" (the guarded default), None (never), or a tensor the caller vouches
+        for."""
+        if fetched_rows is None:
+            return None
+        if not isinstance(fetched_rows, str):
+            return fetched_rows
+        if fetched_rows != "auto":
+            raise RuntimeError("fetched_rows must be 'auto', None or a tensor")
+        rows = getattr(plan, "rows", None)
+        if (not self.reuse_fetched_rows or rows is None or getattr(plan, "first_pos", None) is None
+                or plan.table_stamp != self._table_stamp() or plan.rows_version != rows._version
+                or self._rows_writer.get(rows.untyped_storage().data_ptr(), lambda: None)() is not plan):
+            return None
+        return rows
 
     def fetch(self, ids, out=None):
         """Forward fetch of embedding rows (cached_fetch)."""
@@ -235,6 +312,11 @@ class _SparseRowOptimizer:
         split_done = torch.cuda.Event()
         split_done.record(cur)
         cold.wait_event(split_done)          # the cold stream also still orders after its own fetch
+        self._epoch += 1
+        if cold != cur:       # memory of the caller's stream, read on another one
+            for t in (uids, grad, num_unique):
+                if t is not None:
+                    t.record_stream(cold)
         with torch.cuda.stream(cold):
             self._timed(timing, "cold_update", cold,
                         lambda: self._update_class(uids, grad, cold_pos, counts[1:2], hot=False))
@@ -282,6 +364,7 @@ class _SparseRowOptimizer:
         plan = ops.combine_plan_classed(bufs["keys"][:n], self.dim, kb, workspace=bufs.get("ws", self._ws),
                                         out=(bufs["ukeys"][:n], bufs["nu"], bufs["class_split"]),
                                         first_pos=bufs["first_pos"][:n])
+        self._stamp_forward(plan, out)
         self.join()
         return out, (plan, bufs)
 
@@ -356,7 +439,7 @@ class _SparseRowOptimizer:
             planned.record(srt)
         return {"ids": ids, "out": out, "plan": plan, "bufs": bufs, "loc": loc, "hot_pos": hot_pos[:n],
                 "cold_pos": cold_pos[:n], "counts": counts, "looked_up": looked_up,
-                "gathered": gathered, "planned": planned}
+                "gathered": gathered, "planned": planned, "stamp": self._table_stamp()}
 
     def finish_prefetch(self, p, after=None, timing=None):
         """Completes a prefetched forward half on the current stream, after the backward half of
@@ -377,19 +460,34 @@ class _SparseRowOptimizer:
                         lambda: ops.fetch_listed(self.cold_w, ids, p["cold_pos"], counts[1:2], out,
                                                  only_in=prev.uids, only_in_count=prev.class_split[1:2]))
         cur.wait_event(p["planned"])
+        # The prefetched rows stand for the tables as they are now if nothing has written the
+        # cold table since the prefetch, or if the one write since then is the update of `after`,
+        # whose rows were just read again.  Anything else leaves the state without a valid stamp
+        # and the backward half reads the table.
+        epoch0, version0 = p["stamp"]
+        if after is None:
+            valid = p["stamp"] == self._table_stamp()
+        else:
+            valid = (self._epoch == epoch0 + 1 and getattr(after[0], "update_epoch", None) == self._epoch
+                     and self.cold_w._version == version0)
+        self._stamp_forward(p["plan"], out, None if valid else (None, None))
         return out, (p["plan"], p["bufs"])
 
-    def backward_keyed(self, state, grad, mode=ops.COMBINE_FAST, timing=None, fetched_rows=None,
+    def backward_keyed(self, state, grad, mode=ops.COMBINE_FAST, timing=None, fetched_rows="auto",
                        join=True):
         """Backward half: segmented sums of the cold class, whose update then starts on the cold
         stream while the hot class is summed and updated on the current stream; joins at the end.
         Returns (ukeys, sums, cnts, num_unique, class_split): the distinct rows in class order -
         cold ids ascending, then hot slots ascending with bit key_bits set.
 
-        `fetched_rows` = the rows forward_keyed returned for this batch: the cold update then takes
-        the old weights from them instead of reading the cold table a second time (half the
-        host-link traffic of the update).  The caller vouches that nothing has written the table
-        since that forward pass - true for a trainer with one batch in flight.
+        The cold update takes the old weights from the rows the forward half fetched for this
+        batch instead of reading the cold table a second time (half the host-link traffic of the
+        update) - but only while that is provably the same thing: `fetched_rows` = "auto" (the
+        default) reuses them if this optimizer has issued no update on its tables since that
+        forward half, torch's version counters of the cold table and of the rows are unchanged,
+        and the optimizer was not constructed with reuse_fetched_rows=False; otherwise the table
+        is read again.  Either way the result is the same bit for bit.  None always reads the
+        table; a tensor is taken as the rows on the caller's word.
 
         join=False returns without making the current stream wait for the cold update; the caller
         then calls finish_prefetch(...) or join() before it reads the cold table on that stream."""
@@ -397,6 +495,10 @@ class _SparseRowOptimizer:
         cold = self._split_state()
         cur = torch.cuda.current_stream()
         n = plan.n
+        fetched_rows = self._rows_to_reuse(plan, fetched_rows)
+        plan.reused_rows = fetched_rows is not None
+        self._epoch += 1
+        plan.update_epoch = self._epoch
         out = (bufs["sums"][:n], bufs["cnts"][:n])
         self._timed(timing, "cold_seg_sum", cur,
                     lambda: ops.combine_apply_class(plan, grad, 0, mode, out=out))
@@ -461,13 +563,13 @@ class SparseAdagrad(_SparseRowOptimizer):
     (torch.optim.Adagrad with lr_decay = weight_decay = initial_accumulator_value = 0)."""
 
     def __init__(self, weight_cold, hot_ids, lr=0.01, eps=1e-10, device="cuda",
-                 state_on_device=False, cold_state=None):
+                 state_on_device=False, cold_state=None, reuse_fetched_rows=True):
         """`cold_state` brings the cold Adagrad state instead of a new zero tensor; together with
         a row-strided `weight_cold` it allows one host table [N, 2, D] that holds the weight row
         and the state row of an id next to each other (weight_cold = t[:, 0], cold_state =
         t[:, 1]): one burst per cold row and direction over the host link.  Row-strided cold
         tables are served by the split schedule (fetch_split / update_split / step_split) only."""
-        super().__init__(weight_cold, hot_ids, lr, device, state_on_device)
+        super().__init__(weight_cold, hot_ids, lr, device, state_on_device, reuse_fetched_rows)
         self.eps = eps
         if cold_state is not None:
             if tuple(cold_state.shape) != tuple(weight_cold.shape) or cold_state.dtype != torch.float32:
@@ -486,6 +588,7 @@ class SparseAdagrad(_SparseRowOptimizer):
         ops.adagrad_update_class_(plan, sums, which, w, s, self.lr, self.eps, fetched_rows=fetched_rows)
 
     def update(self, uids, grad, num_unique=None):
+        self._epoch += 1
         ops.adagrad_update_(uids, grad, self.hot_w, self.hot_s, self.cold_w, self.cold_s,
                             self.hot_set, self.lr, self.eps, num_unique)
 
@@ -494,8 +597,8 @@ class SparseAdam(_SparseRowOptimizer):
     """The reference's SparseAdam.update (python/EmbCache/sparse_optim.py:590-685) as one kernel."""
 
     def __init__(self, weight_cold, hot_ids, lr=0.01, betas=(0.9, 0.999), eps=1e-8, device="cuda",
-                 state_on_device=False):
-        super().__init__(weight_cold, hot_ids, lr, device, state_on_device)
+                 state_on_device=False, reuse_fetched_rows=True):
+        super().__init__(weight_cold, hot_ids, lr, device, state_on_device, reuse_fetched_rows)
         self.betas, self.eps = betas, eps
         n, h = self.num_rows, self.hot_ids.numel()
         self.cold_step = self._new_state_like(weight_cold, (n,))
@@ -518,6 +621,7 @@ class SparseAdam(_SparseRowOptimizer):
                                self.betas[0], self.betas[1], self.eps, fetched_rows=fetched_rows)
 
     def update(self, uids, grad, num_unique=None):
+        self._epoch += 1
         ops.adam_update_(uids, grad, (self.hot_w, self.hot_step, self.hot_m, self.hot_v),
                          (self.cold_w, self.cold_step, self.cold_m, self.cold_v), self.hot_set,
                          self.lr, self.betas[0], self.betas[1], self.eps, num_unique)

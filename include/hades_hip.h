@@ -55,7 +55,7 @@ extern "C" {
 const char* hades_last_error(void);
 /* Version of this interface; raised whenever a signature changes, so that a binding can refuse a
  * library built from other sources. */
-#define HADES_ABI_VERSION 120
+#define HADES_ABI_VERSION 130
 int hades_version(void);
 
 /* Kernel timing hook (no counterpart in the reference, whose scripts time whole calls from the
@@ -71,6 +71,15 @@ int hades_version(void);
 #define HADES_KERNEL_ADAM 6         /* hades_adam_update */
 #define HADES_KERNEL_LAST 6
 int hades_profile_kernel(int kernel_id, void* start_event, void* stop_event);
+
+/* Width, in workgroups, of the kernels whose table rows cross the host link (no counterpart in the
+ * reference, whose row kernels are launched one block per 32 rows whatever the memory,
+ * src/cuda/uva_fetch.cu:86-95).  use: 0 a row copy one way (gather from / scatter to a host table),
+ * 1 an update that reads and writes host rows, 2 an update that only writes them.  blocks = 0
+ * restores the default (16 / 128 / 32, or the HADES_HOST_LINK_BLOCKS, _RW, _WO environment
+ * variables, which are read once, at first use).  Process-wide; meant for tuning and measurement. */
+int hades_set_host_link_blocks(int use, int64_t blocks);
+int64_t hades_get_host_link_blocks(int use);
 
 /* ------------------------------------------------------------------------- */
 /* Group 1: one entry point per function bound in src/pybind.cc:46-70          */
@@ -201,7 +210,8 @@ int hades_split_compact(const int64_t* loc, int64_t n, uint8_t* hot_mask, int64_
  * per class): the two position lists then drive hades_fetch_listed / hades_adagrad_update_listed
  * over the hot tables in HBM and over the cold tables on the host, on separate streams.
  * num_live (int64[1] on the device, may be NULL) limits the batch to its first num_live[0] entries
- * (the padded output of hades_combine): later entries are in neither list and get no slot.
+ * (the padded output of hades_combine): later entries are in neither list and get no slot (and
+ * no sort key: num_live together with sort_keys is refused with HADES_ERR_ARG).
  * sort_keys (int64[n], may be NULL) receives a class-ordered sort key per query, for
  * hades_combine_plan_classed:  cold: the id itself;  hot: (1 << key_bits) | slot.  key_bits must
  * cover the table's ids (ids < 2^key_bits).  Sorted by this key a batch has its cold ids first, in

@@ -102,6 +102,14 @@ def test_argument_errors_of_the_split_schedule_entry_points():
     assert b"key_bits" in lib.hades_last_error()
     assert lib.hades_lookup_split(one, null, 10, one, 100, null, one, null, one, one, one, null, 0,
                                   one, 16, null) == 3                                          # workspace
+    assert lib.hades_lookup_split(one, one, 10, one, 100, null, one, null, one, one, one, one, 20,
+                                  one, 1 << 20, null) == 1                  # a live count and sort keys
+    assert b"cannot be combined" in lib.hades_last_error()
+    # host-link grid widths: set, read back, restore the default
+    assert lib.hades_set_host_link_blocks(3, 8) == 1 and lib.hades_set_host_link_blocks(0, -1) == 1
+    d = _lib.query("hades_get_host_link_blocks", 0)
+    assert lib.hades_set_host_link_blocks(0, 48) == 0 and _lib.query("hades_get_host_link_blocks", 0) == 48
+    assert lib.hades_set_host_link_blocks(0, 0) == 0 and _lib.query("hades_get_host_link_blocks", 0) == d
     # classed combine
     assert lib.hades_combine_plan_classed(one, 10, 8, 1 << 20, 1 << 19, one, one, null, null, one, 1 << 20, null) == 1
     assert lib.hades_combine_plan_classed(one, 10, 8, 1 << 20, 1 << 21, one, one, one, null, one, 1 << 20, null) == 1

@@ -1341,11 +1341,11 @@ def test_library_pinned_allocation_through_the_c_abi(lib):
     assert L.hades_host_alloc(None, 16) == 1              # null out pointer: an error code, no crash
 
 
-def test_host_alloc_tensor_and_cudapin_on_pageable_memory(lib):
+def test_host_alloc_tensor_and_pageable_memory_is_refused(lib):
     """EmbCacheLib.host_alloc gives a host tensor the kernels accept as a cold table; cudaPin on a
-    tensor that is already pinned is a no-op; on pageable memory it either registers the memory
-    (then a kernel can read it) or raises RuntimeError where the platform refuses hipHostRegister:
-    it never ends the process (the reference's CUDA_CALL does, src/utils.h:12-24)."""
+    tensor that is already pinned is a no-op; a pageable tensor is refused by the shim with a
+    RuntimeError before any kernel sees it.  (Registering pageable memory is exercised on the CPU
+    side only, in tests/test_shm.py.)"""
     E, ops = lib
     rng = np.random.default_rng(1)
     t = E.host_alloc((3000, 64), torch.float32)
@@ -1362,15 +1362,6 @@ def test_host_alloc_tensor_and_cudapin_on_pageable_memory(lib):
     pageable = torch.from_numpy(rng.standard_normal((1000, 16)).astype(np.float32))
     with pytest.raises(RuntimeError, match="pageable"):
         E.cudaFetch2(pageable, idx % 1000, torch.empty((500, 16), device="cuda"))
-    try:
-        E.cudaPin(pageable)
-    except RuntimeError as err:
-        assert "hipHostRegister" in str(err) or "hades_pin" in str(err)
-    else:
-        o2 = torch.empty((500, 16), device="cuda")
-        E.cudaFetch2(pageable, idx % 1000, o2)
-        assert torch.equal(o2.cpu(), pageable[(idx % 1000).cpu()])
-        E.cudaUnpin(pageable)
     # the process and the HIP runtime are still in working order
     assert torch.equal(ops.lookup(idx, torch.arange(3000, device="cuda")), idx)
 
@@ -1476,7 +1467,8 @@ def test_keyed_backward_with_the_forward_rows(lib, host_cold):
     t_q, t_g = dev(q), dev(grad)
     for it in range(2):
         rows, st = plain.forward_keyed(t_q)
-        plain.backward_keyed(st, t_g, mode=ops.COMBINE_EXACT)
+        plain.backward_keyed(st, t_g, mode=ops.COMBINE_EXACT, fetched_rows=None)
+        assert not st[0].reused_rows
         rows2, st2 = reuse.forward_keyed(t_q)
         assert torch.equal(rows, rows2)
         reuse.backward_keyed(st2, t_g, mode=ops.COMBINE_EXACT, fetched_rows=rows2)
@@ -1495,6 +1487,111 @@ def test_keyed_backward_with_the_forward_rows(lib, host_cold):
     assert np.array_equal(altered.cold_w.cpu().numpy(), cw) and np.array_equal(altered.cold_s.cpu().numpy(), cs)
     assert np.array_equal(altered.hot_w.cpu().numpy(), hw) and np.array_equal(altered.hot_s.cpu().numpy(), hs)
     assert not np.array_equal(cw, plain.cold_w.cpu().numpy())
+
+
+@pytest.mark.parametrize("host_cold", [False, True])
+@pytest.mark.parametrize("kind", ["adagrad", "adam"])
+def test_keyed_backward_reuses_the_forward_rows_only_while_the_table_is_unwritten(lib, host_cold, kind):
+    """The guarded default of backward_keyed.  With nothing in between, the cold update takes its
+    old weights from the forward rows and leaves the tables of the re-reading path, bit for bit.
+    A second update of the same rows between the forward and the backward half, an in-place torch
+    write to the cold table, an in-place change of the rows, another forward half into the same
+    rows buffer, note_table_write() and reuse_fetched_rows=False each make it read the table
+    again - and the result stays that of the sequence as issued (the oracle applies the steps in
+    that order)."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad, SparseAdam
+    rng = np.random.default_rng(777 + host_cold)
+    N, D, H, n = 20_000, 64, 2000, 30_000
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, 0.6)
+    q2 = q.copy()
+    rng.shuffle(q2)
+    q2[: n // 2] = rng.integers(0, N, n // 2)          # shares many cold ids with q
+    g1 = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+    g2 = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+    t_q, t_q2, t_g1, t_g2 = dev(q), dev(q2), dev(g1), dev(g2)
+
+    def make(**kw):
+        t = torch.from_numpy(cold.copy())
+        t = t.pin_memory() if host_cold else t.cuda()
+        if kind == "adam":
+            return SparseAdam(t, torch.from_numpy(hot_ids), **kw)
+        return SparseAdagrad(t, torch.from_numpy(hot_ids), **kw)
+
+    def tables(o):
+        ts = ((o.cold_w, o.cold_s, o.hot_w, o.hot_s) if kind == "adagrad" else
+              (o.cold_w, o.cold_step, o.cold_m, o.cold_v, o.hot_w, o.hot_step, o.hot_m, o.hot_v))
+        torch.cuda.synchronize()
+        return [t.cpu().clone() for t in ts]
+
+    def same(a, b):
+        return all(torch.equal(x, y) for x, y in zip(tables(a), tables(b)))
+
+    guarded, reread, off = make(), make(), make(reuse_fetched_rows=False)
+    # 1. nothing in between: reuse, and the tables of the re-reading path
+    for it in range(2):
+        _, st = guarded.forward_keyed(t_q)
+        guarded.backward_keyed(st, t_g1, mode=ops.COMBINE_EXACT)
+        assert st[0].reused_rows == bool(n)
+        _, st_r = reread.forward_keyed(t_q)
+        reread.backward_keyed(st_r, t_g1, mode=ops.COMBINE_EXACT, fetched_rows=None)
+        assert not st_r[0].reused_rows
+        _, st_o = off.forward_keyed(t_q)
+        off.backward_keyed(st_o, t_g1, mode=ops.COMBINE_EXACT)
+        assert not st_o[0].reused_rows
+    assert same(guarded, reread) and same(off, reread)
+
+    # 2. a second update of overlapping rows between the two halves: fall back, stay exact
+    for o, kw in ((guarded, {}), (reread, {"fetched_rows": None})):
+        _, st = o.forward_keyed(t_q)
+        u2, s2, _ = ops.combine(t_q2, t_g2, mode=ops.COMBINE_EXACT)
+        o.update(u2, s2)                                      # writes cold rows q also names
+        o.backward_keyed(st, t_g1, mode=ops.COMBINE_EXACT, **kw)
+        assert not st[0].reused_rows
+    assert same(guarded, reread)
+    if kind == "adagrad":                                     # and that is what the oracle says
+        cw, cs = cold.copy(), np.zeros_like(cold)
+        hw, hs = cold[hot_ids].copy(), np.zeros((H, D), np.float32)
+        kb = ops.key_bits_for(N)
+        for _ in range(2):
+            O.keyed_step(cw, cs, hw, hs, hot_ids, q, g1, 0.01, 1e-10, kb)
+        wu, ws, _ = O.combine_sequential(q2, g2)
+        O.sparse_adagrad_step(cw, cs, hw, hs, hot_ids, wu, ws, 0.01, 1e-10)
+        O.keyed_step(cw, cs, hw, hs, hot_ids, q, g1, 0.01, 1e-10, kb)
+        got = tables(guarded)
+        for a, b in zip(got, (cw, cs, hw, hs)):
+            assert np.array_equal(a.numpy(), b)
+
+    # 3. the other ways the rows stop standing for the table
+    def backward_after(spoil):
+        rows, st = guarded.forward_keyed(t_q)
+        rows_r, st_r = reread.forward_keyed(t_q)
+        spoil(guarded, rows)
+        spoil(reread, rows_r)
+        guarded.backward_keyed(st, t_g1, mode=ops.COMBINE_EXACT)
+        reread.backward_keyed(st_r, t_g1, mode=ops.COMBINE_EXACT, fetched_rows=None)
+        return st[0].reused_rows
+
+    some = torch.from_numpy(np.unique(q)[:50])
+
+    def table_write(o, rows):
+        torch.cuda.synchronize()
+        idx = some if not o.cold_w.is_cuda else some.cuda()
+        o.cold_w[idx] += 0.5                                   # torch in place: the version counter moves
+
+    assert not backward_after(table_write)
+    assert same(guarded, reread)
+    assert not backward_after(lambda o, rows: rows.mul_(2.0))  # the rows no longer hold the table's values
+    assert same(guarded, reread)
+    assert not backward_after(lambda o, rows: o.note_table_write())
+    assert same(guarded, reread)
+
+    def second_forward_into_the_same_buffer(o, rows):
+        o.forward_keyed(t_q2, out=rows, slot=1)                # raw-pointer write: no version bump
+    assert not backward_after(second_forward_into_the_same_buffer)
+    assert same(guarded, reread)
+    assert backward_after(lambda o, rows: None)                # and with nothing in between it reuses again
+    assert same(guarded, reread)
 
 
 def test_lookup_split_beyond_the_in_kernel_tile_sum(lib):
