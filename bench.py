@@ -7,6 +7,7 @@
     python bench.py --workload cfg4 --flush-rule staleness    the cache server's own per-row rule
     python bench.py --workload neighbours    pre-exchange bucketing, index cache, cold-data cache
     python bench.py --workload random-rows   what distinct random 512-byte rows of a 2 GB table cost
+    python bench.py --workload host-link     what the host link gives kernels: rows, grid width, burst, direction
 
 One step = lookup + cached_fetch of the query rows, combine of the per-query gradients, and the
 sparse Adagrad update of every distinct row, on one batch of synthetic Zipf ids that is already
@@ -57,7 +58,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours", "random-rows"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "neighbours", "random-rows", "host-link"])
     ap.add_argument("--mode", default="fast", choices=["fast", "exact"])
     ap.add_argument("--optimizer", default="adagrad", choices=["adagrad", "adam"],
                     help="row update of the step: sparse Adagrad (the configurations' optimizer) or "
@@ -77,6 +78,12 @@ def parse_args():
                          "from the host table again.  By default it takes them from the rows the "
                          "step's own fetch brought in whenever the optimizer can tell that nothing "
                          "has written the table in between (backward_keyed's guarded default)")
+    ap.add_argument("--cold-state", default="hbm", choices=["hbm", "host"],
+                    help="cfg3 with Adagrad: where the cold optimizer state lives.  hbm (default): "
+                         "the full 111 M-row table, cold weights in pinned host memory, cold state "
+                         "in HBM.  host: the contract layout - weights and state both in pinned host "
+                         "memory, side by side in one [N, 2, D] table - on a table cut to half the "
+                         "rows, which is what one page-locked allocation of this box holds")
     ap.add_argument("--allow-fallback", action="store_true",
                     help="if the host refuses cfg3's page-locked table, measure cfg2 instead and say "
                          "so in config.fallback (without this flag such a run exits non-zero)")
@@ -120,7 +127,7 @@ class Workload:
     """Tables, hot set and pre-generated batches of one configuration, resident on the device
     (cold table in pinned host memory for cfg3)."""
 
-    def __init__(self, name, nbatches, device, optimizer="adagrad"):
+    def __init__(self, name, nbatches, device, optimizer="adagrad", state_on_host=False):
         import torch
         from hades_amd import synth
         from hades_amd.sparse_optim import SparseAdagrad, SparseAdam
@@ -128,19 +135,35 @@ class Workload:
         cfg = synth.CONFIGS[name]
         self.name, self.cfg = name, cfg
         N, D, H = cfg["num_rows"], cfg["dim"], cfg["num_hot"]
+        # state_on_host (cfg3, Adagrad): the contract layout - cold weights AND cold optimizer
+        # state in pinned host memory - on a table cut to half the rows, so that one page-locked
+        # allocation of the size the box grants holds both, side by side: [N/2, 2, D], the weight
+        # row and the state row of an id in one 1 KB stretch.  Batch, skew and hot fraction stay.
+        self.state_on_host = bool(state_on_host) and name == "cfg3" and optimizer == "adagrad"
+        if self.state_on_host:
+            N, H = N // 2, H // 2
         self.N, self.D, self.H = N, D, H
         self.trainers = cfg.get("trainers", 1)
         self.n = cfg["batch"] * self.trainers
         self.host_cold = name == "cfg3"
         seed = 1234 + int(name[3:])
         log("allocating the %d x %d table (%.1f GB, %s)" %
-            (N, D, N * D * 4 / 1e9, "pinned host" if self.host_cold else "HBM"))
-        if self.host_cold:
+            (N, D, N * D * 4 * (2 if self.state_on_host else 1) / 1e9,
+             "pinned host, weight and state rows interleaved" if self.state_on_host
+             else "pinned host" if self.host_cold else "HBM"))
+        both = None
+        if self.state_on_host:
+            both = torch.empty((N, 2, D), dtype=torch.float32, pin_memory=True)
+            table = both[:, 0]
+        elif self.host_cold:
             table = torch.empty((N, D), dtype=torch.float32, pin_memory=True)
         else:
             table = torch.empty((N, D), dtype=torch.float32, device=device)
         log("filling it")
-        synth.fill_normal_(table, 0.01, seed, progress=log if N > 50_000_000 else None)
+        if both is not None:
+            synth.fill_interleaved_(both, 0.01, seed, progress=log)
+        else:
+            synth.fill_normal_(table, 0.01, seed, progress=log if N > 50_000_000 else None)
         hot_ids = synth.hot_ids(N, H, device) if H else torch.empty(0, dtype=torch.int64, device=device)
         log("hot copies and optimizer state")
         # cfg3: the cold weights are the pinned host table; the cold Adagrad state stays in HBM.
@@ -150,6 +173,9 @@ class Workload:
         if optimizer == "adam":      # its cold step / mem / power tables stay in HBM likewise
             self.opt = SparseAdam(table, hot_ids, lr=0.01, betas=(0.9, 0.999), eps=1e-8, device=device,
                                   state_on_device=self.host_cold)
+        elif both is not None:
+            self.opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=device,
+                                     cold_state=both[:, 1])
         else:
             self.opt = SparseAdagrad(table, hot_ids, lr=0.01, eps=1e-10, device=device,
                                      state_on_device=self.host_cold)
@@ -172,6 +198,10 @@ class Workload:
     def describe(self):
         return ("%s: %d x %d fp32 table (%s), hot %d rows in HBM, %d ids/step zipf s=%.2f%s" %
                 (self.name, self.N, self.D,
+                 "cold weights and cold Adagrad state both in pinned host memory, read and written "
+                 "zero-copy, the two rows of an id side by side in one [N, 2, D] table; deviation: "
+                 "the table is cut to half of cfg3's rows so that the one page-locked allocation the "
+                 "box grants holds both" if self.state_on_host else
                  "cold weights in pinned host memory read and written zero-copy; deviation: cold "
                  "optimizer state in HBM, the box refuses the 113.7 GB page-locked allocation that "
                  "would hold weights and state" if self.host_cold
@@ -357,12 +387,13 @@ def parity_gate(wl, step_fn, rows=20_000):
             "against": "torch device ops (searchsorted, indexing, unique + float64 index_add_, %s)" % form}
 
 
-def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows=True):
+def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows=True,
+            state_on_host=False):
     import torch
     from hades_amd import ops
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    wl = Workload(workload, args.batches, dev, args.optimizer)
+    wl = Workload(workload, args.batches, dev, args.optimizer, state_on_host=state_on_host)
     opt = wl.opt
     mode = ops.COMBINE_FAST if args.mode == "fast" else ops.COMBINE_EXACT
     nb = len(wl.ids)
@@ -778,21 +809,32 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
            "unique_per_step": round(U, 1), "unique_hot_per_step": round(U_hot, 1),
            "hot_hit": round(n_hot / n, 4), "parity_gate": gate}
     if wl.host_cold:
-        def link_entry(rows, ms):
-            gbs = rows * 4 * D / (ms * 1e-3) / 1e9
-            e = {"MB": round(rows * 4 * D / 1e6, 2), "GB/s": round(gbs, 2),
+        def link_entry(rows, ms, read_rows=1, write_rows=0):
+            """rows x (read_rows to the device, write_rows to the host) table rows of 4D bytes in
+            ms; GB/s and fraction of nominal are those of the busier direction"""
+            rd, wr = rows * read_rows * 4 * D, rows * write_rows * 4 * D
+            gbs = max(rd, wr) / (ms * 1e-3) / 1e9
+            e = {"MB": round(max(rd, wr) / 1e6, 2), "GB/s": round(gbs, 2),
                  "frac_nominal": round(gbs / PCIE_PEAK_GBS, 4)}
+            if read_rows != write_rows and min(rd, wr) > 0:
+                e["MB_to_device"], e["MB_to_host"] = round(rd / 1e6, 2), round(wr / 1e6, 2)
+                e["GB/s_to_device"] = round(rd / (ms * 1e-3) / 1e9, 2)
+                e["GB/s_to_host"] = round(wr / (ms * 1e-3) / 1e9, 2)
             return e, gbs
         pcie = {"bound": "pcie", "peak": PCIE_PEAK_GBS, "unit": "GB/s per direction",
                 "cold_query_rows": round(n_cold, 1), "cold_unique_rows": round(U_cold, 1),
                 "memcpy": link}
+        write_only = keyed and reuse_rows and reused["no"] == 0 and reused["yes"] > 0
+        # rows of 4D bytes per distinct cold row that the update reads / writes over the link
+        soh = wl.state_on_host
+        u_rd, u_wr = (1 if soh else 0) + (0 if write_only else 1), (2 if soh else 1)
         if split or keyed:
             f, f_gbs = link_entry(n_cold, kernels["cold_fetch"]["us"] / 1e3)
-            u, u_gbs = link_entry(U_cold, kernels["cold_update"]["us"] / 1e3)
+            u, u_gbs = link_entry(U_cold, kernels["cold_update"]["us"] / 1e3, u_rd, u_wr)
             timing_note = "cold-class kernels bracketed by HIP events on the cold stream"
         else:
             f, f_gbs = link_entry(n_cold, kernels["fetch"]["us"] / 1e3)
-            u, u_gbs = link_entry(U_cold, kernels["update"]["us"] / 1e3)
+            u, u_gbs = link_entry(U_cold, kernels["update"]["us"] / 1e3, u_rd, u_wr)
             timing_note = "hot and cold rows share the kernels: kernel time of the whole fetch / update"
         if link:
             f["frac_memcpy_h2d"] = round(f_gbs / link["h2d_GB/s"], 4)
@@ -802,8 +844,14 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
                 u["frac_kernel_probe_both_ways"] = round(u_gbs / link["kernels"]["both_ways_each_GB/s"], 4)
                 f["frac_kernel_probe_gather"] = round(f_gbs / link["kernels"]["gather_GB/s"], 4)
         pcie["fetch_host_to_device"] = f
-        write_only = keyed and reuse_rows and reused["no"] == 0 and reused["yes"] > 0
-        if write_only:
+        if soh:
+            pcie["update_state_on_host"] = u
+            pcie["update_note"] = (
+                "weights and Adagrad state of the cold rows are both in host memory, side by side: per "
+                "distinct cold row the update reads %d B (%s) and writes %d B (new weight and state, "
+                "one stretch) over the link" % (u_rd * 4 * D, "the state; the old weight comes from "
+                "the rows this step fetched" if write_only else "weight and state", u_wr * 4 * D))
+        elif write_only:
             pcie["update_device_to_host_only"] = u
             pcie["update_note"] = ("the cold update takes the old weights from the rows this step's "
                                    "fetch brought in (backward_keyed's guarded default: the optimizer "
@@ -815,10 +863,12 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         pcie["achieved"] = round(min(f_gbs, u_gbs), 2)
         pcie["frac"] = round(min(f_gbs, u_gbs) / PCIE_PEAK_GBS, 4)
         pcie["legs"] = {"fetch_host_to_device": round(f_gbs / PCIE_PEAK_GBS, 4),
-                        ("update_device_to_host_only" if write_only else "update_each_way_at_once"):
+                        ("update_state_on_host" if soh else
+                         "update_device_to_host_only" if write_only else "update_each_way_at_once"):
                             round(u_gbs / PCIE_PEAK_GBS, 4)}
         pcie["note"] = ("%s; %s; achieved/frac = the lower of the two legs" % (
-            timing_note, "the update only writes the cold weight rows (4D bytes per distinct cold row)"
+            timing_note, "the update's rate is that of its busier direction" if soh else
+            "the update only writes the cold weight rows (4D bytes per distinct cold row)"
             if write_only else
             "the update reads and writes the cold weight rows (4D bytes each way per distinct cold row)"))
         res["pcie"] = pcie
@@ -1276,6 +1326,125 @@ def run_random_rows(args):
                       "operators": res}))
 
 
+def run_host_link(args):
+    """What the host link gives kernels on this box: random distinct rows of a 56.8 GB page-locked
+    table moved by the library's own listed kernels, swept over rows per launch, grid width and
+    burst length, one way and both ways at once.  Columns (GB/s of the busier direction):
+      gather          host -> HBM (hades_fetch_listed)
+      scatter         HBM -> host (hades_set_listed)
+      gather||scatter both at once, two kernels on two streams
+      update rw       hades_adagrad_update_listed, state in HBM: reads and writes the weight row
+      update wo       hades_adagrad_update_class with the old rows at hand: only writes it
+      pair rw         weight and state row of an id side by side in the host table ([N, 2, D],
+                      1 KB per id): reads both, writes both
+      pair r1w2       the same with the old weight rows at hand: reads the state, writes both
+    Burst 512 B = rows of 128 floats; 1 KB = the same memory viewed as rows of 256 floats.
+    Prints one JSON line; the table goes to stderr."""
+    import types
+    import torch
+    from hades_amd import ops, synth
+    from hades_amd.sparse_optim import side_stream
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    N, D = synth.CONFIGS["cfg3"]["num_rows"], 128
+    log("allocating the %d x %d pinned host table (%.1f GB) and as much state in HBM" % (N, D, N * D * 4 / 1e9))
+    table = torch.empty((N, D), dtype=torch.float32, pin_memory=True)
+    synth.fill_normal_(table, 0.01, 77, progress=log)
+    state = torch.zeros((N, D), dtype=torch.float32, device=dev)
+    wide = table.view(N // 2, 2 * D)              # 1 KB rows
+    pair = table.view(N // 2, 2, D)               # [ids, (weight, state), D]
+    s1, s2 = side_stream(dev, 0), side_stream(dev, 1)
+    row_counts = [76_000, 300_000, 1_200_000, 2_300_000]
+    widths = [16, 32, 64, 128, 256]
+    gen = torch.Generator().manual_seed(5)
+    results = []
+    reps = 3
+
+    def timed(fns):
+        best = None
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for f in fns:
+                f()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return best
+
+    def case(R, tab_rows):
+        ids = torch.randperm(tab_rows, generator=gen)[:R].to(dev).sort().values
+        pos = torch.arange(R, dtype=torch.int64, device=dev)
+        cnt = torch.tensor([R], dtype=torch.int64, device=dev)
+        plan = types.SimpleNamespace(
+            uids=ids, num_unique=cnt, n=R, key_bits=40,
+            class_split=torch.tensor([R, R], dtype=torch.int64, device=dev),
+            first_pos=torch.arange(R, dtype=torch.int32, device=dev))
+        return ids, pos, cnt, plan
+
+    for R in row_counts:
+        ids5, pos, cnt, plan5 = case(R, N)
+        ids1, _, _, plan1 = case(R, N // 2)
+        buf5 = torch.empty((R, D), dtype=torch.float32, device=dev)
+        src5 = torch.empty((R, D), dtype=torch.float32, device=dev)
+        buf1 = torch.empty((R, 2 * D), dtype=torch.float32, device=dev)
+        src1 = torch.empty((R, 2 * D), dtype=torch.float32, device=dev)
+        grad = torch.randn((R, D), device=dev) * 1e-3
+        ops.fetch_listed(table, ids5, pos, cnt, src5)       # the scatters write back what is there
+        ops.fetch_listed(wide, ids1, pos, cnt, src1)
+        old_pair = torch.empty((R, D), dtype=torch.float32, device=dev)
+        ops.fetch_listed(pair[:, 0], ids1, pos, cnt, old_pair)
+        torch.cuda.synchronize()
+
+        def on(stream, fn):
+            def run():
+                with torch.cuda.stream(stream):
+                    fn()
+            return run
+
+        pats = {
+            ("gather", 512): [on(s1, lambda: ops.fetch_listed(table, ids5, pos, cnt, buf5))],
+            ("scatter", 512): [on(s2, lambda: ops.set_listed(src5, table, ids5, pos, cnt))],
+            ("gather", 1024): [on(s1, lambda: ops.fetch_listed(wide, ids1, pos, cnt, buf1))],
+            ("scatter", 1024): [on(s2, lambda: ops.set_listed(src1, wide, ids1, pos, cnt))],
+            ("update rw", 512): [on(s1, lambda: ops.adagrad_update_listed_(ids5, grad, pos, cnt, table, state, 0.01, 1e-10))],
+            ("update wo", 512): [on(s1, lambda: ops.adagrad_update_class_(plan5, grad, 0, table, state, 0.01, 1e-10,
+                                                                       fetched_rows=src5))],
+            ("pair rw", 1024): [on(s1, lambda: ops.adagrad_update_listed_(ids1, grad, pos, cnt, pair[:, 0], pair[:, 1],
+                                                                       0.01, 1e-10))],
+            ("pair r1w2", 1024): [on(s1, lambda: ops.adagrad_update_class_(plan1, grad, 0, pair[:, 0], pair[:, 1], 0.01,
+                                                                        1e-10, fetched_rows=old_pair))],
+        }
+        pats[("gather||scatter", 512)] = pats[("gather", 512)] + pats[("scatter", 512)]
+        pats[("gather||scatter", 1024)] = pats[("gather", 1024)] + pats[("scatter", 1024)]
+        for B in widths:
+            for use in (ops.LINK_COPY, ops.LINK_READ_WRITE, ops.LINK_WRITE_ONLY):
+                ops.set_host_link_blocks(use, B)
+            for burst in (512, 1024):
+                row = {"rows": R, "burst_B": burst, "blocks": B}
+                for (name, b), fns in pats.items():
+                    if b == burst:
+                        # bytes of the busier direction: one burst per row
+                        row[name] = round(R * burst / timed(fns) / 1e9, 2)
+                results.append(row)
+                log(json.dumps(row))
+        del buf5, src5, buf1, src1, grad, old_pair
+    for use in (ops.LINK_COPY, ops.LINK_READ_WRITE, ops.LINK_WRITE_ONLY):
+        ops.set_host_link_blocks(use, 0)
+    cols = ["gather", "scatter", "gather||scatter", "update rw", "update wo", "pair rw", "pair r1w2"]
+    print("%9s %6s %6s " % ("rows", "burst", "blocks") + " ".join("%16s" % c for c in cols), file=sys.stderr)
+    for r in results:
+        print("%9d %6d %6d " % (r["rows"], r["burst_B"], r["blocks"]) +
+              " ".join("%16s" % ("%.2f" % r[c] if c in r else "-") for c in cols), file=sys.stderr)
+    print(json.dumps({"metric": "host-link GB/s of the busier direction, random distinct rows of a pinned host table",
+                      "unit": "GB/s", "n_gpus": 1, "dtype": "f32", "data": "synthetic",
+                      "peak_nominal_per_direction": PCIE_PEAK_GBS,
+                      "config": {"workload": "%d x %d fp32 page-locked table (%.1f GB); wall clock around one "
+                                             "launch (or one pair of launches), best of %d" %
+                                             (N, D, N * D * 4 / 1e9, reps)},
+                      "rows": results}))
+
+
 def run_cpu_baseline(wl_name, seconds):
     """The same step with the CPU oracle (torch CPU ops, all host threads), on a bounded sample:
     the benchmark's own batches at full table size when that fits the host, repeated for about
@@ -1333,6 +1502,9 @@ def main():
     if args.workload == "random-rows":
         run_random_rows(args)
         return
+    if args.workload == "host-link":
+        run_host_link(args)
+        return
     if args.optimizer != "adagrad":
         if args.workload == "cfg1":
             print("cfg1 is the CPU reference case: it runs with the configurations' Adagrad only",
@@ -1343,7 +1515,8 @@ def main():
         args.no_cpu_baseline = True
     fallback = None
     try:
-        res = run_gpu(args, args.workload, args.schedule, reuse_rows=args.reuse_rows)
+        res = run_gpu(args, args.workload, args.schedule, reuse_rows=args.reuse_rows,
+                      state_on_host=args.cold_state == "host")
     except (RuntimeError, MemoryError) as err:
         # a host that refuses the 56.8 GB page-locked table (or lacks the HBM): say so and measure
         # the all-HBM configuration instead of printing nothing
@@ -1429,6 +1602,27 @@ def main():
                 "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
                             for k, v in sec["kernels"].items()},
                 "parity_gate": sec["parity_gate"]}
+        if schedule == "keyed" and args.reuse_rows and args.cold_state == "hbm":
+            log("secondary: cfg3's batch on a half-size table with the cold Adagrad state in host memory")
+            try:
+                sec = run_gpu(args, "cfg3", "keyed", with_gate=True, with_link=False, reuse_rows=True,
+                              state_on_host=True)
+                line["secondary"]["cfg3_cold_state_in_host_memory"] = {
+                    "what": "the contract layout of the cold class: weights AND Adagrad state of the cold "
+                            "rows in pinned host memory, the two rows of an id side by side ([N, 2, D], "
+                            "1 KB per id), on a table cut to 55.5 M rows with 5.55 M hot so that the one "
+                            "page-locked allocation this box grants (56.8 GB) holds both; cfg3's batch "
+                            "size, skew and 10 % hot fraction",
+                    "workload": sec["workload"],
+                    "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
+                    "step_us": sec["step_us"], "phases": sec["phases"], "pcie": sec["pcie"],
+                    "hot_hit": sec["hot_hit"], "unique_per_step": sec["unique_per_step"],
+                    "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
+                                for k, v in sec["kernels"].items()},
+                    "parity_gate": sec["parity_gate"]}
+            except (RuntimeError, MemoryError) as err:
+                line["secondary"]["cfg3_cold_state_in_host_memory"] = {
+                    "skipped": str(err).splitlines()[0][:300] if str(err) else type(err).__name__}
         if schedule == "keyed" and args.reuse_rows:
             log("secondary: cfg3 with two batches in flight (pipelined schedule, fetched rows reused)")
             sec = run_gpu(args, "cfg3", "pipelined", with_gate=True, with_link=False, reuse_rows=True)

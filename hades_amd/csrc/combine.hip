@@ -469,11 +469,16 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
   const int ngroups = kThreads / G;
   const int bp = ngroups * kChunk;
   const int64_t B0 = static_cast<int64_t>(blockIdx.x) * bp;
+  // runs [run_lo, run_hi) are this launch's to write
+  uint32_t run_lo = 0, run_hi = kNoRun;
   if (a.class_split != nullptr && a.which >= 0) {
     // a block works if its span touches the class; the block that straddles the class border
-    // runs in both launches and writes the same values twice (runs never cross that border)
+    // walks its whole span but writes only the runs of its class (runs never cross that border):
+    // the other class may be summed by another kernel at the same time
     const int64_t sp = a.class_split[0];
     if (a.which == 0 ? B0 >= sp : B0 + bp <= sp) return;
+    const uint32_t sr = static_cast<uint32_t>(a.class_split[1]);
+    if (a.which == 0) run_hi = sr; else run_lo = sr;
   }
   for (int t = threadIdx.x; t < bp + 2; t += kThreads) {
     const int64_t j = B0 - 1 + t;
@@ -527,7 +532,7 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
             // run `cur` ends inside this group: whole unless it is the first run and began earlier
             if (cur == first_run && head_open) {
               s_part[(g * 2 + 0) * G + gl] = acc;
-            } else if (col_ok) {
+            } else if (col_ok && cur >= run_lo && cur < run_hi) {
               *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(cur) * a.dim + col) = acc;
             }
             acc = RowVec<VEC>::zero();
@@ -539,14 +544,15 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
     }
     if (active) {
       // the last run of the group
+      const bool mine = col_ok && cur >= run_lo && cur < run_hi;
       if (cur == first_run) {
         if (!head_open && !tail_open) {
-          if (col_ok) *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(cur) * a.dim + col) = acc;
+          if (mine) *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(cur) * a.dim + col) = acc;
         } else {
           s_part[(g * 2 + 0) * G + gl] = acc;
         }
       } else if (!tail_open) {
-        if (col_ok) *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(cur) * a.dim + col) = acc;
+        if (mine) *reinterpret_cast<V*>(a.sums + static_cast<int64_t>(cur) * a.dim + col) = acc;
       } else {
         s_part[(g * 2 + 1) * G + gl] = acc;
       }
@@ -574,10 +580,11 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
             carry_on = true;
           }
           if (!(single && to)) {                    // ... and it ends inside group gg
-            float* out = (carry_head && carry_outside)
-                             ? a.partial + (2 * static_cast<int64_t>(blockIdx.x)) * a.dim
-                             : a.sums + static_cast<int64_t>(carry_run) * a.dim;
-            if (col_ok) *reinterpret_cast<V*>(out + col) = carry;
+            const bool to_partial = carry_head && carry_outside;
+            float* out = to_partial ? a.partial + (2 * static_cast<int64_t>(blockIdx.x)) * a.dim
+                                    : a.sums + static_cast<int64_t>(carry_run) * a.dim;
+            if (col_ok && (to_partial || (carry_run >= run_lo && carry_run < run_hi)))
+              *reinterpret_cast<V*>(out + col) = carry;
             carry_on = false;
           }
         }
@@ -987,6 +994,20 @@ int sort_ids(const int64_t* ids, int64_t n, int64_t id_bound, void* workspace,
   out->nbad = w.nbad;
   return p.key64 ? run_sort<uint64_t>(ids, n, id_bound, p, w, st, &out->sorted_keys, &out->perm)
                  : run_sort<uint32_t>(ids, n, id_bound, p, w, st, &out->sorted_keys, &out->perm);
+}
+
+int combine_plan_views(void* workspace, size_t workspace_bytes, int64_t n, int64_t dim,
+                       int64_t id_bound, const uint32_t** perm, const uint32_t** seg_start) {
+  HADES_REQUIRE(n >= 1 && n < (int64_t(1) << 30) && dim >= 1 && id_bound >= 0, "bad plan shape");
+  const Plan p = make_plan(n, dim, id_bound, true);
+  const Ws w = carve(workspace, n, dim);
+  if (workspace == nullptr || workspace_bytes < w.bytes)
+    return set_error(HADES_ERR_WORKSPACE, "combine workspace too small: need %zu bytes, got %zu",
+                     w.bytes, workspace_bytes);
+  HADES_REQUIRE((align_of_ptr(workspace) & 255) == 0, "workspace must be 256-byte aligned");
+  *perm = w.sort.vals[(p.passes - 1) & 1];   // where the last pass of the plan left the positions
+  *seg_start = w.seg_start;
+  return HADES_OK;
 }
 
 }  // namespace hades

@@ -72,9 +72,10 @@ bool is_host_memory(const void* p) {
 // Measured on 76 K rows of 512 bytes: a gather reaches the link's read rate (55 GB/s) from 32 to
 // 128 blocks, 53 GB/s with 16; an update that has reads and writes in flight peaks at 128
 // (42.6 GB/s each way); an update that only writes (stores are posted: its waves never wait for
-// the link) saturates it from 32 blocks, and every further store in flight only queues up in front
-// of the HBM traffic of other streams (the segmented sum beside a write-only update of 128 blocks
-// took 690 us, beside one of 32 blocks 155 us, the update itself as long either way).
+// the link) reaches 40 / 50 / 53 GB/s alone with 16 / 32 / 64 blocks and no more beyond; every
+// further store in flight only queues up in front of the HBM traffic of other streams.  Inside a
+// step, beside the hot-class sums: 32 blocks 812 us (sums beside it 153 us), 64 blocks 789 us
+// (573 us), 96 blocks 771 us (642 us, as long as the update itself): 64 it is.
 // HADES_HOST_LINK_BLOCKS / _RW / _WO (read once, at the first use) and
 // hades_set_host_link_blocks() override the three widths for tuning.
 namespace {
@@ -84,7 +85,7 @@ std::atomic<int64_t> g_link_blocks[3] = {{0}, {0}, {0}};   // 0: not set yet
 int64_t host_link_blocks(HostLinkUse use) {
   static const char* const names[] = {"HADES_HOST_LINK_BLOCKS", "HADES_HOST_LINK_BLOCKS_RW",
                                       "HADES_HOST_LINK_BLOCKS_WO"};
-  static const int64_t defaults[] = {16, 128, 32};
+  static const int64_t defaults[] = {16, 128, 64};
   int64_t v = g_link_blocks[use].load(std::memory_order_relaxed);
   if (v > 0) return v;
   v = defaults[use];

@@ -34,6 +34,12 @@ __device__ __forceinline__ int any_flag_set(const int32_t* __restrict__ flags, i
 }
 #endif
 size_t sort_ids_workspace_bytes(int64_t n);
+
+// combine.hip: where a plan made by hades_combine_plan / _plan_classed with the same (n, dim,
+// id_bound) left its sort permutation and its run table inside `workspace`: perm[j] = batch
+// position of sorted position j, seg_start[u] = first sorted position of run u (seg_start[U] = n).
+int combine_plan_views(void* workspace, size_t workspace_bytes, int64_t n, int64_t dim,
+                       int64_t id_bound, const uint32_t** perm, const uint32_t** seg_start);
 int sort_ids(const int64_t* ids, int64_t n, int64_t id_bound, void* workspace,
              size_t workspace_bytes, hipStream_t st, SortResult* out);
 

@@ -8,7 +8,7 @@
 // chunks (scalar when dim is not a multiple of 4): read g, state, w; write state, w.
 // This translation unit is compiled with fused multiply-add contraction off: every operation
 // rounds to fp32 on its own, like the CPU restatement it is checked against.
-#include "common.h"
+#include "internal.h"
 
 namespace hades {
 namespace {
@@ -147,6 +147,15 @@ struct ListedRows {
   const int32_t* first_pos;
   int64_t dim;
   int64_t stride;
+  // Summing class form: `grad` holds one row per QUERY of the batch (not per distinct key) and the
+  // gradient of run u is the sum of rows perm[seg_start[u]] .. perm[seg_start[u + 1] - 1], added
+  // one after the other from +0.0f in that order - the order of occurrence, since the plan's sort
+  // is stable: the arithmetic of the deterministic-order segmented sum, done where it is consumed.
+  // sums_out / cnts_out (optional) receive the summed row and the length of every run.
+  const uint32_t* perm = nullptr;
+  const uint32_t* seg_start = nullptr;
+  float* sums_out = nullptr;
+  int64_t* cnts_out = nullptr;
 };
 
 struct AdagradListedArgs {
@@ -185,22 +194,55 @@ __device__ __forceinline__ void listed_range(const ListedRows& a, int64_t* first
 
 // Offsets of the rows [row0, row0 + rows_here) of the walk: s_tab[r] = table row, s_grad[r] =
 // element offset of the gradient row, s_old[r] = element offset of the old weight row in w_rows.
+template <bool SUMMING>
 __device__ __forceinline__ void resolve_listed(const ListedRows& a, int64_t row0, int rows_here,
-                                               int64_t* s_tab, int64_t* s_grad, int64_t* s_old) {
+                                               int64_t* s_tab, int64_t* s_grad, int64_t* s_old,
+                                               uint32_t* s_j0, uint32_t* s_len) {
   for (int r = threadIdx.x; r < rows_here; r += kThreads) {
     const int64_t p = a.list != nullptr ? a.list[row0 + r] : row0 + r;
     s_tab[r] = a.row_index[p] & a.index_mask;
-    s_grad[r] = p * a.dim;
+    if (SUMMING) {
+      const uint32_t j0 = a.seg_start[p], j1 = a.seg_start[p + 1];
+      s_j0[r] = j0;
+      s_len[r] = j1 - j0;
+      s_grad[r] = static_cast<int64_t>(a.perm[j0]) * a.dim;   // the run's first gradient row
+      if (a.cnts_out != nullptr) a.cnts_out[p] = static_cast<int64_t>(j1 - j0);
+    } else {
+      s_grad[r] = p * a.dim;
+    }
     if (a.w_rows != nullptr) s_old[r] = static_cast<int64_t>(a.first_pos[p]) * a.dim;
   }
 }
 
-template <int VEC>
+// acc + rows 2.. of a run, one after the other in sort order (which is occurrence order); four
+// rows are requested at a time, the additions stay in order
+template <typename V>
+__device__ __forceinline__ V add_rest_of_run(const ListedRows& a, uint32_t j0, uint32_t len,
+                                             int64_t col, V acc) {
+  for (uint32_t j = j0 + 1; j < j0 + len; j += 4) {
+    V row[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (j + t < j0 + len) {
+        const int64_t q = a.perm[j + t];
+        row[t] = __builtin_nontemporal_load(reinterpret_cast<const V*>(a.grad + q * a.dim + col));
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      if (j + t < j0 + len) acc = acc + row[t];
+  }
+  return acc;
+}
+
+template <int VEC, bool SUMMING>
 __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedArgs a) {
   typedef typename Vf<VEC>::type V;
   __shared__ int64_t s_tab[kRows];
   __shared__ int64_t s_grad[kRows];
   __shared__ int64_t s_old[kRows];
+  __shared__ uint32_t s_j0[kRows];
+  __shared__ uint32_t s_len[kRows];
   int64_t first, cnt;
   listed_range(a.r, &first, &cnt);
   const int cpr = static_cast<int>(a.r.dim / VEC);
@@ -208,7 +250,7 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
        row0 += static_cast<int64_t>(gridDim.x) * kRows) {
     const int64_t left = cnt - row0;
     const int rows_here = left < kRows ? static_cast<int>(left) : kRows;
-    resolve_listed(a.r, row0, rows_here, s_tab, s_grad, s_old);
+    resolve_listed<SUMMING>(a.r, row0, rows_here, s_tab, s_grad, s_old, s_j0, s_len);
     __syncthreads();
     const int total = rows_here * cpr;
     for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
@@ -234,16 +276,21 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
       for (int k = 0; k < kUnroll; ++k) {
         const int c = base + k * kThreads;
         if (c < total) {
+          const int r = c / cpr;
+          const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
+          if (SUMMING) {
+            V acc = V(0.0f) + g[k];          // from +0.0f, like the segmented sum: -0.0f becomes +0.0f
+            if (s_len[r] > 1) acc = add_rest_of_run<V>(a.r, s_j0[r], s_len[r], col, acc);
+            g[k] = acc;
+            if (a.r.sums_out != nullptr)
+              *reinterpret_cast<V*>(a.r.sums_out + (row0 + r) * a.r.dim + col) = acc;
+          }
           const V s1 = s[k] + g[k] * g[k];
           const V std_ = vsqrt(s1) + a.eps;
           const V w1 = w[k] - vdiv(a.lr * g[k], std_);
           *sp[k] = s1;
           *wp[k] = w1;
-          if (a.w_out != nullptr) {
-            const int r = c / cpr;
-            const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
-            *reinterpret_cast<V*>(a.w_out + s_grad[r] + col) = w1;
-          }
+          if (a.w_out != nullptr) *reinterpret_cast<V*>(a.w_out + s_grad[r] + col) = w1;
         }
       }
     }
@@ -252,12 +299,14 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
 }
 
 // SparseAdam over the same walk: the arithmetic of adam_kernel below, one table set per launch.
-template <int VEC>
+template <int VEC, bool SUMMING>
 __global__ __launch_bounds__(kThreads) void adam_listed_kernel(AdamListedArgs a) {
   typedef typename Vf<VEC>::type V;
   __shared__ int64_t s_tab[kRows];
   __shared__ int64_t s_grad[kRows];
   __shared__ int64_t s_old[kRows];
+  __shared__ uint32_t s_j0[kRows];
+  __shared__ uint32_t s_len[kRows];
   __shared__ float s_c1[kRows];
   __shared__ float s_c2[kRows];
   int64_t first, cnt;
@@ -267,7 +316,7 @@ __global__ __launch_bounds__(kThreads) void adam_listed_kernel(AdamListedArgs a)
        row0 += static_cast<int64_t>(gridDim.x) * kRows) {
     const int64_t left = cnt - row0;
     const int rows_here = left < kRows ? static_cast<int>(left) : kRows;
-    resolve_listed(a.r, row0, rows_here, s_tab, s_grad, s_old);
+    resolve_listed<SUMMING>(a.r, row0, rows_here, s_tab, s_grad, s_old, s_j0, s_len);
     // thread r wrote s_tab[r] itself: the step counter and the bias corrections of its row
     for (int r = threadIdx.x; r < rows_here; r += kThreads) {
       float* sp = a.step + s_tab[r];
@@ -307,6 +356,15 @@ __global__ __launch_bounds__(kThreads) void adam_listed_kernel(AdamListedArgs a)
       for (int k = 0; k < kUnroll; ++k) {
         const int c = base + k * kThreads;
         if (c < total) {
+          if (SUMMING) {
+            const int r = c / cpr;
+            const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
+            V acc = V(0.0f) + g[k];
+            if (s_len[r] > 1) acc = add_rest_of_run<V>(a.r, s_j0[r], s_len[r], col, acc);
+            g[k] = acc;
+            if (a.r.sums_out != nullptr)
+              *reinterpret_cast<V*>(a.r.sums_out + (row0 + r) * a.r.dim + col) = acc;
+          }
           const V m1 = a.beta1 * m[k] + a.one_minus_beta1 * g[k];
           const V v1 = a.beta2 * v[k] + a.one_minus_beta2 * (g[k] * g[k]);
           const V mc = vdiv(m1, V(c1[k]));
@@ -437,10 +495,15 @@ int launch_adagrad_listed(const AdagradListedArgs& a, void* stream) {
   const dim3 grid = listed_grid(a.r.max_count, w_host || s_host,
                                 s_host || (w_host && a.r.w_rows == nullptr)), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (a.r.dim % 4 == 0 && a.r.stride % 4 == 0 && aligned16({a.r.grad, a.w, a.s, a.r.w_rows, a.w_out}))
-    HADES_LAUNCH((adagrad_listed_kernel<4>), grid, block, 0, st, a);
-  else
-    HADES_LAUNCH((adagrad_listed_kernel<1>), grid, block, 0, st, a);
+  const bool vec4 = a.r.dim % 4 == 0 && a.r.stride % 4 == 0 &&
+                    aligned16({a.r.grad, a.w, a.s, a.r.w_rows, a.w_out, a.r.sums_out});
+  if (a.r.perm != nullptr) {
+    if (vec4) HADES_LAUNCH((adagrad_listed_kernel<4, true>), grid, block, 0, st, a);
+    else HADES_LAUNCH((adagrad_listed_kernel<1, true>), grid, block, 0, st, a);
+  } else {
+    if (vec4) HADES_LAUNCH((adagrad_listed_kernel<4, false>), grid, block, 0, st, a);
+    else HADES_LAUNCH((adagrad_listed_kernel<1, false>), grid, block, 0, st, a);
+  }
   return HADES_OK;
 }
 
@@ -454,10 +517,15 @@ int launch_adam_listed(const ListedRows& r, float* w, float* step, float* m, flo
   const dim3 grid = listed_grid(r.max_count, w_host || state_host,
                                 state_host || (w_host && r.w_rows == nullptr)), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (r.dim % 4 == 0 && r.stride % 4 == 0 && aligned16({r.grad, w, m, v, r.w_rows}))
-    HADES_LAUNCH((adam_listed_kernel<4>), grid, block, 0, st, a);
-  else
-    HADES_LAUNCH((adam_listed_kernel<1>), grid, block, 0, st, a);
+  const bool vec4 = r.dim % 4 == 0 && r.stride % 4 == 0 &&
+                    aligned16({r.grad, w, m, v, r.w_rows, r.sums_out});
+  if (r.perm != nullptr) {
+    if (vec4) HADES_LAUNCH((adam_listed_kernel<4, true>), grid, block, 0, st, a);
+    else HADES_LAUNCH((adam_listed_kernel<1, true>), grid, block, 0, st, a);
+  } else {
+    if (vec4) HADES_LAUNCH((adam_listed_kernel<4, false>), grid, block, 0, st, a);
+    else HADES_LAUNCH((adam_listed_kernel<1, false>), grid, block, 0, st, a);
+  }
   return HADES_OK;
 }
 
@@ -514,6 +582,51 @@ int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const in
   if (rc != HADES_OK || max_rows == 0) return rc;
   HADES_REQUIRE(w && s, "null pointer argument");
   return launch_adagrad_listed(AdagradListedArgs{r, w, s, nullptr, lr, eps}, stream);
+}
+
+int hades_adagrad_update_class_summing(const int64_t* ukeys, const float* grad_rows, int64_t n,
+                                       int64_t key_bound, const int64_t* num_unique,
+                                       const int64_t* class_split, int which, int64_t key_mask,
+                                       int64_t dim, float* w, float* s, int64_t stride,
+                                       const float* w_rows, const int32_t* first_pos,
+                                       float* sums_out, int64_t* cnts_out, float lr, float eps,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+  HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
+  HADES_REQUIRE(n >= 0, "n must be >= 0");
+  if (n == 0) return HADES_OK;
+  ListedRows r{ukeys, grad_rows, nullptr, nullptr, n, num_unique, class_split, which,
+               key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  const int rc = check_listed(r, true);
+  if (rc != HADES_OK) return rc;
+  HADES_REQUIRE(w && s, "null pointer argument");
+  const int rv = combine_plan_views(workspace, workspace_bytes, n, dim, key_bound, &r.perm, &r.seg_start);
+  if (rv != HADES_OK) return rv;
+  r.sums_out = sums_out;
+  r.cnts_out = cnts_out;
+  return launch_adagrad_listed(AdagradListedArgs{r, w, s, nullptr, lr, eps}, stream);
+}
+
+int hades_adam_update_class_summing(const int64_t* ukeys, const float* grad_rows, int64_t n,
+                                    int64_t key_bound, const int64_t* num_unique,
+                                    const int64_t* class_split, int which, int64_t key_mask,
+                                    int64_t dim, float* w, float* step, float* m, float* v,
+                                    int64_t stride, const float* w_rows, const int32_t* first_pos,
+                                    float* sums_out, int64_t* cnts_out, float lr, double beta1,
+                                    double beta2, float eps, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
+  HADES_REQUIRE(n >= 0, "n must be >= 0");
+  if (n == 0) return HADES_OK;
+  ListedRows r{ukeys, grad_rows, nullptr, nullptr, n, num_unique, class_split, which,
+               key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  const int rc = check_listed(r, true);
+  if (rc != HADES_OK) return rc;
+  HADES_REQUIRE(w && step && m && v, "null pointer argument");
+  const int rv = combine_plan_views(workspace, workspace_bytes, n, dim, key_bound, &r.perm, &r.seg_start);
+  if (rv != HADES_OK) return rv;
+  r.sums_out = sums_out;
+  r.cnts_out = cnts_out;
+  return launch_adam_listed(r, w, step, m, v, lr, beta1, beta2, eps, stream);
 }
 
 int hades_adam_update_listed(const int64_t* row_index, const float* grad, const int64_t* list,

@@ -517,45 +517,80 @@ def combine_apply_class(plan, grad, which, mode=COMBINE_FAST, out=None):
     return sums, cnts
 
 
-def adagrad_update_class_(plan, sums, which, w, s, lr, eps, fetched_rows=None):
+def _class_rows(plan, dim, fetched_rows):
+    """first_pos tensor to pass with `fetched_rows` (or None), after checking both"""
+    if fetched_rows is None:
+        return None
+    _dev(fetched_rows, "fetched_rows")
+    _check(plan.first_pos is not None, "the plan was made without first_pos")
+    _check(fetched_rows.dtype == torch.float32 and tuple(fetched_rows.shape) == (plan.n, dim),
+           "fetched_rows must be float32 [n, dim]")
+    return plan.first_pos
+
+
+def _summing_outputs(plan, grad_rows, out):
+    """Checks the per-query gradient rows and the optional (sums, cnts) outputs of a summing
+    class update; returns (sums or None, cnts or None, the plan's live workspace buffer)."""
+    _dev(grad_rows, "grad_rows")
+    _check(grad_rows.dtype == torch.float32 and tuple(grad_rows.shape) == (plan.n, plan.dim),
+           "grad_rows must be float32 [n, dim]: one gradient row per query of the planned batch")
+    sums = cnts = None
+    if out is not None:
+        sums, cnts = out
+        _dev(sums, "sums"); _i64(cnts, "cnts")
+        _check(sums.dtype == torch.float32 and sums.size(0) >= plan.n and sums.size(1) == plan.dim
+               and cnts.numel() >= plan.n, "summing outputs must be float32 [n, dim] and int64 [n]")
+    return sums, cnts, plan.check_live()
+
+
+def adagrad_update_class_(plan, sums, which, w, s, lr, eps, fetched_rows=None, grad_rows=None,
+                          out=None):
     """Sparse Adagrad over one class of a classed plan: the table row of run u is
     plan.uids[u] & (2^key_bits - 1) - the id for the cold class, the slot for the hot class.
     `fetched_rows` (float32[n, D], the rows the forward pass fetched for this batch) makes the
     kernel take the old weight rows from there (row plan.first_pos[u]) instead of reading the
-    table again; valid only while nothing has written those table rows since the fetch."""
-    _dev(sums, "sums")
-    dim = sums.size(1)
+    table again; valid only while nothing has written those table rows since the fetch.
+    With `grad_rows` (float32[n, D], one gradient row per query; `sums` is then ignored and may be
+    None) the kernel sums the rows of every run itself, in occurrence order from +0.0 - the
+    deterministic-order sum - instead of reading them from `sums`; `out` = (sums, cnts) then
+    receives the summed rows and counts of the class."""
+    dim = plan.dim if grad_rows is not None else sums.size(1)
     for name, t in (("w", w), ("s", s)):
         _dev_or_pinned(t, name, contiguous=False)
         _check(t.dtype == torch.float32 and t.dim() == 2 and t.size(1) == dim, "%s: wrong dtype/width" % name)
     stride = _stride_of(w, dim)
     _check(_stride_of(s, dim) == stride, "w and s must have the same row stride")
-    fp = None
-    if fetched_rows is not None:
-        _dev(fetched_rows, "fetched_rows")
-        _check(plan.first_pos is not None, "the plan was made without first_pos")
-        _check(fetched_rows.dtype == torch.float32 and tuple(fetched_rows.shape) == (plan.n, dim),
-               "fetched_rows must be float32 [n, dim]")
-        fp = plan.first_pos
+    fp = _class_rows(plan, dim, fetched_rows)
+    if grad_rows is not None:
+        so, co, ws = _summing_outputs(plan, grad_rows, out)
+        _lib.call("hades_adagrad_update_class_summing", _ptr(plan.uids), _ptr(grad_rows), plan.n,
+                  plan.id_bound, _ptr(plan.num_unique), _ptr(plan.class_split), int(which),
+                  (1 << plan.key_bits) - 1, dim, _ptr(w), _ptr(s), stride, _opt(fetched_rows), _opt(fp),
+                  _opt(so), _opt(co), float(lr), float(eps), _ptr(ws), ws.numel(), _stream())
+        return
+    _dev(sums, "sums")
     _lib.call("hades_adagrad_update_class", _ptr(plan.uids), _ptr(sums), _ptr(plan.num_unique),
               _ptr(plan.class_split), int(which), (1 << plan.key_bits) - 1, plan.uids.numel(), dim,
               _ptr(w), _ptr(s), stride, _opt(fetched_rows), _opt(fp), float(lr), float(eps), _stream())
 
 
-def adam_update_class_(plan, sums, which, tables, lr, beta1, beta2, eps, fetched_rows=None):
-    """SparseAdam over one class of a classed plan; rows and `fetched_rows` as in
-    adagrad_update_class_, `tables` = (w, step, mem, power) of that class."""
-    _dev(sums, "sums")
-    dim = sums.size(1)
+def adam_update_class_(plan, sums, which, tables, lr, beta1, beta2, eps, fetched_rows=None,
+                       grad_rows=None, out=None):
+    """SparseAdam over one class of a classed plan; rows, `fetched_rows`, `grad_rows` and `out` as
+    in adagrad_update_class_, `tables` = (w, step, mem, power) of that class."""
+    dim = plan.dim if grad_rows is not None else sums.size(1)
     stride = _adam_tables(tables, dim)
     w, step, m, v = tables
-    fp = None
-    if fetched_rows is not None:
-        _dev(fetched_rows, "fetched_rows")
-        _check(plan.first_pos is not None, "the plan was made without first_pos")
-        _check(fetched_rows.dtype == torch.float32 and tuple(fetched_rows.shape) == (plan.n, dim),
-               "fetched_rows must be float32 [n, dim]")
-        fp = plan.first_pos
+    fp = _class_rows(plan, dim, fetched_rows)
+    if grad_rows is not None:
+        so, co, ws = _summing_outputs(plan, grad_rows, out)
+        _lib.call("hades_adam_update_class_summing", _ptr(plan.uids), _ptr(grad_rows), plan.n,
+                  plan.id_bound, _ptr(plan.num_unique), _ptr(plan.class_split), int(which),
+                  (1 << plan.key_bits) - 1, dim, _ptr(w), _ptr(step), _ptr(m), _ptr(v), stride,
+                  _opt(fetched_rows), _opt(fp), _opt(so), _opt(co), float(lr), float(beta1),
+                  float(beta2), float(eps), _ptr(ws), ws.numel(), _stream())
+        return
+    _dev(sums, "sums")
     _lib.call("hades_adam_update_class", _ptr(plan.uids), _ptr(sums), _ptr(plan.num_unique),
               _ptr(plan.class_split), int(which), (1 << plan.key_bits) - 1, plan.uids.numel(), dim,
               _ptr(w), _ptr(step), _ptr(m), _ptr(v), stride, _opt(fetched_rows), _opt(fp),

@@ -228,6 +228,9 @@ class _SparseRowOptimizer:
     # one_stream = True runs the cold class on the caller's stream too (no overlap): the same
     # kernels one after the other, e.g. to time each of them undisturbed
     one_stream = False
+    # backward_keyed: the cold update sums the gradient rows of its runs itself instead of waiting
+    # for a segmented sum of the cold class (False: segmented-sum kernels first, as for the hot class)
+    fuse_cold_sums = True
 
     def _split_state(self):
         if getattr(self, "_cold_stream", None) is None:
@@ -500,16 +503,25 @@ class _SparseRowOptimizer:
         self._epoch += 1
         plan.update_epoch = self._epoch
         out = (bufs["sums"][:n], bufs["cnts"][:n])
-        self._timed(timing, "cold_seg_sum", cur,
-                    lambda: ops.combine_apply_class(plan, grad, 0, mode, out=out))
-        cold_summed = torch.cuda.Event()
-        cold_summed.record(cur)
-        cold.wait_event(cold_summed)
+        if self.fuse_cold_sums:
+            # the cold update sums the gradient rows of its runs itself (nearly every cold id
+            # occurs once): it needs the plan and the gradients only, so it starts at once
+            cold.wait_stream(cur)
+            if cold != cur:
+                grad.record_stream(cold)
+        else:
+            self._timed(timing, "cold_seg_sum", cur,
+                        lambda: ops.combine_apply_class(plan, grad, 0, mode, out=out))
+            cold_summed = torch.cuda.Event()
+            cold_summed.record(cur)
+            cold.wait_event(cold_summed)
         if fetched_rows is not None and cold != cur:
             fetched_rows.record_stream(cold)
         with torch.cuda.stream(cold):
             self._timed(timing, "cold_update", cold,
-                        lambda: self._update_keyed(plan, out[0], 0, fetched_rows))
+                        lambda: self._update_keyed(plan, out[0], 0, fetched_rows,
+                                                   grad_rows=grad if self.fuse_cold_sums else None,
+                                                   out=out))
             self._cold_done = torch.cuda.Event()
             self._cold_done.record(cold)
         self._timed(timing, "seg_sum", cur,
@@ -520,7 +532,7 @@ class _SparseRowOptimizer:
             self.join()
         return plan.uids, out[0], out[1], plan.num_unique, plan.class_split
 
-    def _update_keyed(self, plan, sums, which, fetched_rows=None):
+    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None):
         raise NotImplementedError
 
     def distinct_ids_of(self, ukeys, num_unique, key_bits=None):
@@ -568,7 +580,9 @@ class SparseAdagrad(_SparseRowOptimizer):
         a row-strided `weight_cold` it allows one host table [N, 2, D] that holds the weight row
         and the state row of an id next to each other (weight_cold = t[:, 0], cold_state =
         t[:, 1]): one burst per cold row and direction over the host link.  Row-strided cold
-        tables are served by the split schedule (fetch_split / update_split / step_split) only."""
+        tables are served by the split schedule (fetch_split / update_split / step_split) and by
+        the keyed one (forward_keyed / backward_keyed / prefetch_keyed); the one-kernel forms
+        (fetch, update, step) need contiguous tables."""
         super().__init__(weight_cold, hot_ids, lr, device, state_on_device, reuse_fetched_rows)
         self.eps = eps
         if cold_state is not None:
@@ -583,9 +597,10 @@ class SparseAdagrad(_SparseRowOptimizer):
         w, s = (self.hot_w, self.hot_s) if hot else (self.cold_w, self.cold_s)
         ops.adagrad_update_listed_(index, grad, pos, count, w, s, self.lr, self.eps)
 
-    def _update_keyed(self, plan, sums, which, fetched_rows=None):
+    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None):
         w, s = (self.hot_w, self.hot_s) if which else (self.cold_w, self.cold_s)
-        ops.adagrad_update_class_(plan, sums, which, w, s, self.lr, self.eps, fetched_rows=fetched_rows)
+        ops.adagrad_update_class_(plan, sums, which, w, s, self.lr, self.eps, fetched_rows=fetched_rows,
+                                  grad_rows=grad_rows, out=out)
 
     def update(self, uids, grad, num_unique=None):
         self._epoch += 1
@@ -616,9 +631,10 @@ class SparseAdam(_SparseRowOptimizer):
         ops.adam_update_listed_(index, grad, pos, count, self._tables(hot), self.lr,
                                 self.betas[0], self.betas[1], self.eps)
 
-    def _update_keyed(self, plan, sums, which, fetched_rows=None):
+    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None):
         ops.adam_update_class_(plan, sums, which, self._tables(bool(which)), self.lr,
-                               self.betas[0], self.betas[1], self.eps, fetched_rows=fetched_rows)
+                               self.betas[0], self.betas[1], self.eps, fetched_rows=fetched_rows,
+                               grad_rows=grad_rows, out=out)
 
     def update(self, uids, grad, num_unique=None):
         self._epoch += 1

@@ -91,3 +91,25 @@ def fill_normal_(t, std, seed, chunk_rows=1 << 20, progress=None):
         return t
     g = torch.Generator().manual_seed(seed)
     return t.normal_(0.0, std, generator=g)
+
+
+def fill_interleaved_(t, std, seed, chunk_rows=1 << 19, progress=None):
+    """In place, for a pinned host table [N, 2, D] that keeps the weight row and the optimizer
+    state row of an id next to each other: t[:, 0] = N(0, std), t[:, 1] = 0.  Filled from the
+    device in contiguous chunks (a strided host view would be copied through a CPU staging pass)."""
+    assert t.dim() == 3 and t.size(1) == 2 and t.is_contiguous()
+    if not torch.cuda.is_available() or t.is_cuda:
+        g = torch.Generator(device=t.device).manual_seed(seed)
+        t[:, 0].normal_(0.0, std, generator=g)
+        t[:, 1].zero_()
+        return t
+    dev = torch.device("cuda")
+    g = torch.Generator(device=dev).manual_seed(seed)
+    buf = torch.zeros((chunk_rows,) + tuple(t.shape[1:]), dtype=t.dtype, device=dev)
+    for k, r0 in enumerate(range(0, t.size(0), chunk_rows)):
+        rows = min(chunk_rows, t.size(0) - r0)
+        buf[:rows, 0].normal_(0.0, std, generator=g)
+        t[r0:r0 + rows].copy_(buf[:rows])
+        if progress and k % 32 == 31:
+            progress("filled %d of %d rows" % (r0 + rows, t.size(0)))
+    return t

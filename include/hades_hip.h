@@ -76,7 +76,7 @@ int hades_profile_kernel(int kernel_id, void* start_event, void* stop_event);
  * reference, whose row kernels are launched one block per 32 rows whatever the memory,
  * src/cuda/uva_fetch.cu:86-95).  use: 0 a row copy one way (gather from / scatter to a host table),
  * 1 an update that reads and writes host rows, 2 an update that only writes them.  blocks = 0
- * restores the default (16 / 128 / 32, or the HADES_HOST_LINK_BLOCKS, _RW, _WO environment
+ * restores the default (16 / 128 / 64, or the HADES_HOST_LINK_BLOCKS, _RW, _WO environment
  * variables, which are read once, at first use).  Process-wide; meant for tuning and measurement. */
 int hades_set_host_link_blocks(int use, int64_t blocks);
 int64_t hades_get_host_link_blocks(int use);
@@ -405,6 +405,24 @@ int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const in
                                const float* w_rows, const int32_t* first_pos, float lr, float eps,
                                void* stream);
 
+/* hades_adagrad_update_class with the segmented sum of its class folded in: grad_rows holds one
+ * gradient row per QUERY of the batch (float[n, dim]) and the gradient of run u is the sum of the
+ * rows of its occurrences, added one after the other from +0.0f in occurrence order - for every run
+ * exactly what hades_combine_apply_class computes in HADES_COMBINE_EXACT mode (CPU index_add_ order,
+ * python/EmbCache/sparse_optim.py:136-138) - taken from the plan that hades_combine_plan_classed left
+ * in `workspace` for the same n, dim and key_bound.  Meant for the class whose runs are short (the
+ * cold class: nearly every cold id occurs once per batch), where it saves the segmented-sum launches
+ * in front of an update that is bound by the host link anyway; a run of thousands of rows is walked
+ * by one lane group and takes accordingly long.  sums_out (float[n, dim]) and cnts_out (int64[n]),
+ * both optional, receive the summed row and the number of occurrences of every run of the class. */
+int hades_adagrad_update_class_summing(const int64_t* ukeys, const float* grad_rows, int64_t n,
+                                       int64_t key_bound, const int64_t* num_unique,
+                                       const int64_t* class_split, int which, int64_t key_mask,
+                                       int64_t dim, float* w, float* s, int64_t stride,
+                                       const float* w_rows, const int32_t* first_pos,
+                                       float* sums_out, int64_t* cnts_out, float lr, float eps,
+                                       void* workspace, size_t workspace_bytes, void* stream);
+
 /* SparseAdam row update, same fusion (python/EmbCache/sparse_optim.py:632-657,681):
  *   step += 1; m = b1*m + (1-b1)*g; v = b2*v + (1-b2)*g*g
  *   w -= lr * (m / (1 - b1^step)) / (sqrt(v / (1 - b2^step)) + eps)
@@ -434,6 +452,17 @@ int hades_adam_update_class(const int64_t* ukeys, const float* grad, const int64
                             float* v, int64_t stride, const float* w_rows,
                             const int32_t* first_pos, float lr, double beta1, double beta2,
                             float eps, void* stream);
+
+/* SparseAdam over one class with the segmented sum folded in; arguments as in
+ * hades_adagrad_update_class_summing, tables as in hades_adam_update_listed. */
+int hades_adam_update_class_summing(const int64_t* ukeys, const float* grad_rows, int64_t n,
+                                    int64_t key_bound, const int64_t* num_unique,
+                                    const int64_t* class_split, int which, int64_t key_mask,
+                                    int64_t dim, float* w, float* step, float* m, float* v,
+                                    int64_t stride, const float* w_rows, const int32_t* first_pos,
+                                    float* sums_out, int64_t* cnts_out, float lr, double beta1,
+                                    double beta2, float eps, void* workspace,
+                                    size_t workspace_bytes, void* stream);
 
 /* Cold-gradient accumulator (delayed synchronisation): an open-addressing hash table in HBM,
  * int64 key -> fp32[dim] running sum and an int64 count.  Restates on the GPU the arithmetic of

@@ -227,6 +227,70 @@ def test_cfg3_full_size_keyed_and_pipelined(cuda_device):
     assert torch.equal(rows_b, plain_rows(qb))
 
 
+def test_cfg3_batch_with_cold_state_in_host_memory(cuda_device):
+    """The contract layout of the cold class at the size one page-locked allocation allows:
+    weights and Adagrad state of the cold rows both in pinned host memory, the two rows of an id
+    side by side in one [N, 2, D] table of 55.5 M ids (56.8 GB), 5.55 M hot ids in HBM, cfg3's
+    batch of 1 M Zipf(1.05) ids.  Keyed schedule, two steps on the same batch (the second one
+    sees non-zero state in host memory): fetched rows equal plain indexing; weight and state rows
+    of sampled distinct ids (hot, cold, rows beyond 2^31 elements) equal the oracle's Adagrad on
+    their old rows; the state rows of ids outside the batch stay zero."""
+    from hades_amd import ops, synth
+    from hades_amd.sparse_optim import SparseAdagrad
+    cfg = synth.CONFIGS["cfg3"]
+    N, D, H, n = cfg["num_rows"] // 2, cfg["dim"], cfg["num_hot"] // 2, cfg["batch"]
+    dev = cuda_device
+    both = _alloc_or_skip(lambda: torch.empty((N, 2, D), dtype=torch.float32, pin_memory=True),
+                          "the interleaved table needs a 56.8 GB page-locked allocation")
+    synth.fill_interleaved_(both, 0.01, 1239)
+    hot_ids = synth.hot_ids(N, H, dev)
+    opt = _alloc_or_skip(lambda: SparseAdagrad(both[:, 0], hot_ids, lr=0.01, eps=1e-10, device=dev,
+                                               cold_state=both[:, 1]), "needs 10 GB of HBM")
+    assert not opt.cold_s.is_cuda and opt.cold_s.data_ptr() == opt.cold_w.data_ptr() + 4 * D
+    opt.hot_w += 1.0
+    sampler = synth.ZipfSampler(N, cfg["zipf_s"], dev)
+    q = synth.make_ids(sampler, N, n, 1239_000)
+    del sampler
+    uq = torch.unique(q)
+    assert int(uq[-1]) * 2 * D > 2**31
+    gen = torch.Generator().manual_seed(9)
+    pick = torch.randperm(uq.numel(), generator=gen)[:5000].to(dev)
+    sample = torch.unique(torch.cat([uq[pick], uq[-1000:]]))
+
+    def plain_rows(ids):
+        p = torch.searchsorted(hot_ids, ids, right=True)
+        hit = (p > 0) & (hot_ids[(p - 1).clamp(min=0)] == ids)
+        want = _rows_of(opt.cold_w, ids)
+        want[hit] = opt.hot_w[(p - 1)[hit]]
+        return want
+
+    for step in range(2):
+        g = synth.make_grads(n, D, 1239_500 + step, dev)
+        w0, s0, s_hit = _table_rows(opt, sample)
+        assert 0 < int(s_hit.sum()) < sample.numel()
+        want = plain_rows(q)
+        rows, st = opt.forward_keyed(q)
+        torch.cuda.synchronize()
+        assert torch.equal(rows, want)
+        del want
+        ukeys, sums, cnts, nu, split = opt.backward_keyed(st, g, mode=ops.COMBINE_EXACT)
+        torch.cuda.synchronize()
+        assert st[0].reused_rows
+        U = int(nu.item())
+        assert U == uq.numel() and int(cnts[:U].sum()) == n
+        ids = opt.distinct_ids_of(ukeys, nu)
+        order = torch.argsort(ids)
+        assert torch.equal(ids[order], uq)
+        w1, s1 = _sampled_update_check(opt, ids[order], sums[:U][order], U, (w0, s0), sample)
+        gw, gs, _ = _table_rows(opt, sample)
+        assert np.array_equal(gw, w1) and np.array_equal(gs, s1)
+        assert step == 0 or s0.any()
+    others = torch.randint(0, N, (4000,), generator=gen).to(dev)
+    others = others[~torch.isin(others, uq)]
+    _, os_, _ = _table_rows(opt, others)
+    assert not os_.any()
+
+
 def test_cfg5_full_size_local_aggregation_and_update(cuda_device):
     """Four 256 K batches over a 244 M x 64 table in HBM (62.5 GB plus as much Adagrad state):
     combine of the concatenation, then the update; sampled rows against the oracle, the rest of a

@@ -1594,6 +1594,107 @@ def test_keyed_backward_reuses_the_forward_rows_only_while_the_table_is_unwritte
     assert same(guarded, reread)
 
 
+@pytest.mark.parametrize("reuse", [True, False])
+def test_keyed_step_on_an_interleaved_host_table(lib, reuse):
+    """Weights and Adagrad state of the cold rows side by side in one pinned host table
+    [N, 2, D] (weight_cold = t[:, 0], cold_state = t[:, 1]): forward_keyed / backward_keyed over
+    the row-strided views, with and without the reuse of the forward rows, against the oracle -
+    rows, distinct keys, sums and all four tables bit-exact over three steps."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad
+    rng = np.random.default_rng(31 + reuse)
+    N, D, H, n = 9000, 128, 900, 25_000
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, 0.5)
+    q[:300] = q[1]
+    both = torch.zeros((N, 2, D), dtype=torch.float32).pin_memory()
+    both[:, 0] = torch.from_numpy(cold)
+    opt = SparseAdagrad(both[:, 0], torch.from_numpy(hot_ids), lr=0.01, eps=1e-10,
+                        cold_state=both[:, 1], reuse_fetched_rows=reuse)
+    opt.hot_w += 1.0
+    hw = opt.hot_w.cpu().numpy().copy()
+    cw, cs, hs = cold.copy(), np.zeros_like(cold), np.zeros_like(hw)
+    kb = ops.key_bits_for(max(N, H, 2))
+    t_q = dev(q)
+    for it in range(3):
+        grad = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+        rows, state = opt.forward_keyed(t_q)
+        assert np.array_equal(rows.cpu().numpy(), O.cached_fetch(cw, hw, q, hot_ids))
+        ukeys, sums, cnts, nu, split = opt.backward_keyed(state, dev(grad), mode=ops.COMBINE_EXACT)
+        torch.cuda.synchronize()
+        assert state[0].reused_rows == reuse
+        wk, ws, wc, wsplit = O.keyed_step(cw, cs, hw, hs, hot_ids, q, grad, 0.01, 1e-10, kb)
+        U = int(nu.item())
+        assert U == wk.size and np.array_equal(ukeys[:U].cpu().numpy(), wk)
+        assert np.array_equal(cnts[:U].cpu().numpy(), wc) and np.array_equal(sums[:U].cpu().numpy(), ws)
+    assert np.array_equal(both[:, 0].numpy(), cw) and np.array_equal(both[:, 1].numpy(), cs)
+    assert np.array_equal(opt.hot_w.cpu().numpy(), hw) and np.array_equal(opt.hot_s.cpu().numpy(), hs)
+
+
+@pytest.mark.parametrize("kind", ["adagrad", "adam"])
+@pytest.mark.parametrize("host_cold", [False, True])
+@pytest.mark.parametrize("dim", [128, 7])
+def test_cold_update_that_sums_its_own_runs(lib, kind, host_cold, dim):
+    """backward_keyed's cold update adds up the gradient rows of every cold run itself (occurrence
+    order, from +0.0) instead of reading a segmented sum.  Against the path with the segmented-sum
+    kernels in front (fuse_cold_sums = False), in the deterministic-order mode: every table,
+    the returned sums and counts bit-equal over two steps - with cold runs of 1, 2, 5, 70 and
+    3 000 occurrences, gradient rows holding -0.0, and the forward rows reused or not.  In the
+    fast mode the returned sums agree within the combine's tolerance."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad, SparseAdam
+    rng = np.random.default_rng(5150 + dim + host_cold)
+    N, H, n = 40_000, 4000, 30_000
+    cold, hot_ids, q = _split_case(rng, N, dim, H, n, 0.5)
+    cold_ids = np.setdiff1d(np.arange(N, dtype=np.int64), hot_ids)
+    at = 0
+    for k, length in enumerate((2, 5, 70, 3000)):          # planted cold runs, spread over the batch
+        where = rng.choice(n, length, replace=False)
+        q[where] = cold_ids[100 + k]
+    grads = [(rng.standard_normal((n, dim)) * 1e-3).astype(np.float32) for _ in range(2)]
+    grads[0][::7] = -0.0
+    t_q = dev(q)
+
+    def make(fuse, reuse):
+        t = torch.from_numpy(cold.copy())
+        t = t.pin_memory() if host_cold else t.cuda()
+        cls = SparseAdam if kind == "adam" else SparseAdagrad
+        o = cls(t, torch.from_numpy(hot_ids), reuse_fetched_rows=reuse)
+        o.fuse_cold_sums = fuse
+        return o
+
+    def tables(o):
+        ts = ((o.cold_w, o.cold_s, o.hot_w, o.hot_s) if kind == "adagrad" else
+              (o.cold_w, o.cold_step, o.cold_m, o.cold_v, o.hot_w, o.hot_step, o.hot_m, o.hot_v))
+        torch.cuda.synchronize()
+        return [t.cpu().clone() for t in ts]
+
+    for reuse in (True, False):
+        fused, plain = make(True, reuse), make(False, reuse)
+        for g in grads:
+            outs = []
+            for o in (fused, plain):
+                _, st = o.forward_keyed(t_q)
+                uk, sums, cnts, nu, split = o.backward_keyed(st, dev(g), mode=ops.COMBINE_EXACT)
+                torch.cuda.synchronize()
+                U = int(nu.item())
+                outs.append((uk[:U].cpu(), sums[:U].cpu(), cnts[:U].cpu(), split.cpu()))
+            for a, b in zip(outs[0], outs[1]):
+                assert torch.equal(a, b)
+            # signed zeros included: compare the bit patterns of the sums
+            assert np.array_equal(outs[0][1].numpy().view(np.uint32), outs[1][1].numpy().view(np.uint32))
+        for a, b in zip(tables(fused), tables(plain)):
+            assert torch.equal(a, b)
+    # fast mode: the returned sums of both paths within tolerance of the float64 sums
+    fused = make(True, True)
+    _, st = fused.forward_keyed(t_q)
+    uk, sums, cnts, nu, split = fused.backward_keyed(st, dev(grads[1]), mode=ops.COMBINE_FAST)
+    U = int(nu.item())
+    keys = O.class_ordered_keys(q, hot_ids, ops.key_bits_for(N))
+    wk, w64, wc = O.combine_float64(keys, grads[1])
+    assert np.array_equal(uk[:U].cpu().numpy(), wk) and np.array_equal(cnts[:U].cpu().numpy(), wc)
+    assert combine_tol_ok(sums[:U].cpu().numpy(), w64)
+
+
 def test_lookup_split_beyond_the_in_kernel_tile_sum(lib):
     """More than 4 096 tiles of queries: the per-tile counts are prefixed by a scan kernel of their
     own instead of being summed inside every compaction block.  Same lists, same slots."""
