@@ -84,6 +84,8 @@ def parse_args():
                          "in HBM.  host: the contract layout - weights and state both in pinned host "
                          "memory, side by side in one [N, 2, D] table - on a table cut to half the "
                          "rows, which is what one page-locked allocation of this box holds")
+    ap.add_argument("--sort", default=None, choices=["one-sweep", "three-kernels"],
+                    help="form of the radix sort under the combine (default: the library's)")
     ap.add_argument("--allow-fallback", action="store_true",
                     help="if the host refuses cfg3's page-locked table, measure cfg2 instead and say "
                          "so in config.fallback (without this flag such a run exits non-zero)")
@@ -394,6 +396,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     wl = Workload(workload, args.batches, dev, args.optimizer, state_on_host=state_on_host)
+    if args.sort is not None:
+        ops.sort_config(one_sweep=args.sort == "one-sweep")
     opt = wl.opt
     mode = ops.COMBINE_FAST if args.mode == "fast" else ops.COMBINE_EXACT
     nb = len(wl.ids)
@@ -874,6 +878,12 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         res["pcie"] = pcie
     if keyed:
         res["backward_halves_that_reused_the_forward_rows"] = dict(reused)
+    one_sweep = bool(ops._lib.query("hades_sort_mode"))
+    res["sort"] = {"form": "one sweep: histogram of all digits, then one kernel per digit with bounded "
+                           "look-back waits" if one_sweep else
+                           "per digit a count kernel, a scan kernel for large batches and a scatter kernel"}
+    if one_sweep and opt._ws.buf is not None:
+        res["sort"]["tiles_whose_wait_ran_out_in_the_last_sort"] = ops.sort_wait_expiries(opt._ws)
     del wl, opt
     torch.cuda.empty_cache()
     return res

@@ -31,6 +31,7 @@ ABI_VERSION = 130      # HADES_ABI_VERSION of include/hades_hip.h
 _SIGNATURES = {
     "hades_profile_kernel": [c_int, _P, _P],
     "hades_set_host_link_blocks": [c_int, _L],
+    "hades_sort_config": [c_int, _L],
     "hades_pin": [_P, c_size_t],
     "hades_unpin": [_P],
     "hades_host_alloc": [ctypes.POINTER(c_void_p), c_size_t],
@@ -99,6 +100,7 @@ _SIGNATURES = {
                               _L, _P, c_size_t, _P],
 }
 _SIZE_QUERIES = {
+    "hades_sort_mode": [],
     "hades_get_host_link_blocks": [c_int],
     "hades_split_compact_workspace_bytes": [_L],
     "hades_hot_index_bytes": [_L],

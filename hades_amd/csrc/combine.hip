@@ -27,6 +27,8 @@
 //               depends only on (n, dim), so results are reproducible run to run.
 #include "internal.h"
 
+#include <stdlib.h>
+
 #include <atomic>
 #include <mutex>
 
@@ -294,6 +296,253 @@ __global__ __launch_bounds__(kThreads) void radix_pass_kernel(
   }
 }
 
+// ---- the one-sweep sort ---------------------------------------------------------------------
+// One histogram kernel counts the digits of ALL passes in one read of the ids, one small kernel
+// turns the totals into per-pass digit bases, and then every pass is ONE kernel: a tile ranks its
+// keys, publishes its digit counts, obtains the counts of the tiles before it by looking back at
+// what they published, and scatters.  A pass costs one launch instead of two or three.
+//
+// A tile's state is one 32-bit word per digit: status in the two top bits (0 nothing yet, 1 the
+// tile's own count, 2 the count of this tile and all tiles before it), the count below.  The word
+// is read and written whole, so a reader needs no fence: whatever it sees is self-consistent.
+//
+// Every wait is bounded.  A tile waits only for tiles with a smaller block index, which the
+// dispatcher starts earlier; it re-reads their state at most `spin_limit` times and then stops
+// waiting and counts the digits of every key before its own tile straight from the pass's input -
+// which needs no other block - bumps a counter of such events in the workspace, and carries on
+// with the same result.  The sort is correct whatever the order blocks run in; only its speed
+// relies on that order.
+constexpr uint32_t kStatusShift = 30;
+constexpr uint32_t kCountMask = (1u << kStatusShift) - 1u;
+constexpr uint32_t kHasOwn = 1u << kStatusShift;
+constexpr uint32_t kHasAll = 2u << kStatusShift;
+constexpr int kLookback = 8;        // predecessor states a thread requests at a time
+constexpr int kHistThreads = 1024;  // the histogram kernel's block
+constexpr int kHistItems = 8;       // keys per thread of the histogram kernel: chunks of 8192 keys
+constexpr int kHistChunk = kHistThreads * kHistItems;
+constexpr int kSweepStatusWords = 64;   // head of the workspace: [0] tiles whose wait ran out
+
+__device__ __forceinline__ uint32_t load_state(const uint32_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_state(uint32_t* p, uint32_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+struct SweepDigits {
+  int passes;
+  int shift[kMaxPasses];
+  uint32_t mask[kMaxPasses];
+};
+
+// digit counts of every pass over one chunk of the ids; also clears what the pass kernels and the
+// run kernel expect cleared (tile states of pass 0, run-tile states, the event counter) and
+// writes the id-bound flags
+template <typename KeyT>
+__global__ __launch_bounds__(kHistThreads) void sweep_hist_kernel(
+    const int64_t* __restrict__ ids, int64_t n, SweepDigits dg, uint32_t* __restrict__ hist_part,
+    int64_t id_bound, int32_t* __restrict__ bad_blk, int64_t nbad, uint32_t* __restrict__ clear0,
+    int64_t clear0_words, uint32_t* __restrict__ clear1, int64_t clear1_words,
+    uint32_t* __restrict__ status) {
+  __shared__ uint32_t s_hist[kMaxPasses][kBins];
+  for (int i = threadIdx.x; i < dg.passes * kBins; i += kHistThreads) (&s_hist[0][0])[i] = 0;
+  const int64_t c0 = static_cast<int64_t>(blockIdx.x) * kHistChunk;
+  int64_t idv[kHistItems];
+#pragma unroll
+  for (int r = 0; r < kHistItems; ++r) {
+    const int64_t i = c0 + r * kHistThreads + threadIdx.x;
+    idv[r] = i < n ? ids[i] : int64_t(0);
+  }
+  __syncthreads();
+  bool bad = false;
+#pragma unroll
+  for (int r = 0; r < kHistItems; ++r) {
+    const int64_t i = c0 + r * kHistThreads + threadIdx.x;
+    if (i < n) {
+      const int64_t id = idv[r];
+      bad = bad || (id_bound > 0 && (id < 0 || id >= id_bound));
+      const KeyT k = key_from_id<KeyT>(id);
+      for (int p = 0; p < dg.passes; ++p)
+        atomicAdd(&s_hist[p][static_cast<uint32_t>(k >> dg.shift[p]) & dg.mask[p]], 1u);
+    }
+  }
+  const int any_bad = __syncthreads_or(bad ? 1 : 0);
+  if (threadIdx.x == 0) bad_blk[blockIdx.x] = any_bad;
+  // flags past the last chunk belong to nobody: block 0 writes them, so that a reader of all
+  // nbad flags never sees a stale one
+  if (blockIdx.x == 0)
+    for (int64_t b = gridDim.x + threadIdx.x; b < nbad; b += kHistThreads) bad_blk[b] = 0;
+  for (int i = threadIdx.x; i < dg.passes * kBins; i += kHistThreads)
+    hist_part[static_cast<int64_t>(blockIdx.x) * dg.passes * kBins + i] = (&s_hist[0][0])[i];
+  // clearing, spread over the grid
+  const int64_t per0 = (clear0_words + gridDim.x - 1) / gridDim.x;
+  const int64_t per1 = (clear1_words + gridDim.x - 1) / gridDim.x;
+  for (int64_t i = blockIdx.x * per0 + threadIdx.x; i < (blockIdx.x + 1) * per0 && i < clear0_words;
+       i += kHistThreads)
+    clear0[i] = 0;
+  for (int64_t i = blockIdx.x * per1 + threadIdx.x; i < (blockIdx.x + 1) * per1 && i < clear1_words;
+       i += kHistThreads)
+    clear1[i] = 0;
+  if (blockIdx.x == 0 && threadIdx.x < kSweepStatusWords) status[threadIdx.x] = 0;
+}
+
+// bases[p][d] = keys of the whole batch whose digit in pass p is below d.  One block per pass;
+// thread (g, d) adds up the chunk rows g, g + 4, ... of digit d, eight loads in flight.
+__global__ __launch_bounds__(kHistThreads) void sweep_bases_kernel(const uint32_t* __restrict__ hist_part,
+                                                                  int64_t nchunks, int passes,
+                                                                  uint32_t* __restrict__ bases) {
+  constexpr int kParts = kHistThreads / kBins;
+  __shared__ uint32_t s_part[kParts][kBins];
+  __shared__ uint32_t s_scan[kHistThreads / kWave + 1];
+  const int p = blockIdx.x, d = threadIdx.x % kBins, g = threadIdx.x / kBins;
+  uint32_t tot = 0;
+  for (int64_t c0 = g; c0 < nchunks; c0 += 8 * kParts) {
+    uint32_t v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int64_t c = c0 + static_cast<int64_t>(k) * kParts;
+      v[k] = c < nchunks ? hist_part[(c * passes + p) * kBins + d] : 0u;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) tot += v[k];
+  }
+  s_part[g][d] = tot;
+  __syncthreads();
+  uint32_t sum = 0;
+  if (g == 0) {
+#pragma unroll
+    for (int k = 0; k < kParts; ++k) sum += s_part[k][d];
+  }
+  uint32_t total;    // threads beyond the first kBins add nothing and come after them in the scan
+  const uint32_t ex = block_exclusive_sum<uint32_t, kHistThreads>(sum, s_scan, &total);
+  if (g == 0) bases[p * kBins + d] = ex;
+}
+
+// one pass of the one-sweep sort; tile order and ranks exactly as in radix_pass_kernel, so both
+// sorts give the same permutation
+template <typename KeyT, bool FIRST, int IPT>
+__global__ __launch_bounds__(kThreads) void sweep_pass_kernel(
+    const void* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, int64_t n, int shift,
+    uint32_t mask, int bits, const uint32_t* __restrict__ bases, uint32_t* __restrict__ state,
+    uint32_t* __restrict__ next_state, int spin_limit, uint32_t* __restrict__ status,
+    KeyT* __restrict__ keys_out, uint32_t* __restrict__ vals_out) {
+  __shared__ uint32_t s_cnt[kWaves][kBins];
+  __shared__ uint32_t s_glob[kBins];
+  __shared__ int s_gave_up;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t tile = blockIdx.x;
+  const int64_t tile0 = tile * (kThreads * IPT);
+  const int64_t wave0 = tile0 + wave * (IPT * kWave);
+  KeyT key[IPT];
+  uint32_t val[IPT];
+#pragma unroll
+  for (int r = 0; r < IPT; ++r) {
+    const int64_t i = wave0 + r * kWave + lane;
+    const bool valid = i < n;
+    key[r] = valid ? load_key<KeyT, FIRST>(keys_in, i) : KeyT(0);
+    val[r] = valid ? (FIRST ? static_cast<uint32_t>(i) : vals_in[i]) : 0u;
+  }
+  const int d = threadIdx.x;                    // the digit this thread owns (kThreads == kBins)
+  const uint32_t base = bases[d];
+  // the states of the NEXT pass live in the other buffer, last used two passes ago: this tile
+  // clears its own row of it (the kernel boundary makes that visible to the next pass)
+  if (next_state != nullptr) next_state[tile * kBins + d] = 0;
+  for (int i = threadIdx.x; i < kWaves * kBins; i += kThreads) (&s_cnt[0][0])[i] = 0;
+  if (threadIdx.x == 0) s_gave_up = 0;
+  __syncthreads();
+
+  uint32_t rank[IPT];
+  const uint64_t lt_mask = (uint64_t(1) << lane) - 1;
+#pragma unroll
+  for (int r = 0; r < IPT; ++r) {
+    const int64_t i = wave0 + r * kWave + lane;
+    const bool valid = i < n;
+    const uint32_t dd = static_cast<uint32_t>(key[r] >> shift) & mask;
+    const uint64_t peers = match_any(dd, bits, __ballot(valid));
+    uint32_t old = 0;
+    if (valid) old = s_cnt[wave][dd];
+    __builtin_amdgcn_wave_barrier();   // every peer has read the counter before the leader bumps it
+    if (valid && (peers & lt_mask) == 0) s_cnt[wave][dd] = old + __popcll(peers);
+    rank[r] = old + __popcll(peers & lt_mask);
+  }
+  __syncthreads();
+  // exclusive prefix over the waves per digit; own = this tile's keys with digit d
+  uint32_t own = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    const uint32_t t = s_cnt[w][d];
+    s_cnt[w][d] = own;
+    own += t;
+  }
+  uint32_t* my_state = state + tile * kBins + d;
+  uint32_t before = 0;                          // keys with digit d in the tiles before this one
+  if (tile == 0) {
+    store_state(my_state, kHasAll | own);
+  } else {
+    store_state(my_state, kHasOwn | own);
+    // look back, kLookback tiles at a time; wave-uniform control, no block barrier inside
+    int64_t p = tile - 1;
+    bool done = false;
+    int spins = 0;
+    while (true) {
+      bool stuck = false;
+      if (!done) {
+        uint32_t v[kLookback];
+#pragma unroll
+        for (int k = 0; k < kLookback; ++k)
+          v[k] = p - k >= 0 ? load_state(state + (p - k) * kBins + d) : kHasAll;
+#pragma unroll
+        for (int k = 0; k < kLookback; ++k) {
+          if (!done && !stuck) {
+            const uint32_t st = v[k] >> kStatusShift;
+            if (st == 0) {
+              stuck = true;
+            } else {
+              before += v[k] & kCountMask;
+              --p;
+              if (st == 2) done = true;
+            }
+          }
+        }
+      }
+      if (__ballot(!done) == 0) break;
+      if (__ballot(stuck) != 0) {
+        if (++spins > spin_limit) {
+          if (lane == 0) s_gave_up = 1;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+  }
+  __syncthreads();
+  if (s_gave_up) {
+    // the wait ran out: count the digits of every key before this tile from the input itself
+    __shared__ uint32_t s_all[kBins];
+    s_all[d] = 0;
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < tile0; i += kThreads)
+      atomicAdd(&s_all[static_cast<uint32_t>(load_key<KeyT, FIRST>(keys_in, i) >> shift) & mask], 1u);
+    __syncthreads();
+    before = s_all[d];
+    if (threadIdx.x == 0) atomicAdd(status, 1u);
+  }
+  if (tile != 0) store_state(my_state, kHasAll | (before + own));
+  s_glob[d] = base + before;
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < IPT; ++r) {
+    const int64_t i = wave0 + r * kWave + lane;
+    if (i < n) {
+      const uint32_t dd = static_cast<uint32_t>(key[r] >> shift) & mask;
+      const uint32_t pos = s_glob[dd] + s_cnt[wave][dd] + rank[r];
+      keys_out[pos] = key[r];
+      vals_out[pos] = val[r];
+    }
+  }
+}
+
 // ---- run boundaries ---------------------------------------------------------
 constexpr int kUItems = 8;
 constexpr int kUTile = kThreads * kUItems;
@@ -390,6 +639,132 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
           seg_start[u] = static_cast<uint32_t>(n);
           num_unique[0] = violated ? int64_t(-1) : static_cast<int64_t>(u);
           if (class_split != nullptr && kk[k] < thr) {   // no key reaches the threshold
+            class_split[0] = n;
+            class_split[1] = static_cast<int64_t>(u);
+          }
+        }
+      }
+    }
+  }
+}
+
+// run boundaries in one kernel: run_count_kernel's count, the number of runs that begin in earlier
+// tiles obtained by looking back at what those tiles published (one state word per tile, the
+// protocol and the bounded wait of sweep_pass_kernel), then run_emit_kernel's output
+template <typename KeyT>
+__global__ __launch_bounds__(kThreads) void run_sweep_kernel(
+    const KeyT* __restrict__ keys, const uint32_t* __restrict__ perm, int64_t n,
+    uint32_t* __restrict__ tile_state, int spin_limit, uint32_t* __restrict__ status,
+    int64_t* __restrict__ uids, uint32_t* __restrict__ seg_start, uint32_t* __restrict__ seg_of,
+    int64_t* __restrict__ num_unique, int32_t* __restrict__ inverse,
+    const int32_t* __restrict__ bad_blk, int64_t nbad, KeyT thr, int64_t* __restrict__ class_split,
+    int32_t* __restrict__ first_pos) {
+  __shared__ uint32_t smem[kWaves + 1];
+  __shared__ uint32_t s_base;
+  __shared__ int s_gave_up;
+  const int lane = threadIdx.x & (kWave - 1);
+  int violated = 0;
+  if (blockIdx.x == gridDim.x - 1) {
+    for (int64_t b = threadIdx.x; b < nbad; b += kThreads) violated |= bad_blk[b];
+    violated = __syncthreads_or(violated);
+  }
+  const int64_t tile = blockIdx.x;
+  const int64_t j0 = tile * kUTile + threadIdx.x * kUItems;
+  uint32_t flag[kUItems];
+  KeyT kk[kUItems];
+  uint32_t c = 0;
+  if (j0 < n) {
+    KeyT prev = j0 > 0 ? keys[j0 - 1] : KeyT(0);
+#pragma unroll
+    for (int k = 0; k < kUItems; ++k) {
+      const int64_t j = j0 + k;
+      flag[k] = 0;
+      if (j < n) {
+        kk[k] = keys[j];
+        flag[k] = (j == 0 || kk[k] != prev) ? 1u : 0u;
+        prev = kk[k];
+        c += flag[k];
+      }
+    }
+  }
+  uint32_t total;
+  const uint32_t local = block_exclusive_sum<uint32_t, kThreads>(c, smem, &total);
+  if (threadIdx.x == 0) s_gave_up = 0;
+  __syncthreads();
+  // wave 0: publish, look back 64 tiles at a time, publish again
+  if (threadIdx.x < kWave) {
+    uint32_t before = 0;
+    if (tile == 0) {
+      if (lane == 0) store_state(tile_state, kHasAll | total);
+    } else {
+      if (lane == 0) store_state(tile_state + tile, kHasOwn | total);
+      int64_t p = tile - 1;
+      int spins = 0;
+      bool gave_up = false;
+      while (true) {
+        const uint32_t v = p - lane >= 0 ? load_state(tile_state + (p - lane)) : kHasAll;
+        const uint32_t st = v >> kStatusShift;
+        const uint64_t all_m = __ballot(st == 2), none_m = __ballot(st == 0);
+        // the nearest tile that knows everything before it, and whether every tile nearer than
+        // that has at least published its own count
+        const int first_all = all_m ? __builtin_ctzll(all_m) : kWave;
+        const int first_none = none_m ? __builtin_ctzll(none_m) : kWave;
+        const int upto = first_all < first_none ? first_all + 1 : first_none;   // lanes [0, upto) count
+        uint32_t part = lane < upto ? (v & kCountMask) : 0u;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+        before += part;
+        p -= upto;
+        if (first_all < first_none) break;
+        if (first_none < kWave) {               // a tile in the window has published nothing yet
+          if (++spins > spin_limit) { gave_up = true; break; }
+          __builtin_amdgcn_s_sleep(1);
+        }
+      }
+      if (gave_up && lane == 0) s_gave_up = 1;
+    }
+    if (lane == 0) s_base = before;
+  }
+  __syncthreads();
+  if (s_gave_up) {
+    // the wait ran out: count the runs that begin before this tile from the keys themselves
+    uint32_t cnt = 0;
+    for (int64_t j = threadIdx.x; j < tile * kUTile && j < n; j += kThreads)
+      cnt += (j == 0 || keys[j] != keys[j - 1]) ? 1u : 0u;
+    uint32_t tot2;
+    (void)block_exclusive_sum<uint32_t, kThreads>(cnt, smem, &tot2);
+    if (threadIdx.x == 0) {
+      s_base = tot2;
+      atomicAdd(status, 1u);
+    }
+    __syncthreads();
+  }
+  const uint32_t blk_base = s_base;
+  if (threadIdx.x == 0 && tile != 0) store_state(tile_state + tile, kHasAll | (blk_base + total));
+  uint32_t u = blk_base + local;   // runs that begin before j0
+  if (j0 < n) {
+#pragma unroll
+    for (int k = 0; k < kUItems; ++k) {
+      const int64_t j = j0 + k;
+      if (j < n) {
+        u += flag[k];
+        const uint32_t seg = u - 1;
+        seg_of[j] = seg;
+        if (inverse) inverse[perm[j]] = static_cast<int32_t>(seg);
+        if (flag[k]) {
+          uids[seg] = id_from_key<KeyT>(kk[k]);
+          seg_start[seg] = static_cast<uint32_t>(j);
+          if (first_pos != nullptr) first_pos[seg] = static_cast<int32_t>(perm[j]);
+          if (class_split != nullptr && kk[k] >= thr &&
+              (j == 0 || (k > 0 ? kk[k - 1] : keys[j - 1]) < thr)) {
+            class_split[0] = j;
+            class_split[1] = static_cast<int64_t>(seg);
+          }
+        }
+        if (j == n - 1) {
+          seg_start[u] = static_cast<uint32_t>(n);
+          num_unique[0] = violated ? int64_t(-1) : static_cast<int64_t>(u);
+          if (class_split != nullptr && kk[k] < thr) {
             class_split[0] = n;
             class_split[1] = static_cast<int64_t>(u);
           }
@@ -862,32 +1237,45 @@ Plan make_plan(int64_t n, int64_t dim, int64_t id_bound, bool grad_aligned) {
 
 // workspace of the sort alone
 struct SortWs {
-  int32_t* bad;         // [ceil(ntiles / kGroup)]: 1 where a block of the first count pass saw an id
-                        // outside [0, id_bound); rewritten in full by every sort
+  uint32_t* status;     // [kSweepStatusWords], first thing in the workspace: [0] = tiles of the last
+                        // one-sweep sort whose bounded wait ran out (they recounted instead)
+  int32_t* bad;         // [nbad]: 1 where a block of the first count pass saw an id outside
+                        // [0, id_bound); rewritten in full by every sort
   int64_t nbad;
   void* keys[2];
   uint32_t* vals[2];
-  uint32_t* cnt;        // [ntiles][kBins], rewritten by every pass
+  uint32_t* cnt;        // [ntiles][kBins], rewritten by every pass; the one-sweep sort keeps the
+                        // tile states of its even passes here
   uint32_t* gcnt;       // [ceil(ntiles / kGroup)][kBins]: sums of kGroup consecutive rows of cnt
   int64_t cnt_len;
+  uint32_t* state1;     // [ntiles][kBins]: tile states of the odd passes of the one-sweep sort
+  uint32_t* hist_part;  // [nchunks][kMaxPasses][kBins]: per-chunk digit counts of every pass
+  uint32_t* bases;      // [kMaxPasses][kBins]
+  int64_t nchunks;
   size_t bytes;
 };
 
 void carve_sort(Carver& c, int64_t n, SortWs* w) {
   const int64_t nn = n > 0 ? n : 1;
+  w->status = c.take<uint32_t>(kSweepStatusWords);
   for (int i = 0; i < 2; ++i) w->keys[i] = c.take<uint64_t>(nn);  // sized for 64-bit keys
   for (int i = 0; i < 2; ++i) w->vals[i] = c.take<uint32_t>(nn);
   w->cnt_len = make_plan(nn, 1, 0, true).ntiles * kBins;  // the tile count depends on n only
-  w->nbad = ceil_div(w->cnt_len / kBins, kGroup);
+  w->nchunks = ceil_div(nn, kHistChunk);
+  const int64_t ngroups = ceil_div(w->cnt_len / kBins, kGroup);
+  w->nbad = ngroups > w->nchunks ? ngroups : w->nchunks;
   w->bad = c.take<int32_t>(w->nbad);
   w->cnt = c.take<uint32_t>(w->cnt_len);
-  w->gcnt = c.take<uint32_t>((ceil_div(w->cnt_len / kBins, kGroup) + 1) * kBins);  // + totals row
+  w->gcnt = c.take<uint32_t>((ngroups + 1) * kBins);  // + totals row
+  w->state1 = c.take<uint32_t>(w->cnt_len);
+  w->hist_part = c.take<uint32_t>(w->nchunks * kMaxPasses * kBins);
+  w->bases = c.take<uint32_t>(kMaxPasses * kBins);
   w->bytes = c.total();
 }
 
 struct Ws {
   SortWs sort;
-  uint32_t* run_cnt;
+  uint32_t* run_cnt;    // [run tiles + 1]: per-tile run counts, or the tile states of run_sweep_kernel
   uint32_t* seg_of;
   uint32_t* seg_start;
   float* partial;
@@ -908,9 +1296,18 @@ Ws carve(void* ws, int64_t n, int64_t dim) {
   return w;
 }
 
+// process-wide choice of the sort and the bound of its waits (hades_sort_config).  The default is
+// the form without waits: measured on 65 K / 200 K / 1 M keys the one-sweep form was slower by
+// 10 / 19 / 30 us per sort - a pass with the look-back inside costs 12 - 14 us at 200 K keys and
+// 20 - 26 us at 1 M, as much as the count, scan and scatter kernels it replaces (4.5 + 8.8 us and
+// 5 + 3.5 + 14.4 us), and the histogram and base kernels come on top.
+std::atomic<int> g_one_sweep{0};
+std::atomic<int> g_spin_limit{50000};
+
 template <typename KeyT>
-int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
-                 hipStream_t st, const void** keys_out, const uint32_t** perm_out) {
+int run_sort_three_kernels(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
+                           const SortWs& w, hipStream_t st, const void** keys_out,
+                           const uint32_t** perm_out) {
   const int64_t ngroups = ceil_div(p.ntiles, kGroup);
   HADES_REQUIRE(p.ntiles * kBins <= w.cnt_len, "internal: radix count buffer too small");
   constexpr int IPT = kIpt;
@@ -955,12 +1352,83 @@ int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, con
   return HADES_OK;
 }
 
+// The one-sweep sort: histogram of all passes, digit bases, then one kernel per pass.
+// run_state / run_state_words: further words to clear for the run kernel that follows (or null).
+template <typename KeyT>
+int run_sort_one_sweep(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
+                       const SortWs& w, hipStream_t st, uint32_t* run_state,
+                       int64_t run_state_words, const void** keys_out, const uint32_t** perm_out) {
+  HADES_REQUIRE(p.ntiles * kBins <= w.cnt_len, "internal: tile state buffer too small");
+  constexpr int IPT = kIpt;
+  SweepDigits dg;
+  dg.passes = p.passes;
+  const int base = p.key_bits / p.passes, extra = p.key_bits % p.passes;
+  int bits_of[kMaxPasses];
+  int shift = 0;
+  for (int pass = 0; pass < kMaxPasses; ++pass) {
+    bits_of[pass] = pass < p.passes ? base + (pass < extra ? 1 : 0) : 0;
+    dg.shift[pass] = shift;
+    dg.mask[pass] = bits_of[pass] ? (1u << bits_of[pass]) - 1u : 0u;
+    shift += bits_of[pass];
+  }
+  const dim3 block(kThreads), hblock(kHistThreads), hgrid(static_cast<unsigned>(w.nchunks)),
+      grid(static_cast<unsigned>(p.ntiles));
+  HADES_LAUNCH((sweep_hist_kernel<KeyT>), hgrid, hblock, 0, st, idx, n, dg, w.hist_part, id_bound,
+               w.bad, w.nbad, w.cnt, p.ntiles * kBins, run_state, run_state_words, w.status);
+  HADES_LAUNCH(sweep_bases_kernel, dim3(static_cast<unsigned>(p.passes)), hblock, 0, st,
+               w.hist_part, w.nchunks, p.passes, w.bases);
+  const int spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+  // keys per thread of a pass: larger tiles for larger batches, so that a pass has a few hundred
+  // tiles whatever the size - the look-back chain and its traffic grow with the number of tiles
+  static const int ipt_env = [] { const char* e = getenv("HADES_SWEEP_IPT"); return e ? atoi(e) : 0; }();
+  int ipt = n > (int64_t(1) << 19) ? 16 : (n > (int64_t(1) << 18) ? 8 : 4);
+  if (ipt_env == 4 || ipt_env == 8 || ipt_env == 16) ipt = ipt_env;
+  const dim3 pgrid(static_cast<unsigned>(ceil_div(n, static_cast<int64_t>(kThreads) * ipt)));
+  const void* kin = idx;
+  const uint32_t* vin = nullptr;
+  int cur = 0;
+  for (int pass = 0; pass < p.passes; ++pass) {
+    KeyT* kout = static_cast<KeyT*>(w.keys[cur]);
+    uint32_t* vout = w.vals[cur];
+    uint32_t* state = (pass & 1) ? w.state1 : w.cnt;
+    uint32_t* next_state = pass + 1 < p.passes ? ((pass & 1) ? w.cnt : w.state1) : nullptr;
+#define HADES_SWEEP_PASS(FIRST_, IPT_)                                                             \
+  HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (sweep_pass_kernel<KeyT, FIRST_, IPT_>), pgrid,  \
+                     block, 0, st, kin, vin, n, dg.shift[pass], dg.mask[pass], bits_of[pass],      \
+                     w.bases + pass * kBins, state, next_state, spin_limit, w.status, kout, vout)
+    if (pass == 0) {
+      if (ipt == 16) HADES_SWEEP_PASS(true, 16);
+      else if (ipt == 8) HADES_SWEEP_PASS(true, 8);
+      else HADES_SWEEP_PASS(true, 4);
+    } else {
+      if (ipt == 16) HADES_SWEEP_PASS(false, 16);
+      else if (ipt == 8) HADES_SWEEP_PASS(false, 8);
+      else HADES_SWEEP_PASS(false, 4);
+    }
+#undef HADES_SWEEP_PASS
+    kin = kout;
+    vin = vout;
+    cur ^= 1;
+  }
+  *keys_out = kin;
+  *perm_out = vin;
+  return HADES_OK;
+}
+
 template <typename KeyT>
 int run_runs(const void* sorted_keys, const uint32_t* perm, int64_t n, const Plan& p, const Ws& w,
-             int64_t* uids, int64_t* num_unique, int32_t* inverse, hipStream_t st,
+             int64_t* uids, int64_t* num_unique, int32_t* inverse, hipStream_t st, bool one_sweep,
              int64_t threshold = 0, int64_t* class_split = nullptr, int32_t* first_pos = nullptr) {
   const KeyT* keys = static_cast<const KeyT*>(sorted_keys);
   const dim3 rgrid(static_cast<unsigned>(p.nblocks_runs)), block(kThreads);
+  if (one_sweep) {
+    // w.run_cnt holds the tile states, cleared by the sort's histogram kernel
+    HADES_LAUNCH((run_sweep_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt,
+                 g_spin_limit.load(std::memory_order_relaxed), w.sort.status, uids, w.seg_start,
+                 w.seg_of, num_unique, inverse, w.sort.bad, w.sort.nbad,
+                 key_from_id<KeyT>(threshold), class_split, first_pos);
+    return HADES_OK;
+  }
   HADES_LAUNCH((run_count_kernel<KeyT>), rgrid, block, 0, st, keys, n, w.run_cnt);
   HADES_LAUNCH_CHECK();
   HADES_LAUNCH((run_emit_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt, uids,
@@ -968,6 +1436,16 @@ int run_runs(const void* sorted_keys, const uint32_t* perm, int64_t n, const Pla
                      key_from_id<KeyT>(threshold), class_split, first_pos);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
+}
+
+template <typename KeyT>
+int run_sort(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p, const SortWs& w,
+             hipStream_t st, bool one_sweep, uint32_t* run_state, int64_t run_state_words,
+             const void** keys_out, const uint32_t** perm_out) {
+  if (one_sweep)
+    return run_sort_one_sweep<KeyT>(idx, n, id_bound, p, w, st, run_state, run_state_words,
+                                    keys_out, perm_out);
+  return run_sort_three_kernels<KeyT>(idx, n, id_bound, p, w, st, keys_out, perm_out);
 }
 
 }  // namespace
@@ -992,8 +1470,11 @@ int sort_ids(const int64_t* ids, int64_t n, int64_t id_bound, void* workspace,
   out->key64 = p.key64;
   out->bad = w.bad;
   out->nbad = w.nbad;
-  return p.key64 ? run_sort<uint64_t>(ids, n, id_bound, p, w, st, &out->sorted_keys, &out->perm)
-                 : run_sort<uint32_t>(ids, n, id_bound, p, w, st, &out->sorted_keys, &out->perm);
+  const bool sweep = g_one_sweep.load(std::memory_order_relaxed) != 0;
+  return p.key64 ? run_sort<uint64_t>(ids, n, id_bound, p, w, st, sweep, nullptr, 0,
+                                      &out->sorted_keys, &out->perm)
+                 : run_sort<uint32_t>(ids, n, id_bound, p, w, st, sweep, nullptr, 0,
+                                      &out->sorted_keys, &out->perm);
 }
 
 int combine_plan_views(void* workspace, size_t workspace_bytes, int64_t n, int64_t dim,
@@ -1015,6 +1496,17 @@ int combine_plan_views(void* workspace, size_t workspace_bytes, int64_t n, int64
 using namespace hades;
 
 extern "C" {
+
+int hades_sort_config(int one_sweep, int64_t spin_limit) {
+  HADES_REQUIRE(one_sweep >= -1 && one_sweep <= 1, "one_sweep must be 0, 1 or -1 (leave as it is)");
+  HADES_REQUIRE(spin_limit >= -1 && spin_limit <= (int64_t(1) << 30),
+                "spin_limit must be in [0, 2^30] or -1 (leave as it is)");
+  if (one_sweep >= 0) g_one_sweep.store(one_sweep, std::memory_order_relaxed);
+  if (spin_limit >= 0) g_spin_limit.store(static_cast<int>(spin_limit), std::memory_order_relaxed);
+  return HADES_OK;
+}
+
+int hades_sort_mode(void) { return g_one_sweep.load(std::memory_order_relaxed); }
 
 size_t hades_combine_workspace_bytes(int64_t n, int64_t dim) {
   if (n < 0 || dim < 1) return 0;
@@ -1055,13 +1547,16 @@ int combine_plan_impl(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bou
 
   const uint32_t* perm = nullptr;
   const void* sorted_keys = nullptr;
-  int rc = p.key64 ? run_sort<uint64_t>(idx, n, id_bound, p, w.sort, st, &sorted_keys, &perm)
-                   : run_sort<uint32_t>(idx, n, id_bound, p, w.sort, st, &sorted_keys, &perm);
+  const bool sweep = g_one_sweep.load(std::memory_order_relaxed) != 0;
+  int rc = p.key64 ? run_sort<uint64_t>(idx, n, id_bound, p, w.sort, st, sweep, w.run_cnt,
+                                        p.nblocks_runs + 1, &sorted_keys, &perm)
+                   : run_sort<uint32_t>(idx, n, id_bound, p, w.sort, st, sweep, w.run_cnt,
+                                        p.nblocks_runs + 1, &sorted_keys, &perm);
   if (rc != HADES_OK) return rc;
   return p.key64 ? run_runs<uint64_t>(sorted_keys, perm, n, p, w, uids, num_unique, inverse, st,
-                                      threshold, class_split, first_pos)
+                                      sweep, threshold, class_split, first_pos)
                  : run_runs<uint32_t>(sorted_keys, perm, n, p, w, uids, num_unique, inverse, st,
-                                      threshold, class_split, first_pos);
+                                      sweep, threshold, class_split, first_pos);
 }
 
 }  // namespace

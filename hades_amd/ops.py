@@ -106,6 +106,25 @@ def set_host_link_blocks(use, blocks):
     return old
 
 
+def sort_config(one_sweep=None, spin_limit=None):
+    """Chooses the sort under combine / bucketing / flush (process-wide): one_sweep True = one
+    kernel per digit with bounded look-back waits, False = count + scatter kernels per digit;
+    spin_limit = re-reads a tile spends on a predecessor that has published nothing before it
+    recounts by itself (0: at once).  None leaves a setting alone.  Returns the form in force
+    before the call (True = one sweep)."""
+    old = bool(_lib.query("hades_sort_mode"))
+    _lib.call("hades_sort_config", -1 if one_sweep is None else int(bool(one_sweep)),
+              -1 if spin_limit is None else int(spin_limit))
+    return old
+
+
+def sort_wait_expiries(workspace):
+    """Tiles of the last one-sweep sort in `workspace` (a Workspace, or the uint8 buffer itself)
+    whose bounded wait ran out and which recounted instead.  One host synchronisation."""
+    buf = workspace.buf if isinstance(workspace, Workspace) else workspace
+    return int(buf[:4].view(torch.int32).item())
+
+
 # ---- the hot set and lookup -----------------------------------------------------
 class HotSet:
     """The ascending, duplicate-free hot ids on the device together with the bucket index that

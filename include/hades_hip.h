@@ -301,6 +301,23 @@ int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim,
                   int mode, int64_t* uids, float* sums, int64_t* cnts, int64_t* num_unique,
                   int32_t* inverse, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The sort under hades_combine (and under the bucketing, the accumulator's flush and the index
+ * cache).  The reference gets its sort from torch.unique (python/EmbCache/sparse_optim.py:133-135);
+ * here it is a stable LSD radix sort in one of two forms that give the same permutation:
+ *   one_sweep = 1: one histogram kernel for all digits, then ONE kernel per digit in which
+ *     every tile learns the digit counts of the tiles before it by looking back at what they have
+ *     published.  Each such wait is bounded: after spin_limit fruitless re-reads a tile stops
+ *     waiting, counts the keys before it from the pass's input itself and goes on - same result,
+ *     and the first 32-bit word of the workspace (cleared by every sort) counts the tiles that did.
+ *   one_sweep = 0 (default: the faster one on MI355X at every batch size measured): per digit a
+ *     count kernel, for large batches a scan kernel, and a scatter kernel; no kernel ever waits for
+ *     another block.
+ * -1 leaves a setting as it is.  spin_limit 0 makes every tile that finds a predecessor not ready
+ * give up at once (a way to exercise the recount from the host).  Process-wide; hades_sort_mode
+ * returns the current form. */
+int hades_sort_config(int one_sweep, int64_t spin_limit);
+int hades_sort_mode(void);
+
 /* The same in two halves.  The sort and the run boundaries depend on the ids alone, which a
  * trainer knows at forward time (python/EmbCache/dist_emb.py:276-288 saves them for the optimizer),
  * long before the gradients exist: hades_combine_plan can run then, on another stream, and

@@ -564,9 +564,18 @@ CASES = [  # (n, dim, id space, kind)
 ]
 
 
+@pytest.fixture(params=["one_sweep", "three_kernels"])
+def sort_form(request, lib):
+    """runs a test once with each form of the sort under the combine; restores the default"""
+    _, ops = lib
+    before = ops.sort_config(one_sweep=request.param == "one_sweep")
+    yield request.param
+    ops.sort_config(one_sweep=before)
+
+
 @pytest.mark.parametrize("n,dim,space,kind", CASES)
 @pytest.mark.parametrize("bounded", [True, False])
-def test_combine(lib, n, dim, space, kind, bounded):
+def test_combine(lib, sort_form, n, dim, space, kind, bounded):
     _, ops = lib
     rng = np.random.default_rng(9 + n + dim)
     if kind == "same":
@@ -608,6 +617,53 @@ def test_combine(lib, n, dim, space, kind, bounded):
         # runs that fit inside one chunk are summed left to right: bit-equal to the exact mode
         short = wc <= 1
         assert np.array_equal(got[short], ws[short])
+
+
+@pytest.mark.parametrize("n,space,bounded", [(5000, 300, True), (70_001, 5000, True), (262_145, 3_000_000, True),
+                                             (150_000, 40, True), (100_000, 2_400_000, False)])
+def test_one_sweep_sort_when_its_waits_run_out(lib, n, space, bounded):
+    """The one-sweep sort with a spin limit of 0: every tile that finds a predecessor not ready
+    gives up at once and counts the keys before it from the input itself.  The result (distinct
+    ids, counts, inverse, deterministic-order sums) is that of the oracle all the same; the
+    workspace's counter says how many tiles went that way; every kernel returned (the stream
+    synchronises).  With the default limit the same call reports no such tile."""
+    _, ops = lib
+    rng = np.random.default_rng(n)
+    idx = zipfish(rng, n, space)
+    if not bounded:
+        idx = idx.copy()
+        idx[:3] = [-5, 2**40 + 7, -(2**50)]
+    grad = (rng.standard_normal((n, 4)) * 1e-3).astype(np.float32)
+    wu, ws, wc = O.combine_sequential(idx, grad)
+    t_idx, t_grad = dev(idx), dev(grad)
+    ws_buf = ops.Workspace("cuda")
+    before = ops.sort_config(one_sweep=True, spin_limit=0)
+    try:
+        expiries = []
+        for _ in range(3):
+            uids, sums, cnts, nu, inv = ops.combine_padded(t_idx, t_grad, space if bounded else 0,
+                                                           ops.COMBINE_EXACT, return_inverse=True,
+                                                           workspace=ws_buf)
+            torch.cuda.synchronize()
+            expiries.append(ops.sort_wait_expiries(ws_buf))
+            U = int(nu.item())
+            assert U == wu.size and np.array_equal(uids[:U].cpu().numpy(), wu)
+            assert np.array_equal(cnts[:U].cpu().numpy(), wc) and np.array_equal(sums[:U].cpu().numpy(), ws)
+            assert np.array_equal(wu[inv.cpu().numpy()], idx)
+        # with more than a handful of tiles in flight at once some tile always finds a
+        # predecessor that has not published yet
+        assert n < 50_000 or max(expiries) > 0
+    finally:
+        ops.sort_config(one_sweep=before, spin_limit=50000)
+    ops.sort_config(one_sweep=True)
+    try:
+        uids, sums, cnts, nu = ops.combine_padded(t_idx, t_grad, space if bounded else 0, ops.COMBINE_EXACT,
+                                                  workspace=ws_buf)
+        torch.cuda.synchronize()
+        assert ops.sort_wait_expiries(ws_buf) == 0
+        assert np.array_equal(uids[:int(nu.item())].cpu().numpy(), wu)
+    finally:
+        ops.sort_config(one_sweep=before)
 
 
 def test_rows_and_update_generated_shapes(lib):
