@@ -84,6 +84,11 @@ def parse_args():
                          "in HBM.  host: the contract layout - weights and state both in pinned host "
                          "memory, side by side in one [N, 2, D] table - on a table cut to half the "
                          "rows, which is what one page-locked allocation of this box holds")
+    ap.add_argument("--average", default=None, choices=["sum", "mean", "one_plus"],
+                    help="what the update applies for an id that occurs several times in a batch: the "
+                         "sum of its gradient rows (the configurations' combine; default for Adagrad), "
+                         "or their mean as the reference's update does (unique_grads; default for "
+                         "--optimizer adam), or the sum over one plus the occurrences")
     ap.add_argument("--sort", default=None, choices=["one-sweep", "three-kernels"],
                     help="form of the radix sort under the combine (default: the library's)")
     ap.add_argument("--allow-fallback", action="store_true",
@@ -293,7 +298,7 @@ def link_kernel_probe(wl, reps=3):
     return out
 
 
-def parity_gate(wl, step_fn, rows=20_000):
+def parity_gate(wl, step_fn, rows=20_000, average=None, rows_are_sums=True):
     """One untimed step in the deterministic-order mode on the first `rows` ids of batch 0,
     through the same schedule as the timed steps, checked against torch's own device operators:
     slots and fetched rows bit-exact, distinct ids and counts exact, summed gradients and the
@@ -357,8 +362,15 @@ def parity_gate(wl, step_fn, rows=20_000):
         assert worst <= 1e-5, "parity gate: %s off by %.3g relative" % (what, worst)
         return worst
 
-    e_sum = close(sums[:u], sums64, "summed gradients")
-    gs = sums[:u]
+    # the keyed schedule returns the sums and divides inside its update kernels; the other
+    # schedules divide the combined rows in place before the update
+    div = (cnt + (1 if average == "one_plus" else 0)).to(torch.float32).unsqueeze(1) if average else None
+    if average and not rows_are_sums:
+        e_sum = close(sums[:u], sums64 / div.double(), "averaged gradients")
+        gs = sums[:u]
+    else:
+        e_sum = close(sums[:u], sums64, "summed gradients")
+        gs = sums[:u] / div if average else sums[:u]
     w_got, _ = table_rows(opt.cold_w, opt.hot_w, uniq)
     if adam:
         # the reference's float32 arithmetic (python/EmbCache/sparse_optim.py:632-657,681) in torch
@@ -417,6 +429,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         return evs
 
     uids_o, sums_o, cnts_o, nu_o = wl.comb_out
+    average = args.average if args.average is not None else ("mean" if args.optimizer == "adam" else None)
+    average = None if average == "sum" else average
     reused = {"yes": 0, "no": 0}    # backward halves that took / did not take the forward rows
 
     def run_step(q, g, cmode, events=None, timing=None):
@@ -443,7 +457,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
             if events: events[1].record()
             if events: events[2].record()
             res = opt.backward_keyed(state, g, cmode, timing=timing,
-                                     fetched_rows="auto" if reuse_rows else None)
+                                     fetched_rows="auto" if reuse_rows else None, average=average)
             reused["yes" if state[0].reused_rows else "no"] += 1
         elif split:
             opt.fetch_split(q, out=rows, join=False, timing=timing)
@@ -452,7 +466,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
             if events: events[1].record()
             res = ops.combine_apply(plan, g, cmode, out=out_sum)
             if events: events[2].record()
-            opt.update_split(res[0], res[1], res[3], join=True, timing=timing)
+            opt.update_split(res[0], res[1], res[3], join=True, timing=timing, cnts=res[2],
+                             average=average)
         else:
             if overlap:
                 plan = opt.prepare(q, out=out_ids)
@@ -464,6 +479,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
                 plan = ops.combine_plan(q, D, id_bound=N, workspace=opt._ws, out=out_ids)
             res = ops.combine_apply(plan, g, cmode, out=out_sum)
             if events: events[2].record()
+            if average:
+                ops.rows_div_count_(res[1], res[2], res[3], one_plus=average == "one_plus")
             opt.update(res[0], res[1], res[3])
         if events: events[3].record()
         return rows, res
@@ -490,7 +507,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
         if events: events[1].record()
         if events: events[2].record()
         res = opt.backward_keyed(st, wl.grads[i % nb], cmode, timing=timing,
-                                 fetched_rows="auto" if reuse_rows else None, join=False)
+                                 fetched_rows="auto" if reuse_rows else None, join=False,
+                                 average=average)
         reused["yes" if st[0].reused_rows else "no"] += 1
         rows2, st2 = opt.finish_prefetch(nxt, after=st, timing=timing)
         if events: events[3].record()
@@ -512,7 +530,8 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
             rows, st = opt.forward_keyed(q, out=row_bufs[0][:q.numel()], slot=0)
             rows = rows.clone()
             nxt = opt.prefetch_keyed(q, slot=1, out=row_bufs[1][:q.numel()])
-            res = opt.backward_keyed(st, g, m, fetched_rows="auto" if reuse_rows else None, join=False)
+            res = opt.backward_keyed(st, g, m, fetched_rows="auto" if reuse_rows else None, join=False,
+                                     average=average)
             rows2, _ = opt.finish_prefetch(nxt, after=st)
             torch.cuda.synchronize()
             want2 = ops.cached_fetch(opt.cold_w, opt.hot_w, q, opt.hot_set)
@@ -530,7 +549,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
 
     gate = None
     if with_gate:
-        gate = parity_gate(wl, gate_step)
+        gate = parity_gate(wl, gate_step, average=average, rows_are_sums=keyed)
         log("parity gate passed: %s" % json.dumps(gate["max_rel_err"]))
     link = link_probe(dev) if (with_link and wl.host_cold) else None
     if link:
@@ -1569,6 +1588,14 @@ def main():
                    "optimizer": ("SparseAdam lr=0.01 betas=(0.9, 0.999) eps=1e-8 (the reference's "
                                  "optimizer; the configurations name Adagrad)" if args.optimizer == "adam"
                                  else "sparse Adagrad lr=0.01 eps=1e-10"),
+                   "duplicate_ids": {None: "the update applies the SUM of an id's gradient rows",
+                                     "sum": "the update applies the SUM of an id's gradient rows",
+                                     "mean": "the update applies the MEAN of an id's gradient rows, as the "
+                                             "reference's update does (unique_grads)",
+                                     "one_plus": "the update applies the sum of an id's gradient rows over "
+                                                 "one plus its occurrences"}[
+                       args.average if args.average is not None else
+                       ("mean" if args.optimizer == "adam" else None)],
                    "schedule": {"serial": "one stream, hot and cold rows in the same kernels",
                                 "split": "lookup + hot/cold partition; hot rows on the main stream, "
                                          "cold rows on a second stream of the same priority",

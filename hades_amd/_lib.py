@@ -66,11 +66,12 @@ _SIGNATURES = {
     "hades_combine": [_P, _P, _L, _L, _L, c_int, _P, _P, _P, _P, _P, _P, c_size_t, _P],
     "hades_combine_plan_classed": [_P, _L, _L, _L, _L, _P, _P, _P, _P, _P, c_size_t, _P],
     "hades_combine_apply_class": [_P, _L, _L, _L, c_int, c_int, _P, _P, _P, _P, _P, c_size_t, _P],
-    "hades_adagrad_update_class": [_P, _P, _P, _P, c_int, _L, _L, _L, _P, _P, _L, _P, _P, c_float, c_float, _P],
+    "hades_adagrad_update_class": [_P, _P, _P, _P, c_int, _L, _L, _L, _P, _P, _L, _P, _P, _P, c_int,
+                                   c_float, c_float, _P],
     "hades_adagrad_update_class_summing": [_P, _P, _L, _L, _P, _P, c_int, _L, _L, _P, _P, _L, _P, _P, _P, _P,
-                                           c_float, c_float, _P, c_size_t, _P],
+                                           c_int, c_float, c_float, _P, c_size_t, _P],
     "hades_adam_update_class_summing": [_P, _P, _L, _L, _P, _P, c_int, _L, _L, _P, _P, _P, _P, _L, _P, _P,
-                                        _P, _P, c_float, ctypes.c_double, ctypes.c_double, c_float, _P,
+                                        _P, _P, c_int, c_float, ctypes.c_double, ctypes.c_double, c_float, _P,
                                         c_size_t, _P],
     "hades_combine_static": [_P, _P, _L, _L, _L, c_int, _P, _P, _P, _P, _P, _P],
     "hades_combine_plan": [_P, _L, _L, _L, _P, _P, _P, _P, c_size_t, _P],
@@ -81,7 +82,7 @@ _SIGNATURES = {
                           c_float, ctypes.c_double, ctypes.c_double, c_float, _P],
     "hades_adam_update_listed": [_P, _P, _P, _P, _L, _L, _P, _P, _P, _P, _L, c_float,
                                  ctypes.c_double, ctypes.c_double, c_float, _P],
-    "hades_adam_update_class": [_P, _P, _P, _P, c_int, _L, _L, _L, _P, _P, _P, _P, _L, _P, _P,
+    "hades_adam_update_class": [_P, _P, _P, _P, c_int, _L, _L, _L, _P, _P, _P, _P, _L, _P, _P, _P, c_int,
                                 c_float, ctypes.c_double, ctypes.c_double, c_float, _P],
     "hades_hash_clear": [_P, _P, _P, _L, _L, _P],
     "hades_hash_accumulate": [_P, _P, _P, _L, _P, _P, _P, _P, _L, _L, _P, _P],

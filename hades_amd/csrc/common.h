@@ -120,22 +120,25 @@ __device__ __forceinline__ int64_t lookup_slot_dev(const int64_t* __restrict__ a
 }
 
 // The hot-ID set as the kernels see it: the ascending ids, and optionally a bucket index over
-// them.  Index layout (uint32 words): [0] shift, [1] log2(buckets), [2] valid, [3] unused, then
-// table[buckets + 1] with table[b] = first position whose id >= (b << shift).  A lookup is then
-// one table read (two adjacent words) plus a search over the handful of ids of one bucket,
-// instead of log2(n) dependent probes.
+// them.  Index layout (uint32 words): [0] shift, [1] log2(buckets), [2] form, [3] unused, then the
+// bucket table; bucket b holds the ids with (id >> shift) == b.
+//   form 1: table[b] (one word) = first position whose id >= (b << shift); a lookup reads two
+//           adjacent words and then searches the ids of the bucket: two dependent reads.
+//   form 2 (built whenever shift <= 24): table[b] (two words) = {first position, (count << 24) |
+//           the low `shift` bits of the bucket's first id}, count saturating at 255.  All ids of a
+//           bucket share their high bits, so the low bits identify the first id: a query that is
+//           the first id of its bucket, or falls into an empty bucket, or below the first id, or
+//           into a bucket of one, is answered from the one 8-byte entry - with about one bucket
+//           per hot id that is three queries in four - and only the rest go on to search the
+//           other ids of the bucket.
+//   form 0: no usable index (negative ids, or more than 2^32 - 1 of them): plain binary search.
 constexpr int kHotIndexHeader = 4;
 struct HotSet {
   const int64_t* sorted;
   int64_t n;
   const uint32_t* index;  // may be null
 
-  __device__ __forceinline__ int64_t slot(int64_t v) const {
-    if (index == nullptr || index[2] == 0u) return lookup_slot_dev(sorted, n, v);
-    if (v < 0) return -1;
-    const uint64_t b = static_cast<uint64_t>(v) >> index[0];
-    if (b >> index[1]) return -1;  // beyond the largest hot id
-    int64_t lo = index[kHotIndexHeader + b], hi = index[kHotIndexHeader + b + 1];
+  __device__ __forceinline__ int64_t search(int64_t lo, int64_t hi, int64_t v) const {
     while (lo < hi) {
       const int64_t mid = (lo + hi) >> 1;
       const int64_t x = sorted[mid];
@@ -143,6 +146,28 @@ struct HotSet {
       if (x < v) lo = mid + 1; else hi = mid;
     }
     return -1;
+  }
+
+  __device__ __forceinline__ int64_t slot(int64_t v) const {
+    if (index == nullptr || index[2] == 0u) return lookup_slot_dev(sorted, n, v);
+    if (v < 0) return -1;
+    const uint32_t shift = index[0];
+    const uint64_t b = static_cast<uint64_t>(v) >> shift;
+    if (b >> index[1]) return -1;  // beyond the largest hot id
+    if (index[2] == 2u) {
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2* table = reinterpret_cast<const u32x2*>(index + kHotIndexHeader);
+      const u32x2 e = table[b];
+      const uint32_t cnt = e.y >> 24;
+      if (cnt == 0u) return -1;
+      const uint32_t low = static_cast<uint32_t>(v) & ((1u << shift) - 1u);
+      const uint32_t first = e.y & 0xffffffu;
+      if (low == first) return e.x;
+      if (low < first || cnt == 1u) return -1;
+      const int64_t hi = cnt < 255u ? static_cast<int64_t>(e.x) + cnt : static_cast<int64_t>(table[b + 1].x);
+      return search(static_cast<int64_t>(e.x) + 1, hi, v);
+    }
+    return search(index[kHotIndexHeader + b], index[kHotIndexHeader + b + 1], v);
   }
 };
 

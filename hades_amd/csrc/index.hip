@@ -45,21 +45,32 @@ __global__ __launch_bounds__(kThreads) void lookup_sorted_kernel(const int64_t* 
 }
 
 // ---- bucket index over the sorted hot set ------------------------------------
-// header: shift such that (largest id >> shift) < buckets; valid only for non-negative ids
+// header: shift such that (largest id >> shift) < buckets; usable only for non-negative ids.
+// form 2 (position + count + low bits of the first id in one entry) when the low bits fit 24 bits.
 __global__ void hot_index_header_kernel(const int64_t* __restrict__ sorted, int64_t num_hot,
                                         int buckets_log2, uint32_t* __restrict__ index) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  uint32_t shift = 0, valid = 0;
+  uint32_t shift = 0, form = 0;
   if (num_hot > 0 && num_hot < (int64_t(1) << 32) && sorted[0] >= 0) {
     const uint64_t mx = static_cast<uint64_t>(sorted[num_hot - 1]);
     const int bits = mx == 0 ? 1 : 64 - __clzll(static_cast<long long>(mx));
     shift = bits > buckets_log2 ? static_cast<uint32_t>(bits - buckets_log2) : 0u;
-    valid = 1;
+    form = shift <= 24u ? 2u : 1u;
   }
   index[0] = shift;
   index[1] = static_cast<uint32_t>(buckets_log2);
-  index[2] = valid;
+  index[2] = form;
   index[3] = 0;
+}
+
+// first position whose id >= (b << shift), for b in [0, buckets]: ids are >= 0, so this is
+// upper_bound(key - 1) (the last entry closes the last bucket: every id is below buckets << shift)
+__device__ __forceinline__ int64_t bucket_start(const int64_t* __restrict__ sorted, int64_t num_hot,
+                                                int64_t b, int64_t buckets, uint32_t shift) {
+  if (b >= buckets) return num_hot;
+  const int64_t key = static_cast<int64_t>(static_cast<uint64_t>(b) << shift);
+  if (key <= 0) return 0;
+  return upper_bound_dev<int64_t>(sorted, num_hot, key - 1);
 }
 
 __global__ __launch_bounds__(kThreads) void hot_index_table_kernel(const int64_t* __restrict__ sorted,
@@ -68,18 +79,21 @@ __global__ __launch_bounds__(kThreads) void hot_index_table_kernel(const int64_t
   const int64_t b = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   const int64_t buckets = int64_t(1) << index[1];
   if (b > buckets) return;
-  if (index[2] == 0u) {
+  const uint32_t form = index[2], shift = index[0];
+  if (form == 0u) {
     index[kHotIndexHeader + b] = 0;
     return;
   }
-  // first position whose id >= (b << shift): ids are >= 0, so this is upper_bound(key - 1)
-  // (the last entry closes the last bucket: every id is below buckets << shift)
-  const int64_t key = static_cast<int64_t>(static_cast<uint64_t>(b) << index[0]);
-  int64_t pos;
-  if (b == buckets) pos = num_hot;
-  else if (key <= 0) pos = 0;
-  else pos = upper_bound_dev<int64_t>(sorted, num_hot, key - 1);
-  index[kHotIndexHeader + b] = static_cast<uint32_t>(pos);
+  const int64_t pos = bucket_start(sorted, num_hot, b, buckets, shift);
+  if (form == 1u) {
+    index[kHotIndexHeader + b] = static_cast<uint32_t>(pos);
+    return;
+  }
+  const int64_t next = bucket_start(sorted, num_hot, b + 1, buckets, shift);
+  const int64_t cnt = next - pos;
+  const uint32_t low = cnt > 0 ? static_cast<uint32_t>(sorted[pos]) & ((1u << shift) - 1u) : 0u;
+  index[kHotIndexHeader + 2 * b] = static_cast<uint32_t>(pos);
+  index[kHotIndexHeader + 2 * b + 1] = (static_cast<uint32_t>(cnt < 255 ? cnt : 255) << 24) | low;
 }
 
 int hot_index_buckets_log2(int64_t num_hot) {
@@ -457,7 +471,7 @@ int hades_lookup_sorted(const int64_t* q, int64_t n, const int64_t* sorted_hot, 
 size_t hades_hot_index_bytes(int64_t num_hot) {
   if (num_hot < 0) return 0;
   const int64_t buckets = int64_t(1) << hot_index_buckets_log2(num_hot);
-  return static_cast<size_t>(kHotIndexHeader + buckets + 1) * sizeof(uint32_t);
+  return static_cast<size_t>(kHotIndexHeader + 2 * (buckets + 1)) * sizeof(uint32_t);   // form 2
 }
 
 int hades_hot_index_build(const int64_t* sorted_hot, int64_t num_hot, void* hot_index,

@@ -156,6 +156,12 @@ struct ListedRows {
   const uint32_t* seg_start = nullptr;
   float* sums_out = nullptr;
   int64_t* cnts_out = nullptr;
+  // Averaging (unique_grads, python/EmbCache/sparse_optim.py:142-157): the gradient of a row is
+  // divided by its number of occurrences (average = 1) or by one more than that (average = 2:
+  // the reference's count starts from ones when counts come with the rows, :145-148) before the
+  // update.  The occurrences are the run length (summing form) or run_cnts[p].
+  int average = 0;
+  const int64_t* run_cnts = nullptr;
 };
 
 struct AdagradListedArgs {
@@ -197,19 +203,23 @@ __device__ __forceinline__ void listed_range(const ListedRows& a, int64_t* first
 template <bool SUMMING>
 __device__ __forceinline__ void resolve_listed(const ListedRows& a, int64_t row0, int rows_here,
                                                int64_t* s_tab, int64_t* s_grad, int64_t* s_old,
-                                               uint32_t* s_j0, uint32_t* s_len) {
+                                               uint32_t* s_j0, uint32_t* s_len, float* s_div) {
   for (int r = threadIdx.x; r < rows_here; r += kThreads) {
     const int64_t p = a.list != nullptr ? a.list[row0 + r] : row0 + r;
     s_tab[r] = a.row_index[p] & a.index_mask;
+    int64_t occurrences = 1;
     if (SUMMING) {
       const uint32_t j0 = a.seg_start[p], j1 = a.seg_start[p + 1];
       s_j0[r] = j0;
       s_len[r] = j1 - j0;
       s_grad[r] = static_cast<int64_t>(a.perm[j0]) * a.dim;   // the run's first gradient row
       if (a.cnts_out != nullptr) a.cnts_out[p] = static_cast<int64_t>(j1 - j0);
+      occurrences = j1 - j0;
     } else {
       s_grad[r] = p * a.dim;
+      if (a.average != 0) occurrences = a.run_cnts[p];
     }
+    if (a.average != 0) s_div[r] = static_cast<float>(occurrences + (a.average == 2 ? 1 : 0));
     if (a.w_rows != nullptr) s_old[r] = static_cast<int64_t>(a.first_pos[p]) * a.dim;
   }
 }
@@ -243,6 +253,7 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
   __shared__ int64_t s_old[kRows];
   __shared__ uint32_t s_j0[kRows];
   __shared__ uint32_t s_len[kRows];
+  __shared__ float s_div[kRows];
   int64_t first, cnt;
   listed_range(a.r, &first, &cnt);
   const int cpr = static_cast<int>(a.r.dim / VEC);
@@ -250,7 +261,7 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
        row0 += static_cast<int64_t>(gridDim.x) * kRows) {
     const int64_t left = cnt - row0;
     const int rows_here = left < kRows ? static_cast<int>(left) : kRows;
-    resolve_listed<SUMMING>(a.r, row0, rows_here, s_tab, s_grad, s_old, s_j0, s_len);
+    resolve_listed<SUMMING>(a.r, row0, rows_here, s_tab, s_grad, s_old, s_j0, s_len, s_div);
     __syncthreads();
     const int total = rows_here * cpr;
     for (int base = threadIdx.x; base < total; base += kThreads * kUnroll) {
@@ -285,6 +296,7 @@ __global__ __launch_bounds__(kThreads) void adagrad_listed_kernel(AdagradListedA
             if (a.r.sums_out != nullptr)
               *reinterpret_cast<V*>(a.r.sums_out + (row0 + r) * a.r.dim + col) = acc;
           }
+          if (a.r.average != 0) g[k] = vdiv(g[k], V(s_div[r]));
           const V s1 = s[k] + g[k] * g[k];
           const V std_ = vsqrt(s1) + a.eps;
           const V w1 = w[k] - vdiv(a.lr * g[k], std_);
@@ -307,6 +319,7 @@ __global__ __launch_bounds__(kThreads) void adam_listed_kernel(AdamListedArgs a)
   __shared__ int64_t s_old[kRows];
   __shared__ uint32_t s_j0[kRows];
   __shared__ uint32_t s_len[kRows];
+  __shared__ float s_div[kRows];
   __shared__ float s_c1[kRows];
   __shared__ float s_c2[kRows];
   int64_t first, cnt;
@@ -316,7 +329,7 @@ __global__ __launch_bounds__(kThreads) void adam_listed_kernel(AdamListedArgs a)
        row0 += static_cast<int64_t>(gridDim.x) * kRows) {
     const int64_t left = cnt - row0;
     const int rows_here = left < kRows ? static_cast<int>(left) : kRows;
-    resolve_listed<SUMMING>(a.r, row0, rows_here, s_tab, s_grad, s_old, s_j0, s_len);
+    resolve_listed<SUMMING>(a.r, row0, rows_here, s_tab, s_grad, s_old, s_j0, s_len, s_div);
     // thread r wrote s_tab[r] itself: the step counter and the bias corrections of its row
     for (int r = threadIdx.x; r < rows_here; r += kThreads) {
       float* sp = a.step + s_tab[r];
@@ -356,8 +369,8 @@ __global__ __launch_bounds__(kThreads) void adam_listed_kernel(AdamListedArgs a)
       for (int k = 0; k < kUnroll; ++k) {
         const int c = base + k * kThreads;
         if (c < total) {
+          const int r = c / cpr;
           if (SUMMING) {
-            const int r = c / cpr;
             const int64_t col = static_cast<int64_t>(c - r * cpr) * VEC;
             V acc = V(0.0f) + g[k];
             if (s_len[r] > 1) acc = add_rest_of_run<V>(a.r, s_j0[r], s_len[r], col, acc);
@@ -365,6 +378,7 @@ __global__ __launch_bounds__(kThreads) void adam_listed_kernel(AdamListedArgs a)
             if (a.r.sums_out != nullptr)
               *reinterpret_cast<V*>(a.r.sums_out + (row0 + r) * a.r.dim + col) = acc;
           }
+          if (a.r.average != 0) g[k] = vdiv(g[k], V(s_div[r]));
           const V m1 = a.beta1 * m[k] + a.one_minus_beta1 * g[k];
           const V v1 = a.beta2 * v[k] + a.one_minus_beta2 * (g[k] * g[k]);
           const V mc = vdiv(m1, V(c1[k]));
@@ -479,6 +493,9 @@ int check_listed(const ListedRows& r, bool class_form) {
   HADES_REQUIRE(r.dim * kRows < (int64_t(1) << 30), "dim too large");
   if (r.max_count == 0) return HADES_OK;
   HADES_REQUIRE(r.row_index && r.grad, "null pointer argument");
+  HADES_REQUIRE(r.average >= 0 && r.average <= 2, "average must be 0, 1 or 2");
+  HADES_REQUIRE(r.average == 0 || r.perm != nullptr || r.run_cnts != nullptr,
+                "averaging needs the occurrence counts of the rows (run_cnts)");
   if (class_form) {
     HADES_REQUIRE(r.which == 0 || r.which == 1, "which must be 0 or 1");
     HADES_REQUIRE(r.num_unique && r.class_split, "null pointer argument");
@@ -573,11 +590,14 @@ int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, con
 int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
                                const int64_t* class_split, int which, int64_t key_mask,
                                int64_t max_rows, int64_t dim, float* w, float* s, int64_t stride,
-                               const float* w_rows, const int32_t* first_pos, float lr, float eps,
+                               const float* w_rows, const int32_t* first_pos,
+                               const int64_t* run_cnts, int average, float lr, float eps,
                                void* stream) {
   HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
-  const ListedRows r{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
-                     key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  ListedRows r{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
+               key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  r.average = average;
+  r.run_cnts = run_cnts;
   const int rc = check_listed(r, true);
   if (rc != HADES_OK || max_rows == 0) return rc;
   HADES_REQUIRE(w && s, "null pointer argument");
@@ -589,18 +609,20 @@ int hades_adagrad_update_class_summing(const int64_t* ukeys, const float* grad_r
                                        const int64_t* class_split, int which, int64_t key_mask,
                                        int64_t dim, float* w, float* s, int64_t stride,
                                        const float* w_rows, const int32_t* first_pos,
-                                       float* sums_out, int64_t* cnts_out, float lr, float eps,
-                                       void* workspace, size_t workspace_bytes, void* stream) {
+                                       float* sums_out, int64_t* cnts_out, int average, float lr,
+                                       float eps, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
   HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
   HADES_REQUIRE(n >= 0, "n must be >= 0");
   if (n == 0) return HADES_OK;
   ListedRows r{ukeys, grad_rows, nullptr, nullptr, n, num_unique, class_split, which,
                key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  r.average = average;
+  const int rv = combine_plan_views(workspace, workspace_bytes, n, dim, key_bound, &r.perm, &r.seg_start);
+  if (rv != HADES_OK) return rv;
   const int rc = check_listed(r, true);
   if (rc != HADES_OK) return rc;
   HADES_REQUIRE(w && s, "null pointer argument");
-  const int rv = combine_plan_views(workspace, workspace_bytes, n, dim, key_bound, &r.perm, &r.seg_start);
-  if (rv != HADES_OK) return rv;
   r.sums_out = sums_out;
   r.cnts_out = cnts_out;
   return launch_adagrad_listed(AdagradListedArgs{r, w, s, nullptr, lr, eps}, stream);
@@ -611,19 +633,20 @@ int hades_adam_update_class_summing(const int64_t* ukeys, const float* grad_rows
                                     const int64_t* class_split, int which, int64_t key_mask,
                                     int64_t dim, float* w, float* step, float* m, float* v,
                                     int64_t stride, const float* w_rows, const int32_t* first_pos,
-                                    float* sums_out, int64_t* cnts_out, float lr, double beta1,
-                                    double beta2, float eps, void* workspace,
+                                    float* sums_out, int64_t* cnts_out, int average, float lr,
+                                    double beta1, double beta2, float eps, void* workspace,
                                     size_t workspace_bytes, void* stream) {
   HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
   HADES_REQUIRE(n >= 0, "n must be >= 0");
   if (n == 0) return HADES_OK;
   ListedRows r{ukeys, grad_rows, nullptr, nullptr, n, num_unique, class_split, which,
                key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  r.average = average;
+  const int rv = combine_plan_views(workspace, workspace_bytes, n, dim, key_bound, &r.perm, &r.seg_start);
+  if (rv != HADES_OK) return rv;
   const int rc = check_listed(r, true);
   if (rc != HADES_OK) return rc;
   HADES_REQUIRE(w && step && m && v, "null pointer argument");
-  const int rv = combine_plan_views(workspace, workspace_bytes, n, dim, key_bound, &r.perm, &r.seg_start);
-  if (rv != HADES_OK) return rv;
   r.sums_out = sums_out;
   r.cnts_out = cnts_out;
   return launch_adam_listed(r, w, step, m, v, lr, beta1, beta2, eps, stream);
@@ -646,11 +669,13 @@ int hades_adam_update_class(const int64_t* ukeys, const float* grad, const int64
                             const int64_t* class_split, int which, int64_t key_mask,
                             int64_t max_rows, int64_t dim, float* w, float* step, float* m,
                             float* v, int64_t stride, const float* w_rows,
-                            const int32_t* first_pos, float lr, double beta1, double beta2,
-                            float eps, void* stream) {
+                            const int32_t* first_pos, const int64_t* run_cnts, int average,
+                            float lr, double beta1, double beta2, float eps, void* stream) {
   HADES_REQUIRE(stride >= 0, "stride must be 0 or >= dim");
-  const ListedRows r{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
-                     key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  ListedRows r{ukeys, grad, nullptr, nullptr, max_rows, num_unique, class_split, which,
+               key_mask, w_rows, first_pos, dim, stride == 0 ? dim : stride};
+  r.average = average;
+  r.run_cnts = run_cnts;
   const int rc = check_listed(r, true);
   if (rc != HADES_OK || max_rows == 0) return rc;
   HADES_REQUIRE(w && step && m && v, "null pointer argument");

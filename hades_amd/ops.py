@@ -562,8 +562,16 @@ def _summing_outputs(plan, grad_rows, out):
     return sums, cnts, plan.check_live()
 
 
+AVERAGE = {None: 0, "sum": 0, "mean": 1, "one_plus": 2}
+
+
+def _average_code(average):
+    _check(average in AVERAGE, "average must be None, 'mean' or 'one_plus'")
+    return AVERAGE[average]
+
+
 def adagrad_update_class_(plan, sums, which, w, s, lr, eps, fetched_rows=None, grad_rows=None,
-                          out=None):
+                          out=None, average=None, cnts=None):
     """Sparse Adagrad over one class of a classed plan: the table row of run u is
     plan.uids[u] & (2^key_bits - 1) - the id for the cold class, the slot for the hot class.
     `fetched_rows` (float32[n, D], the rows the forward pass fetched for this batch) makes the
@@ -572,7 +580,14 @@ def adagrad_update_class_(plan, sums, which, w, s, lr, eps, fetched_rows=None, g
     With `grad_rows` (float32[n, D], one gradient row per query; `sums` is then ignored and may be
     None) the kernel sums the rows of every run itself, in occurrence order from +0.0 - the
     deterministic-order sum - instead of reading them from `sums`; `out` = (sums, cnts) then
-    receives the summed rows and counts of the class."""
+    receives the summed rows and counts of the class.
+    `average` = "mean" divides every row by its number of occurrences before the update
+    (unique_grads, python/EmbCache/sparse_optim.py:150-156), "one_plus" by one more (:145-148);
+    without grad_rows the occurrences come from `cnts` (the counts combine_apply_class wrote)."""
+    avg = _average_code(average)
+    if avg and grad_rows is None:
+        _check(cnts is not None, "averaging needs cnts")
+        _i64(cnts, "cnts")
     dim = plan.dim if grad_rows is not None else sums.size(1)
     for name, t in (("w", w), ("s", s)):
         _dev_or_pinned(t, name, contiguous=False)
@@ -585,18 +600,24 @@ def adagrad_update_class_(plan, sums, which, w, s, lr, eps, fetched_rows=None, g
         _lib.call("hades_adagrad_update_class_summing", _ptr(plan.uids), _ptr(grad_rows), plan.n,
                   plan.id_bound, _ptr(plan.num_unique), _ptr(plan.class_split), int(which),
                   (1 << plan.key_bits) - 1, dim, _ptr(w), _ptr(s), stride, _opt(fetched_rows), _opt(fp),
-                  _opt(so), _opt(co), float(lr), float(eps), _ptr(ws), ws.numel(), _stream())
+                  _opt(so), _opt(co), avg, float(lr), float(eps), _ptr(ws), ws.numel(), _stream())
         return
     _dev(sums, "sums")
     _lib.call("hades_adagrad_update_class", _ptr(plan.uids), _ptr(sums), _ptr(plan.num_unique),
               _ptr(plan.class_split), int(which), (1 << plan.key_bits) - 1, plan.uids.numel(), dim,
-              _ptr(w), _ptr(s), stride, _opt(fetched_rows), _opt(fp), float(lr), float(eps), _stream())
+              _ptr(w), _ptr(s), stride, _opt(fetched_rows), _opt(fp), _opt(cnts if avg else None), avg,
+              float(lr), float(eps), _stream())
 
 
 def adam_update_class_(plan, sums, which, tables, lr, beta1, beta2, eps, fetched_rows=None,
-                       grad_rows=None, out=None):
-    """SparseAdam over one class of a classed plan; rows, `fetched_rows`, `grad_rows` and `out` as
-    in adagrad_update_class_, `tables` = (w, step, mem, power) of that class."""
+                       grad_rows=None, out=None, average=None, cnts=None):
+    """SparseAdam over one class of a classed plan; rows, `fetched_rows`, `grad_rows`, `out`,
+    `average` and `cnts` as in adagrad_update_class_, `tables` = (w, step, mem, power) of that
+    class."""
+    avg = _average_code(average)
+    if avg and grad_rows is None:
+        _check(cnts is not None, "averaging needs cnts")
+        _i64(cnts, "cnts")
     dim = plan.dim if grad_rows is not None else sums.size(1)
     stride = _adam_tables(tables, dim)
     w, step, m, v = tables
@@ -606,14 +627,15 @@ def adam_update_class_(plan, sums, which, tables, lr, beta1, beta2, eps, fetched
         _lib.call("hades_adam_update_class_summing", _ptr(plan.uids), _ptr(grad_rows), plan.n,
                   plan.id_bound, _ptr(plan.num_unique), _ptr(plan.class_split), int(which),
                   (1 << plan.key_bits) - 1, dim, _ptr(w), _ptr(step), _ptr(m), _ptr(v), stride,
-                  _opt(fetched_rows), _opt(fp), _opt(so), _opt(co), float(lr), float(beta1),
+                  _opt(fetched_rows), _opt(fp), _opt(so), _opt(co), avg, float(lr), float(beta1),
                   float(beta2), float(eps), _ptr(ws), ws.numel(), _stream())
         return
     _dev(sums, "sums")
     _lib.call("hades_adam_update_class", _ptr(plan.uids), _ptr(sums), _ptr(plan.num_unique),
               _ptr(plan.class_split), int(which), (1 << plan.key_bits) - 1, plan.uids.numel(), dim,
               _ptr(w), _ptr(step), _ptr(m), _ptr(v), stride, _opt(fetched_rows), _opt(fp),
-              float(lr), float(beta1), float(beta2), float(eps), _stream())
+              _opt(cnts if avg else None), avg, float(lr), float(beta1), float(beta2), float(eps),
+              _stream())
 
 
 def combine(idx, grad, id_bound=0, mode=COMBINE_FAST, workspace=None):

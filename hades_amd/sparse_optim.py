@@ -305,13 +305,20 @@ class _SparseRowOptimizer:
     def _update_class(self, index, grad, pos, count, hot):
         raise NotImplementedError
 
-    def update_split(self, uids, grad, num_unique=None, join=True, timing=None):
+    def update_split(self, uids, grad, num_unique=None, join=True, timing=None, cnts=None,
+                     average=None):
         """The row update over a combined batch as lookup -> partition -> one update kernel per
         class, hot on the current stream and cold on the cold stream ("hot_update" /
-        "cold_update" in `timing`)."""
+        "cold_update" in `timing`).  `average` = "mean" / "one_plus" with `cnts` (the combine's
+        counts) divides the rows of `grad` in place by their counts (plus one) first: the
+        reference's unique_grads (python/EmbCache/sparse_optim.py:142-157)."""
         cold = self._split_state()
         cur = torch.cuda.current_stream()
         n = uids.numel()
+        if ops._average_code(average):
+            if cnts is None:
+                raise RuntimeError("update_split(average=...) needs the combine's cnts")
+            ops.rows_div_count_(grad, cnts, num_unique, one_plus=average == "one_plus")
         loc, hot_pos, cold_pos, counts = ops.lookup_split(
             uids, self.hot_set, num_live=num_unique, workspace=self._split_ws,
             out=self._split_out("update", n))
@@ -483,7 +490,7 @@ class _SparseRowOptimizer:
         return out, (p["plan"], p["bufs"])
 
     def backward_keyed(self, state, grad, mode=ops.COMBINE_FAST, timing=None, fetched_rows="auto",
-                       join=True):
+                       join=True, average=None):
         """Backward half: segmented sums of the cold class, whose update then starts on the cold
         stream while the hot class is summed and updated on the current stream; joins at the end.
         Returns (ukeys, sums, cnts, num_unique, class_split): the distinct rows in class order -
@@ -497,6 +504,14 @@ class _SparseRowOptimizer:
         and the optimizer was not constructed with reuse_fetched_rows=False; otherwise the table
         is read again.  Either way the result is the same bit for bit.  None always reads the
         table; a tensor is taken as the rows on the caller's word.
+
+        `average`: None applies the per-id SUMS of the gradient rows (the combine of the
+        benchmark configurations); "mean" divides every id's sum by its number of occurrences
+        first, which is what the reference's update does with duplicate ids (unique_grads,
+        python/EmbCache/sparse_optim.py:142-157,613); "one_plus" divides by one more than that
+        (the reference's divisor when every row arrives with a count of one, :145-148).  The
+        division happens inside the update kernels; the returned rows stay the sums and `cnts`
+        the occurrences.
 
         join=False returns without making the current stream wait for the cold update; the caller
         then calls finish_prefetch(...) or join() before it reads the cold table on that stream."""
@@ -532,7 +547,7 @@ class _SparseRowOptimizer:
             self._timed(timing, "cold_update", cold,
                         lambda: self._update_keyed(plan, out[0], 0, fetched_rows,
                                                    grad_rows=grad if self.fuse_cold_sums else None,
-                                                   out=out))
+                                                   out=out, average=average))
             self._cold_done = torch.cuda.Event()
             self._cold_done.record(cold)
         if narrow:
@@ -540,12 +555,14 @@ class _SparseRowOptimizer:
         self._timed(timing, "seg_sum", cur,
                     lambda: ops.combine_apply_class(plan, grad, 1, mode, out=out))
         if self.hot_ids.numel():
-            self._timed(timing, "hot_update", cur, lambda: self._update_keyed(plan, out[0], 1))
+            self._timed(timing, "hot_update", cur,
+                        lambda: self._update_keyed(plan, out[0], 1, out=out, average=average))
         if join:        # join=False: finish_prefetch (or join()) waits for the cold update later
             self.join()
         return plan.uids, out[0], out[1], plan.num_unique, plan.class_split
 
-    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None):
+    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None,
+                      average=None):
         raise NotImplementedError
 
     def distinct_ids_of(self, ukeys, num_unique, key_bits=None):
@@ -561,14 +578,14 @@ class _SparseRowOptimizer:
         ids[hot] = self.hot_ids[k[hot] - (1 << kb)]
         return ids
 
-    def step_split(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None):
-        """step() on the split schedule."""
+    def step_split(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None, average=None):
+        """step() on the split schedule; with `average` the returned rows are the averaged ones."""
         if plan is None:
             plan = ops.combine_plan(idx, self.dim, id_bound=self.num_rows, workspace=self._ws)
         else:
             torch.cuda.current_stream().wait_event(plan.ready)
         uids, sums, cnts, nu = ops.combine_apply(plan, grad, mode, out=out)
-        self.update_split(uids, sums, nu)
+        self.update_split(uids, sums, nu, cnts=cnts, average=average)
         return uids, sums, cnts, nu
 
     def step(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None):
@@ -610,10 +627,12 @@ class SparseAdagrad(_SparseRowOptimizer):
         w, s = (self.hot_w, self.hot_s) if hot else (self.cold_w, self.cold_s)
         ops.adagrad_update_listed_(index, grad, pos, count, w, s, self.lr, self.eps)
 
-    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None):
+    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None,
+                      average=None):
         w, s = (self.hot_w, self.hot_s) if which else (self.cold_w, self.cold_s)
         ops.adagrad_update_class_(plan, sums, which, w, s, self.lr, self.eps, fetched_rows=fetched_rows,
-                                  grad_rows=grad_rows, out=out)
+                                  grad_rows=grad_rows, out=out if grad_rows is not None else None,
+                                  average=average, cnts=out[1] if out is not None else None)
 
     def update(self, uids, grad, num_unique=None):
         self._epoch += 1
@@ -644,10 +663,12 @@ class SparseAdam(_SparseRowOptimizer):
         ops.adam_update_listed_(index, grad, pos, count, self._tables(hot), self.lr,
                                 self.betas[0], self.betas[1], self.eps)
 
-    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None):
+    def _update_keyed(self, plan, sums, which, fetched_rows=None, grad_rows=None, out=None,
+                      average=None):
         ops.adam_update_class_(plan, sums, which, self._tables(bool(which)), self.lr,
                                self.betas[0], self.betas[1], self.eps, fetched_rows=fetched_rows,
-                               grad_rows=grad_rows, out=out)
+                               grad_rows=grad_rows, out=out if grad_rows is not None else None,
+                               average=average, cnts=out[1] if out is not None else None)
 
     def update(self, uids, grad, num_unique=None):
         self._epoch += 1

@@ -181,11 +181,13 @@ int hades_split(const void* ids, int id_type, const int8_t* class_table, int64_t
 int hades_lookup_sorted(const int64_t* q, int64_t n, const int64_t* sorted_hot, int64_t num_hot,
                         const void* hot_index, int64_t* loc, void* stream);
 
-/* Optional bucket index over the hot set: table[b] = first position whose id >= (b << shift), with
- * about one bucket per hot id.  With it a lookup is one table read plus a search over the few ids
- * of one bucket instead of log2(num_hot) dependent probes of the sorted array; results are
+/* Optional bucket index over the hot set, about one bucket per hot id: an entry holds the first
+ * position of its bucket in sorted_hot, the number of ids in it and the low bits of its first id,
+ * so that a lookup is ONE 8-byte read for three queries in four (the query is the bucket's first
+ * id, or the bucket is empty, or has one id) and one more search over the few ids of the bucket
+ * for the rest, instead of log2(num_hot) dependent probes of the sorted array; results are
  * identical.  Build it once per hot set (the reference builds its dense index_map once per cache,
- * python/EmbCache/cache.py:163-171; this takes 4 bytes per hot id instead of 8 per table row) and
+ * python/EmbCache/cache.py:163-171; this takes 8 - 16 bytes per hot id instead of 8 per table row) and
  * pass it as `hot_index` to the operators below; NULL there means plain binary search.  The
  * buffer is device memory, 16-byte aligned, hades_hot_index_bytes(num_hot) bytes. */
 size_t hades_hot_index_bytes(int64_t num_hot);
@@ -415,11 +417,16 @@ int hades_adagrad_update_listed(const int64_t* row_index, const float* grad, con
  * cold table in host memory this halves what the update moves over the link.  Only valid while
  * nothing has written those table rows since they were fetched (one batch in flight per table:
  * the reference's trainers are of that kind, python/EmbCache/sparse_optim.py:590-685 runs between
- * a batch's forward and the next one's). */
+ * a batch's forward and the next one's).
+ * average: 0 the rows of grad are applied as they are (sums); 1 row u is divided by run_cnts[u], its
+ * number of occurrences, first (the mean of unique_grads, python/EmbCache/sparse_optim.py:150-156);
+ * 2 by run_cnts[u] + 1 (the reference's count starts from ones when counts come with the rows,
+ * :145-148).  run_cnts (int64, the cnts of hades_combine_apply_class) may be NULL when average is 0. */
 int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const int64_t* num_unique,
                                const int64_t* class_split, int which, int64_t key_mask,
                                int64_t max_rows, int64_t dim, float* w, float* s, int64_t stride,
-                               const float* w_rows, const int32_t* first_pos, float lr, float eps,
+                               const float* w_rows, const int32_t* first_pos,
+                               const int64_t* run_cnts, int average, float lr, float eps,
                                void* stream);
 
 /* hades_adagrad_update_class with the segmented sum of its class folded in: grad_rows holds one
@@ -431,14 +438,17 @@ int hades_adagrad_update_class(const int64_t* ukeys, const float* grad, const in
  * cold class: nearly every cold id occurs once per batch), where it saves the segmented-sum launches
  * in front of an update that is bound by the host link anyway; a run of thousands of rows is walked
  * by one lane group and takes accordingly long.  sums_out (float[n, dim]) and cnts_out (int64[n]),
- * both optional, receive the summed row and the number of occurrences of every run of the class. */
+ * both optional, receive the summed row and the number of occurrences of every run of the class.
+ * average as in hades_adagrad_update_class, with the run length as the number of occurrences (the
+ * division happens after sums_out is written: sums_out keeps the sums). */
 int hades_adagrad_update_class_summing(const int64_t* ukeys, const float* grad_rows, int64_t n,
                                        int64_t key_bound, const int64_t* num_unique,
                                        const int64_t* class_split, int which, int64_t key_mask,
                                        int64_t dim, float* w, float* s, int64_t stride,
                                        const float* w_rows, const int32_t* first_pos,
-                                       float* sums_out, int64_t* cnts_out, float lr, float eps,
-                                       void* workspace, size_t workspace_bytes, void* stream);
+                                       float* sums_out, int64_t* cnts_out, int average, float lr,
+                                       float eps, void* workspace, size_t workspace_bytes,
+                                       void* stream);
 
 /* SparseAdam row update, same fusion (python/EmbCache/sparse_optim.py:632-657,681):
  *   step += 1; m = b1*m + (1-b1)*g; v = b2*v + (1-b2)*g*g
@@ -467,8 +477,8 @@ int hades_adam_update_class(const int64_t* ukeys, const float* grad, const int64
                             const int64_t* class_split, int which, int64_t key_mask,
                             int64_t max_rows, int64_t dim, float* w, float* step, float* m,
                             float* v, int64_t stride, const float* w_rows,
-                            const int32_t* first_pos, float lr, double beta1, double beta2,
-                            float eps, void* stream);
+                            const int32_t* first_pos, const int64_t* run_cnts, int average,
+                            float lr, double beta1, double beta2, float eps, void* stream);
 
 /* SparseAdam over one class with the segmented sum folded in; arguments as in
  * hades_adagrad_update_class_summing, tables as in hades_adam_update_listed. */
@@ -477,8 +487,8 @@ int hades_adam_update_class_summing(const int64_t* ukeys, const float* grad_rows
                                     const int64_t* class_split, int which, int64_t key_mask,
                                     int64_t dim, float* w, float* step, float* m, float* v,
                                     int64_t stride, const float* w_rows, const int32_t* first_pos,
-                                    float* sums_out, int64_t* cnts_out, float lr, double beta1,
-                                    double beta2, float eps, void* workspace,
+                                    float* sums_out, int64_t* cnts_out, int average, float lr,
+                                    double beta1, double beta2, float eps, void* workspace,
                                     size_t workspace_bytes, void* stream);
 
 /* Cold-gradient accumulator (delayed synchronisation): an open-addressing hash table in HBM,

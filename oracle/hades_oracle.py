@@ -306,8 +306,19 @@ def class_ordered_keys(q, sorted_hot, key_bits):
     return np.where(loc >= 0, (np.int64(1) << np.int64(key_bits)) | loc, q).astype(np.int64)
 
 
+def averaged(sums, cnts, average):
+    """The division of unique_grads (python/EmbCache/sparse_optim.py:142-157): per-id sums over
+    their occurrence counts ("mean", :150-156), or over one more ("one_plus": with a count vector
+    of ones the reference's divisor is 1 + the occurrences, :145-148), in float32 as torch does
+    it (float32 tensor / int64 tensor).  None returns the sums."""
+    if average in (None, "sum"):
+        return sums
+    div = cnts.astype(np.int64) + (1 if average == "one_plus" else 0)
+    return (sums / div.astype(np.float32)[:, None]).astype(np.float32)
+
+
 def keyed_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps, key_bits,
-               fetched_rows=None):
+               fetched_rows=None, average=None):
     """One combine + Adagrad step done the keyed way: combine over the class-ordered keys
     (only_unique_grads arithmetic, python/EmbCache/sparse_optim.py:132-139, on another key), then
     the cold runs update the cold tables at row = key and the hot runs the hot tables at row =
@@ -317,6 +328,7 @@ def keyed_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps, key_b
     Returns (ukeys, sums, cnts, first hot run)."""
     keys = class_ordered_keys(q, sorted_hot, key_bits)
     ukeys, sums, cnts = combine_sequential(keys, grad)
+    applied = averaged(sums, cnts, average)
     thr = np.int64(1) << np.int64(key_bits)
     split = int(np.searchsorted(ukeys, thr, side="left"))
     rows = ukeys[:split]
@@ -324,26 +336,27 @@ def keyed_step(cold_w, cold_s, hot_w, hot_s, sorted_hot, q, grad, lr, eps, key_b
     if fetched_rows is not None:
         first = np.array([np.flatnonzero(keys == k)[0] for k in rows], dtype=np.int64)
         old = np.asarray(fetched_rows)[first] if rows.size else old
-    w1, s1 = adagrad_rows(old, cold_s[rows], sums[:split], lr, eps)
+    w1, s1 = adagrad_rows(old, cold_s[rows], applied[:split], lr, eps)
     cold_w[rows], cold_s[rows] = w1, s1
     slots = ukeys[split:] - thr
-    w1, s1 = adagrad_rows(hot_w[slots], hot_s[slots], sums[split:], lr, eps)
+    w1, s1 = adagrad_rows(hot_w[slots], hot_s[slots], applied[split:], lr, eps)
     hot_w[slots], hot_s[slots] = w1, s1
     return ukeys, sums, cnts, split
 
 
 def keyed_step_adam(cold, hot, sorted_hot, q, grad, lr, beta1, beta2, eps, key_bits,
-                    fetched_rows=None):
+                    fetched_rows=None, average=None):
     """keyed_step with the reference's SparseAdam arithmetic (adam_rows) in place of Adagrad.
     `cold` and `hot` are (w, step, m, v) table sets, updated in place.  Must equal
     combine_sequential on the ids followed by adam_rows on the gathered rows of each id.
     Returns (ukeys, sums, cnts, first hot run)."""
     keys = class_ordered_keys(q, sorted_hot, key_bits)
     ukeys, sums, cnts = combine_sequential(keys, grad)
+    applied = averaged(sums, cnts, average)
     thr = np.int64(1) << np.int64(key_bits)
     split = int(np.searchsorted(ukeys, thr, side="left"))
-    for tabs, rows, g, is_cold in ((cold, ukeys[:split], sums[:split], True),
-                                   (hot, ukeys[split:] - thr, sums[split:], False)):
+    for tabs, rows, g, is_cold in ((cold, ukeys[:split], applied[:split], True),
+                                   (hot, ukeys[split:] - thr, applied[split:], False)):
         if rows.size == 0:
             continue
         w, step, m, v = tabs

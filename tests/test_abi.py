@@ -72,10 +72,23 @@ def test_argument_errors_of_the_split_schedule_entry_points():
     assert lib.hades_adagrad_update_listed(one, one, one, null, 10, 8, one, one, 0, null, 0.01, 1e-10, null) == 1
     assert lib.hades_adagrad_update_listed(null, null, null, null, 0, 8, null, null, 0, null, 0.01, 1e-10, null) == 0
     assert lib.hades_adagrad_update_class(one, one, one, one, 2, 255, 10, 8, one, one, 0, null, null,
-                                          0.01, 1e-10, null) == 1                              # which
+                                          null, 0, 0.01, 1e-10, null) == 1                     # which
     assert lib.hades_adagrad_update_class(one, one, one, one, 0, 255, 10, 8, one, one, 0, one, null,
-                                          0.01, 1e-10, null) == 1                              # rows without positions
+                                          null, 0, 0.01, 1e-10, null) == 1                     # rows without positions
     assert b"go together" in lib.hades_last_error()
+    assert lib.hades_adagrad_update_class(one, one, one, one, 0, 255, 10, 8, one, one, 0, null, null,
+                                          null, 1, 0.01, 1e-10, null) == 1                     # mean without counts
+    assert b"run_cnts" in lib.hades_last_error()
+    assert lib.hades_adagrad_update_class(one, one, one, one, 0, 255, 10, 8, one, one, 0, null, null,
+                                          one, 3, 0.01, 1e-10, null) == 1                      # average code
+    # the summing forms look for their plan in the workspace: too small a one is refused
+    assert lib.hades_adagrad_update_class_summing(one, one, 10, 1 << 20, one, one, 0, 255, 8, one, one, 0,
+                                                  null, null, null, null, 0, 0.01, 1e-10, one, 16, null) == 3
+    assert lib.hades_adam_update_class_summing(one, one, 10, 1 << 20, one, one, 0, 255, 8, one, one, one, one,
+                                               0, null, null, null, null, 0, 0.01, 0.9, 0.999, 1e-8, one, 16,
+                                               null) == 3
+    assert lib.hades_adagrad_update_class_summing(null, null, 0, 1 << 20, null, null, 0, 255, 8, null, null, 0,
+                                                  null, null, null, null, 0, 0.01, 1e-10, null, 0, null) == 0
     # listed gather restricted to a set
     assert lib.hades_fetch_listed_in_set(one, 4, one, one, one, 10, one, one, 5, one, 8, _lib.F32, null) == 1   # stride < dim
     assert lib.hades_fetch_listed_in_set(one, 0, one, one, one, 10, null, one, 5, one, 8, _lib.F32, null) == 1  # set is null
@@ -90,12 +103,12 @@ def test_argument_errors_of_the_split_schedule_entry_points():
     assert lib.hades_adam_update_listed(null, null, null, null, 0, 8, null, null, null, null, 0, 0.01, 0.9,
                                         0.999, 1e-8, null) == 0
     assert lib.hades_adam_update_class(one, one, one, one, 3, 255, 10, 8, one, one, one, one, 0, null, null,
-                                       0.01, 0.9, 0.999, 1e-8, null) == 1                      # which
+                                       null, 0, 0.01, 0.9, 0.999, 1e-8, null) == 1             # which
     assert lib.hades_adam_update_class(one, one, one, one, 1, 255, 10, 8, one, one, one, one, 0, null, one,
-                                       0.01, 0.9, 0.999, 1e-8, null) == 1
+                                       null, 0, 0.01, 0.9, 0.999, 1e-8, null) == 1
     assert b"go together" in lib.hades_last_error()
     assert lib.hades_adam_update_class(null, null, null, null, 0, 255, 0, 8, null, null, null, null, 0, null,
-                                       null, 0.01, 0.9, 0.999, 1e-8, null) == 0
+                                       null, null, 0, 0.01, 0.9, 0.999, 1e-8, null) == 0
     # lookup + split: key bits must leave room for the slots
     assert lib.hades_lookup_split(one, null, 10, one, 1 << 20, null, one, null, one, one, one, one, 8,
                                   one, 1 << 20, null) == 1

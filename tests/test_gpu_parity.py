@@ -1751,6 +1751,72 @@ def test_cold_update_that_sums_its_own_runs(lib, kind, host_cold, dim):
     assert combine_tol_ok(sums[:U].cpu().numpy(), w64)
 
 
+@pytest.mark.parametrize("kind", ["adagrad", "adam"])
+@pytest.mark.parametrize("average", ["mean", "one_plus"])
+@pytest.mark.parametrize("host_cold", [False, True])
+def test_keyed_and_split_steps_that_average_like_the_reference(lib, kind, average, host_cold):
+    """The reference's update averages duplicate ids before the row update (unique_grads,
+    python/EmbCache/sparse_optim.py:142-157,613).  backward_keyed(average=...) and
+    step_split(average=...) do the division on the device, inside the update kernels (keyed) or in
+    place on the combined rows (split): all tables bit-equal to the oracle's combine -> division ->
+    row update over three steps, with long runs in both classes and the summing cold update on
+    and off."""
+    _, ops = lib
+    from hades_amd.sparse_optim import SparseAdagrad, SparseAdam
+    rng = np.random.default_rng(303 + host_cold)
+    N, D, H, n = 30_000, 64, 3000, 24_000
+    cold, hot_ids, q = _split_case(rng, N, D, H, n, 0.6)
+    cold_ids = np.setdiff1d(np.arange(N, dtype=np.int64), hot_ids)
+    q[rng.choice(n, 700, replace=False)] = hot_ids[5]
+    q[rng.choice(n, 90, replace=False)] = cold_ids[7]
+    kb = ops.key_bits_for(N)
+    t_q = dev(q)
+
+    def make():
+        t = torch.from_numpy(cold.copy())
+        t = t.pin_memory() if host_cold else t.cuda()
+        return (SparseAdam if kind == "adam" else SparseAdagrad)(t, torch.from_numpy(hot_ids))
+
+    def tables(o):
+        ts = ((o.cold_w, o.cold_s, o.hot_w, o.hot_s) if kind == "adagrad" else
+              (o.cold_w, o.cold_step, o.cold_m, o.cold_v, o.hot_w, o.hot_step, o.hot_m, o.hot_v))
+        torch.cuda.synchronize()
+        return [t.cpu().numpy().copy() for t in ts]
+
+    keyed, unfused, split = make(), make(), make()
+    unfused.fuse_cold_sums = False
+    if kind == "adagrad":
+        want = [cold.copy(), np.zeros_like(cold), cold[hot_ids].copy(), np.zeros((H, D), np.float32)]
+    else:
+        z = lambda *sh: np.zeros(sh, np.float32)
+        want = [cold.copy(), z(N), z(N, D), z(N, D), cold[hot_ids].copy(), z(H), z(H, D), z(H, D)]
+    for it in range(3):
+        g = (rng.standard_normal((n, D)) * 1e-3).astype(np.float32)
+        t_g = dev(g)
+        for o in (keyed, unfused):
+            _, st = o.forward_keyed(t_q)
+            uk, sums, cnts, nu, _ = o.backward_keyed(st, t_g, mode=ops.COMBINE_EXACT, average=average)
+        split.step_split(t_q, t_g, mode=ops.COMBINE_EXACT, average=average)
+        if kind == "adagrad":
+            wk, ws, wc, _ = O.keyed_step(want[0], want[1], want[2], want[3], hot_ids, q, g, 0.01, 1e-10, kb,
+                                         average=average)
+        else:
+            wk, ws, wc, _ = O.keyed_step_adam(want[:4], want[4:], hot_ids, q, g, 0.01, 0.9, 0.999, 1e-8, kb,
+                                              average=average)
+        U = int(nu.item())
+        # the returned rows stay the sums, the counts the occurrences
+        assert np.array_equal(uk[:U].cpu().numpy(), wk) and np.array_equal(cnts[:U].cpu().numpy(), wc)
+        assert np.array_equal(sums[:U].cpu().numpy(), ws)
+    tk, tu, tsp = tables(keyed), tables(unfused), tables(split)
+    for a, b, c, w in zip(tk, tu, tsp, want):
+        assert np.array_equal(a, b) and np.array_equal(a, c)
+        if kind == "adagrad":
+            assert np.array_equal(a, w)
+    if kind == "adam":      # the oracle's Adam is pinned to 1e-4 of one update only (device powf)
+        for a, w in zip(tk, want):
+            assert np.allclose(a, w, rtol=0, atol=5e-6)
+
+
 def test_lookup_split_beyond_the_in_kernel_tile_sum(lib):
     """More than 4 096 tiles of queries: the per-tile counts are prefixed by a scan kernel of their
     own instead of being summed inside every compaction block.  Same lists, same slots."""

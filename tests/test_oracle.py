@@ -283,6 +283,41 @@ def test_unique_grads_mean_and_count_quirk():
     assert m.flatten().tolist() == [6.0 / 3, 9.0 / 4]
 
 
+def test_averaged_is_the_division_of_unique_grads():
+    """O.averaged restates the last line of unique_grads (python/EmbCache/sparse_optim.py:156)
+    on top of the sequential sums: pinned bit for bit by the reference's own torch code
+    (O.unique_grads: unique + index_add_ + division), for the plain mean and for the count that
+    starts from ones when a count vector of ones comes along (:145-148); and a keyed step with
+    `average` equals combine -> that division -> Adagrad on the ids."""
+    rng = np.random.default_rng(91)
+    n, D, N = 6000, 5, 900
+    q = np.minimum(rng.pareto(0.7, n).astype(np.int64) * 13 % N, N - 1)
+    g = (rng.standard_normal((n, D)) * 1e-2).astype(np.float32)
+    wu, ws, wc = O.combine_sequential(q, g)
+    assert wc.max() > 100                                    # divisors beyond small integers
+    tu, tm = O.unique_grads(torch.from_numpy(q), torch.from_numpy(g))
+    assert np.array_equal(tu.numpy(), wu) and np.array_equal(tm.numpy(), O.averaged(ws, wc, "mean"))
+    tu, tm = O.unique_grads(torch.from_numpy(q), torch.from_numpy(g), cnt=torch.ones(n, dtype=torch.int64))
+    assert np.array_equal(tm.numpy(), O.averaged(ws, wc, "one_plus"))
+    assert O.averaged(ws, wc, None) is ws
+    # closed forms: n copies of one row average to that row; a single occurrence is unchanged
+    row = g[:1]
+    same = O.averaged(*O.combine_sequential(np.zeros(64, np.int64), np.repeat(row, 64, 0))[1:], "mean")
+    assert np.allclose(same, row, rtol=1e-6) and np.array_equal(O.averaged(ws[wc == 1], wc[wc == 1], "mean"), ws[wc == 1])
+    # keyed step with the mean = combine, divide, update on the ids
+    H, kb = 120, 10
+    cold = rng.standard_normal((N, D)).astype(np.float32)
+    hot_ids = np.sort(rng.choice(N, H, replace=False)).astype(np.int64)
+    for avg in ("mean", "one_plus"):
+        a = [cold.copy(), np.zeros((N, D), np.float32), cold[hot_ids] + 1, np.zeros((H, D), np.float32)]
+        b = [x.copy() for x in a]
+        for _ in range(2):
+            O.sparse_adagrad_step(a[0], a[1], a[2], a[3], hot_ids, wu, O.averaged(ws, wc, avg), 0.01, 1e-10)
+            O.keyed_step(b[0], b[1], b[2], b[3], hot_ids, q, g, 0.01, 1e-10, kb, average=avg)
+        for x, y in zip(a, b):
+            assert np.array_equal(x, y)
+
+
 # ---- optimizers --------------------------------------------------------------------------
 def test_adagrad_matches_torch_optim():
     rng = np.random.default_rng(10)
