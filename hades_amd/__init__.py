@@ -4,6 +4,7 @@
     hades_amd.ops           fused operators: lookup, split, cached_fetch/set, combine, optimizers
     hades_amd.cache         EmbCache: hot-row cache keyed by the sorted hot-ID set
     hades_amd.sparse_optim  only_unique_grads / unique_grads / bucket_gradients / SparseAdagrad / SparseAdam
+    hades_amd.dist_emb      DistEmb / DistEmbeddingTensor and the trace-driven SparseAdam / SparseAdagrad
     hades_amd.index_cache   IndexCache / LocalCache: the set-associative index cache, in HBM
     hades_amd.cold_cache    ColdDataCache: the cache server's gradient path with its staleness rule
     hades_amd.shm           shared-memory segments and tensors, ShmTensorPool

@@ -84,9 +84,9 @@ _SIGNATURES = {
                                  ctypes.c_double, ctypes.c_double, c_float, _P],
     "hades_adam_update_class": [_P, _P, _P, _P, c_int, _L, _L, _L, _P, _P, _P, _P, _L, _P, _P, _P, c_int,
                                 c_float, ctypes.c_double, ctypes.c_double, c_float, _P],
-    "hades_hash_clear": [_P, _P, _P, _L, _L, _P],
-    "hades_hash_accumulate": [_P, _P, _P, _L, _P, _P, _P, _P, _L, _L, _P, _P],
-    "hades_hash_flush": [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P, _P, c_size_t, _P],
+    "hades_hash_clear": [_P, _P, _P, _L, _L, _L, _P],
+    "hades_hash_accumulate": [_P, _P, _P, _L, _P, _P, _P, _P, _L, _L, _P, _L, _P],
+    "hades_hash_flush": [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _L, _P, _L, _P, c_size_t, _P],
     "hades_bucket_by_owner": [_P, _L, _P, _L, _L, _L, _P, _L, c_int, _P, _P, _P, _P, _P, _P, _P,
                               c_size_t, _P],
     "hades_sacache_init": [_P, _P, _L, _P],

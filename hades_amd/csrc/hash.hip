@@ -35,12 +35,13 @@ __device__ __forceinline__ uint64_t mix64(uint64_t x) {
 __global__ __launch_bounds__(kThreads) void hash_clear_kernel(int64_t* __restrict__ keys,
                                                              float* __restrict__ accum,
                                                              int64_t* __restrict__ cnt,
-                                                             int64_t num_slots, int64_t dim) {
+                                                             int64_t num_slots, int64_t dim,
+                                                             int64_t ss) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
   const int64_t t = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   for (int64_t i = t; i < num_slots; i += stride) {
-    keys[i] = kEmpty;
-    cnt[i] = 0;
+    keys[i * ss] = kEmpty;
+    cnt[i * ss] = 0;
   }
   const int64_t total = num_slots * dim;
   for (int64_t i = t; i < total; i += stride) accum[i] = 0.f;
@@ -50,6 +51,7 @@ struct AccArgs {
   int64_t* keys; float* accum; int64_t* cnt; int64_t num_slots;
   const int64_t* ids; const float* grad; const int64_t* in_cnt; const int64_t* num_rows;
   int64_t max_rows; int64_t dim; int32_t* status;
+  int64_t ss;   // int64 words between the keys (and between the counts) of consecutive slots
 };
 
 template <int VEC>
@@ -68,12 +70,12 @@ __global__ __launch_bounds__(kThreads) void hash_accumulate_kernel(AccArgs a) {
     // a negative id is never stored (-1 marks an empty slot): its row is dropped, status bit 3
     // bounded probe: every wave leaves the loop after at most num_slots steps
     for (int64_t probe = 0; id >= 0 && probe < a.num_slots; ++probe) {
-      unsigned long long* kp = reinterpret_cast<unsigned long long*>(a.keys + h);
+      unsigned long long* kp = reinterpret_cast<unsigned long long*>(a.keys + h * a.ss);
       // A plain load is enough to look: a key, once stored, stays until the flush, so a
       // non-empty value is never stale in a harmful way, and a stale "empty" only sends the
       // thread to the compare-and-swap below, which is the arbiter (device-scope atomics are
       // executed beyond the per-XCD L2 and cost a round trip of their own).
-      int64_t k = a.keys[h];
+      int64_t k = a.keys[h * a.ss];
       if (k == kEmpty) {
         k = static_cast<int64_t>(atomicCAS(kp, static_cast<unsigned long long>(kEmpty),
                                            static_cast<unsigned long long>(id)));
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(kThreads) void hash_accumulate_kernel(AccArgs a) {
     if (slot < 0) {
       atomicOr(a.status, id < 0 ? 8 : 1);
     } else {
-      a.cnt[slot] += a.in_cnt ? a.in_cnt[row0 + r] : 1;
+      a.cnt[slot * a.ss] += a.in_cnt ? a.in_cnt[row0 + r] : 1;
     }
     s_slot[r] = slot;
   }
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(kThreads) void hash_accumulate_kernel(AccArgs a) {
 __global__ __launch_bounds__(kThreads) void flush_gather_ids_kernel(
     const int64_t* __restrict__ keys, const int64_t* __restrict__ live_pos,
     const int64_t* __restrict__ live_count, int64_t cap, int64_t pad, int64_t* __restrict__ ids_out,
-    int64_t* __restrict__ num_out, int32_t* __restrict__ status) {
+    int64_t* __restrict__ num_out, int32_t* __restrict__ status, int64_t ss) {
   const int64_t L = live_count[0];
   const bool overflow = L > cap;
   const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(kThreads) void flush_gather_ids_kernel(
     num_out[0] = overflow ? 0 : L;
     if (overflow) atomicOr(status, 2);
   }
-  if (j < cap) ids_out[j] = (!overflow && j < L) ? keys[live_pos[j]] : pad;
+  if (j < cap) ids_out[j] = (!overflow && j < L) ? keys[live_pos[j] * ss] : pad;
 }
 
 struct FlushArgs {
@@ -141,6 +143,7 @@ struct FlushArgs {
   const int64_t* live_pos; const uint32_t* perm; const int64_t* num_out;
   int64_t* out_ids; float* out_sums; int64_t* out_cnts; int64_t cap;
   const int32_t* bad; int64_t nbad; int32_t* status;
+  int64_t ss;
 };
 
 // out row j <- the live slot with the j-th smallest id; the slot is emptied
@@ -161,10 +164,10 @@ __global__ __launch_bounds__(kThreads) void flush_emit_kernel(FlushArgs a) {
   for (int r = threadIdx.x; r < rows_here; r += kThreads) {
     const int64_t slot = a.live_pos[a.perm[row0 + r]];
     s_slot[r] = slot;
-    a.out_ids[row0 + r] = a.keys[slot];
-    a.out_cnts[row0 + r] = a.cnt[slot];
-    a.keys[slot] = kEmpty;
-    a.cnt[slot] = 0;
+    a.out_ids[row0 + r] = a.keys[slot * a.ss];
+    a.out_cnts[row0 + r] = a.cnt[slot * a.ss];
+    a.keys[slot * a.ss] = kEmpty;
+    a.cnt[slot * a.ss] = 0;
   }
   __syncthreads();
   if (rows_here == 0) return;
@@ -229,14 +232,16 @@ using namespace hades;
 extern "C" {
 
 int hades_hash_clear(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots, int64_t dim,
-                     void* stream) {
+                     int64_t slot_stride, void* stream) {
   HADES_REQUIRE(is_pow2(num_slots), "num_slots must be a power of two (got %lld)",
                 (long long)num_slots);
   HADES_REQUIRE(dim >= 1 && keys && accum && cnt, "bad argument");
+  HADES_REQUIRE(slot_stride >= 0, "slot_stride must be >= 0");
+  const int64_t ss = slot_stride ? slot_stride : 1;
   int64_t blocks = ceil_div(num_slots * dim, kThreads * 8);
   if (blocks > 65536) blocks = 65536;
   HADES_LAUNCH(hash_clear_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(stream), keys, accum, cnt, num_slots, dim);
+                     static_cast<hipStream_t>(stream), keys, accum, cnt, num_slots, dim, ss);
   HADES_LAUNCH_CHECK();
   return HADES_OK;
 }
@@ -244,14 +249,16 @@ int hades_hash_clear(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slot
 int hades_hash_accumulate(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots,
                           const int64_t* ids, const float* grad, const int64_t* in_cnt,
                           const int64_t* num_rows, int64_t max_rows, int64_t dim, int32_t* status,
-                          void* stream) {
+                          int64_t slot_stride, void* stream) {
   HADES_REQUIRE(is_pow2(num_slots), "num_slots must be a power of two (got %lld)",
                 (long long)num_slots);
   HADES_REQUIRE(dim >= 1 && max_rows >= 0, "bad dim or max_rows");
+  HADES_REQUIRE(slot_stride >= 0, "slot_stride must be >= 0");
   HADES_REQUIRE(dim * kRows < (int64_t(1) << 30), "dim too large");
   if (max_rows == 0) return HADES_OK;
   HADES_REQUIRE(keys && accum && cnt && ids && grad && status, "null pointer argument");
-  AccArgs a{keys, accum, cnt, num_slots, ids, grad, in_cnt, num_rows, max_rows, dim, status};
+  AccArgs a{keys, accum, cnt, num_slots, ids, grad, in_cnt, num_rows, max_rows, dim, status,
+            slot_stride ? slot_stride : 1};
   const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec4 = dim % 4 == 0 && (align_of_ptr(accum) % 16) == 0 && (align_of_ptr(grad) % 16) == 0;
@@ -271,10 +278,12 @@ size_t hades_hash_flush_workspace_bytes(int64_t num_slots, int64_t cap) {
 
 int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots, int64_t dim,
                      int64_t id_bound, int64_t* out_ids, float* out_sums, int64_t* out_cnts,
-                     int64_t* num_out, int64_t cap, int32_t* status, void* workspace,
-                     size_t workspace_bytes, void* stream) {
+                     int64_t* num_out, int64_t cap, int32_t* status, int64_t slot_stride,
+                     void* workspace, size_t workspace_bytes, void* stream) {
   HADES_REQUIRE(is_pow2(num_slots), "num_slots must be a power of two (got %lld)",
                 (long long)num_slots);
+  HADES_REQUIRE(slot_stride >= 0, "slot_stride must be >= 0");
+  const int64_t ss = slot_stride ? slot_stride : 1;
   HADES_REQUIRE(dim >= 1 && cap >= 1 && cap < (int64_t(1) << 30), "bad dim or cap");
   HADES_REQUIRE(id_bound >= 0 && id_bound < INT64_MAX, "bad id_bound");
   HADES_REQUIRE(keys && accum && cnt && out_ids && out_sums && out_cnts && num_out && status,
@@ -286,18 +295,18 @@ int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slot
   HADES_REQUIRE((align_of_ptr(workspace) & 255) == 0, "workspace must be 256-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc = compact_live_keys(keys, num_slots, w.live_pos, w.live_count, w.compact_ws,
-                             w.compact_bytes, st);
+                             w.compact_bytes, st, ss);
   if (rc != HADES_OK) return rc;
   const int64_t pad = id_bound > 0 ? id_bound : INT64_MAX;
   HADES_LAUNCH(flush_gather_ids_kernel, dim3((unsigned)ceil_div(cap, kThreads)),
                      dim3(kThreads), 0, st, keys, w.live_pos, w.live_count, cap, pad, w.ids, num_out,
-                     status);
+                     status, ss);
   HADES_LAUNCH_CHECK();
   SortResult sr;
   rc = sort_ids(w.ids, cap, id_bound > 0 ? id_bound + 1 : 0, w.sort_ws, w.sort_bytes, st, &sr);
   if (rc != HADES_OK) return rc;
   FlushArgs a{keys, accum, cnt, dim, w.live_pos, sr.perm, num_out, out_ids, out_sums, out_cnts, cap,
-              sr.bad, sr.nbad, status};
+              sr.bad, sr.nbad, status, ss};
   const dim3 grid(static_cast<unsigned>(ceil_div(cap, kRows))), block(kThreads);
   const bool vec4 = dim % 4 == 0 && (align_of_ptr(accum) % 16) == 0 && (align_of_ptr(out_sums) % 16) == 0;
   if (vec4)

@@ -318,8 +318,9 @@ struct ClassifyLookup {
 
 struct ClassifyLive {
   const int64_t* keys;
+  int64_t stride;
   __device__ __forceinline__ uint32_t operator()(int64_t i) const {
-    return keys[i] != int64_t(-1) ? 0u : kNone;
+    return keys[i * stride] != int64_t(-1) ? 0u : kNone;
   }
 };
 
@@ -392,9 +393,10 @@ inline unsigned grid_1d(int64_t n) { return static_cast<unsigned>(ceil_div(n, kT
 size_t compact_live_workspace_bytes(int64_t n) { return carve_compact(nullptr, n < 0 ? 0 : n).bytes; }
 
 int compact_live_keys(const int64_t* keys, int64_t n, int64_t* pos_out, int64_t* count_out,
-                      void* workspace, size_t workspace_bytes, hipStream_t st) {
+                      void* workspace, size_t workspace_bytes, hipStream_t st, int64_t key_stride) {
   CompactOut out{{nullptr, nullptr, nullptr}, {pos_out, nullptr, nullptr}};
-  return run_compact(ClassifyLive{keys}, n, 1, out, count_out, workspace, workspace_bytes, st);
+  return run_compact(ClassifyLive{keys, key_stride}, n, 1, out, count_out, workspace,
+                     workspace_bytes, st);
 }
 
 }  // namespace hades

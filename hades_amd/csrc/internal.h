@@ -5,11 +5,12 @@
 
 namespace hades {
 
-// index.hip: ascending positions i with keys[i] != -1, and their number (device).
+// index.hip: ascending positions i with keys[i * key_stride] != -1, and their number (device).
 // pos_out needs capacity n.
 size_t compact_live_workspace_bytes(int64_t n);
 int compact_live_keys(const int64_t* keys, int64_t n, int64_t* pos_out, int64_t* count_out,
-                      void* workspace, size_t workspace_bytes, hipStream_t st);
+                      void* workspace, size_t workspace_bytes, hipStream_t st,
+                      int64_t key_stride = 1);
 
 // combine.hip: stable radix sort of (id, position) over the bits id_bound leaves significant.
 // On return *perm_out[j] is the position in `ids` of the j-th smallest id and *sorted_keys the

@@ -725,16 +725,18 @@ class ColdGradAccumulator:
         _check(num_slots > 0 and (num_slots & (num_slots - 1)) == 0, "num_slots must be a power of two")
         self.num_slots, self.dim, self.id_bound = int(num_slots), int(dim), int(id_bound)
         self.device = torch.device(device)
-        self.keys = torch.empty(num_slots, dtype=torch.int64, device=self.device)
+        # key and count of a slot share one 16-byte record: a probe and the count update touch one
+        # memory sector instead of two
+        self.slots = torch.empty((num_slots, 2), dtype=torch.int64, device=self.device)
+        self.keys, self.cnt = self.slots[:, 0], self.slots[:, 1]
         self.accum = torch.empty((num_slots, dim), dtype=torch.float32, device=self.device)
-        self.cnt = torch.empty(num_slots, dtype=torch.int64, device=self.device)
         self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
         self._ws = Workspace(self.device)
         self.clear()
 
     def clear(self):
         _lib.call("hades_hash_clear", _ptr(self.keys), _ptr(self.accum), _ptr(self.cnt),
-                  self.num_slots, self.dim, _stream())
+                  self.num_slots, self.dim, 2, _stream())
 
     def accumulate(self, ids, grad, cnt=None, num_rows=None):
         _i64(ids, "ids"); _dev(grad, "grad")
@@ -742,7 +744,7 @@ class ColdGradAccumulator:
                "grad must be float32 [rows, dim]")
         _lib.call("hades_hash_accumulate", _ptr(self.keys), _ptr(self.accum), _ptr(self.cnt),
                   self.num_slots, _ptr(ids), _ptr(grad), _opt(cnt), _opt(num_rows), ids.numel(),
-                  self.dim, _ptr(self.status), _stream())
+                  self.dim, _ptr(self.status), 2, _stream())
 
     def flush_padded(self, cap, out=None):
         """Returns (ids int64[cap], sums float32[cap, dim], cnts int64[cap], num_out int64[1]);
@@ -761,7 +763,7 @@ class ColdGradAccumulator:
         ws = self._ws.get(nbytes)
         _lib.call("hades_hash_flush", _ptr(self.keys), _ptr(self.accum), _ptr(self.cnt),
                   self.num_slots, self.dim, self.id_bound, _ptr(out_ids), _ptr(out_sums),
-                  _ptr(out_cnts), _ptr(num_out), cap, _ptr(self.status), _ptr(ws), ws.numel(),
+                  _ptr(out_cnts), _ptr(num_out), cap, _ptr(self.status), 2, _ptr(ws), ws.numel(),
                   _stream())
         return out_ids, out_sums, out_cnts, num_out
 

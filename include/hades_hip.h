@@ -501,13 +501,17 @@ int hades_adam_update_class_summing(const int64_t* ukeys, const float* grad_rows
  * status[0] (int32, device, sticky, cleared by the caller) collects error bits: 1 the table was
  * full and a row was dropped; 2 more live entries than the flush capacity (nothing emitted);
  * 4 a stored id was outside [0, id_bound] at flush time (rows emitted, but not in ascending
- * order); 8 a negative id was offered to accumulate (its row was dropped: -1 marks an empty slot). */
+ * order); 8 a negative id was offered to accumulate (its row was dropped: -1 marks an empty slot).
+ * slot_stride (int64 words; 0 = 1): the key of slot i is keys[i * slot_stride] and its count
+ * cnt[i * slot_stride], so that key and count of a slot may share one 16-byte record
+ * (cnt = keys + 1, slot_stride = 2): a probe and the count update then touch one memory sector
+ * instead of two. */
 int hades_hash_clear(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots, int64_t dim,
-                     void* stream);
+                     int64_t slot_stride, void* stream);
 int hades_hash_accumulate(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots,
                           const int64_t* ids, const float* grad, const int64_t* in_cnt,
                           const int64_t* num_rows, int64_t max_rows, int64_t dim,
-                          int32_t* status, void* stream);
+                          int32_t* status, int64_t slot_stride, void* stream);
 /* Flush: emit every live slot as (id, sum row, count) in ascending id order, then clear the table
  * (evident intent of python/EmbCache/server.py:413-419; see the note on :414 in the oracle).
  *   out_ids int64[cap], out_sums float[cap, dim], out_cnts int64[cap], num_out int64[1] (device)
@@ -515,7 +519,7 @@ int hades_hash_accumulate(int64_t* keys, float* accum, int64_t* cnt, int64_t num
 size_t hades_hash_flush_workspace_bytes(int64_t num_slots, int64_t cap);
 int hades_hash_flush(int64_t* keys, float* accum, int64_t* cnt, int64_t num_slots, int64_t dim,
                      int64_t id_bound, int64_t* out_ids, float* out_sums, int64_t* out_cnts,
-                     int64_t* num_out, int64_t cap, int32_t* status,
+                     int64_t* num_out, int64_t cap, int32_t* status, int64_t slot_stride,
                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* Pre-exchange bucketing: what swap_gradients does on one GPU before the all-to-all

@@ -48,9 +48,10 @@ def test_argument_errors_are_codes_and_messages():
     assert lib.hades_combine(one, one, 10, 8, 0, 5, one, one, one, one, null, one, 1 << 20, null) == 1
     assert lib.hades_combine(one, one, 10, 8, 0, 0, one, one, one, one, null, one, 16, null) == 3
     assert b"workspace too small" in lib.hades_last_error()
-    assert lib.hades_hash_clear(one, one, one, 1000, 8, null) == 1                  # not a power of two
+    assert lib.hades_hash_clear(one, one, one, 1000, 8, 0, null) == 1               # not a power of two
     with pytest.raises(RuntimeError, match="power of two"):
-        _lib.call("hades_hash_clear", one, one, one, 1000, 8, null)
+        _lib.call("hades_hash_clear", one, one, one, 1000, 8, 0, null)
+    assert lib.hades_hash_clear(one, one, one, 1024, 8, -2, null) == 1              # slot stride
 
 
 def test_argument_errors_of_the_split_schedule_entry_points():

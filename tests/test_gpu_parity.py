@@ -1817,6 +1817,78 @@ def test_keyed_and_split_steps_that_average_like_the_reference(lib, kind, averag
             assert np.allclose(a, w, rtol=0, atol=5e-6)
 
 
+@pytest.mark.parametrize("kind", ["adam", "adagrad"])
+@pytest.mark.parametrize("pin", [True, False])
+def test_dist_emb_module_trains_like_the_explicit_keyed_calls(lib, kind, pin):
+    """DistEmb + the trace-driven optimizer (the reference's training loop: emb(ids) ... backward
+    ... optimizer.step(), python/EmbCache/dist_emb.py:46-47,276-288, sparse_optim.py:212-238)
+    against the explicit forward_keyed / backward_keyed(average="mean") calls on an identically
+    initialised row optimizer: rows of every forward call and all tables after three steps are
+    bit-equal.  A step with two forward calls goes through the concatenated path and matches the
+    oracle's combine -> mean -> Adagrad on the concatenation."""
+    _, ops = lib
+    from hades_amd import dist_emb, sparse_optim
+    rng = np.random.default_rng(808 + pin)
+    N, D, n = 12_000, 32, 9000
+    weight = torch.from_numpy((rng.standard_normal((N, D)) * 0.05).astype(np.float32))
+    hotness = torch.from_numpy(rng.integers(0, 400, N))
+    emb = dist_emb.DistEmb(N, D, torch.float32, "emb", cache_rate=0.2, hotness_list=hotness,
+                           hot_threshold=300, weight=weight.clone(), pin_memory=pin)
+    hot_ids = emb.sparse_emb.hot_ids
+    assert 0 < hot_ids.numel() <= int(N * 0.2) and bool((hotness[hot_ids] >= 300).all())
+    if kind == "adam":
+        opt = dist_emb.SparseAdam([emb.sparse_emb], lr=0.01)
+        ref = sparse_optim.SparseAdam((weight.clone().pin_memory() if pin else weight.clone().cuda()), hot_ids, lr=0.01)
+    else:
+        opt = dist_emb.SparseAdagrad([emb.sparse_emb], lr=0.01)
+        ref = sparse_optim.SparseAdagrad((weight.clone().pin_memory() if pin else weight.clone().cuda()), hot_ids,
+                                         lr=0.01)
+    eng = opt._state["emb"]
+    coeff = dev((rng.standard_normal((n, D)) * 1e-2).astype(np.float32))
+    emb.train()
+    for it in range(3):
+        ids = dev(zipfish(rng, n, N))
+        rows = emb(ids)
+        want_rows, state = ref.forward_keyed(ids)
+        assert torch.equal(rows.detach(), want_rows)
+        (rows * coeff).sum().backward()
+        assert len(emb.sparse_emb.trace) == 1
+        opt.step()
+        assert emb.sparse_emb.trace == []
+        ref.backward_keyed(state, coeff, average="mean")
+        torch.cuda.synchronize()
+    names = (("cold_w", "cold_step", "cold_m", "cold_v", "hot_w", "hot_step", "hot_m", "hot_v") if kind == "adam"
+             else ("cold_w", "cold_s", "hot_w", "hot_s"))
+    for k in names:
+        assert torch.equal(getattr(eng, k).cpu(), getattr(ref, k).cpu()), k
+    # evaluation mode: plain rows, no trace
+    emb.eval()
+    probe = dev(rng.integers(0, N, 500).astype(np.int64))
+    with torch.no_grad():
+        got = emb(probe)
+    assert emb.sparse_emb.trace == [] and not got.requires_grad
+    assert np.array_equal(got.cpu().numpy(), O.cached_fetch(eng.cold_w.cpu().numpy(), eng.hot_w.cpu().numpy(),
+                                                            probe.cpu().numpy(), hot_ids.numpy()))
+    if kind == "adagrad":
+        # two forward calls in one step: concatenated, combined, averaged, applied once
+        emb.train()
+        cw, cs = eng.cold_w.cpu().numpy().copy(), eng.cold_s.cpu().numpy().copy()
+        hw, hs = eng.hot_w.cpu().numpy().copy(), eng.hot_s.cpu().numpy().copy()
+        ids_a, ids_b = zipfish(rng, 4000, N), zipfish(rng, 3000, N)
+        ca = (rng.standard_normal((4000, D)) * 1e-2).astype(np.float32)
+        cb = (rng.standard_normal((3000, D)) * 1e-2).astype(np.float32)
+        ra, rb = emb(dev(ids_a)), emb(dev(ids_b))
+        ((ra * dev(ca)).sum() + (rb * dev(cb)).sum()).backward()
+        assert len(emb.sparse_emb.trace) == 2
+        opt.step()
+        torch.cuda.synchronize()
+        wu, ws, wc = O.combine_sequential(np.concatenate([ids_a, ids_b]), np.concatenate([ca, cb]))
+        # the concatenated path sums in the fast mode: compare through the tolerance of the combine
+        O.sparse_adagrad_step(cw, cs, hw, hs, hot_ids.numpy(), wu, O.averaged(ws, wc, "mean"), 0.01, 1e-10)
+        for got_t, want in ((eng.cold_w, cw), (eng.cold_s, cs), (eng.hot_w, hw), (eng.hot_s, hs)):
+            assert np.allclose(got_t.cpu().numpy(), want, rtol=1e-4, atol=1e-7)
+
+
 def test_lookup_split_beyond_the_in_kernel_tile_sum(lib):
     """More than 4 096 tiles of queries: the per-tile counts are prefixed by a scan kernel of their
     own instead of being summed inside every compaction block.  Same lists, same slots."""
