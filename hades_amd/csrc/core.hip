@@ -74,8 +74,9 @@ bool is_host_memory(const void* p) {
 // (42.6 GB/s each way); an update that only writes (stores are posted: its waves never wait for
 // the link) reaches 40 / 50 / 53 GB/s alone with 16 / 32 / 64 blocks and no more beyond; every
 // further store in flight only queues up in front of the HBM traffic of other streams.  Inside a
-// step, beside the hot-class sums: 32 blocks 812 us (sums beside it 153 us), 64 blocks 789 us
-// (573 us), 96 blocks 771 us (642 us, as long as the update itself): 64 it is.
+// step, beside the hot-class sums and update (blocks: cold update / hot sums + hot update, us):
+// 24: 951 / 272; 32: 849 / 291; 36: 808 / 305; 40: 787 / 352; 44: 772 / 492; 64: 798 / 662.
+// 40 keeps the step within 1 % of its best and the hot class well clear of the cold update.
 // HADES_HOST_LINK_BLOCKS / _RW / _WO (read once, at the first use) and
 // hades_set_host_link_blocks() override the three widths for tuning.
 namespace {
@@ -85,7 +86,7 @@ std::atomic<int64_t> g_link_blocks[3] = {{0}, {0}, {0}};   // 0: not set yet
 int64_t host_link_blocks(HostLinkUse use) {
   static const char* const names[] = {"HADES_HOST_LINK_BLOCKS", "HADES_HOST_LINK_BLOCKS_RW",
                                       "HADES_HOST_LINK_BLOCKS_WO"};
-  static const int64_t defaults[] = {16, 128, 64};
+  static const int64_t defaults[] = {16, 128, 40};
   int64_t v = g_link_blocks[use].load(std::memory_order_relaxed);
   if (v > 0) return v;
   v = defaults[use];

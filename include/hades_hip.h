@@ -76,7 +76,7 @@ int hades_profile_kernel(int kernel_id, void* start_event, void* stop_event);
  * reference, whose row kernels are launched one block per 32 rows whatever the memory,
  * src/cuda/uva_fetch.cu:86-95).  use: 0 a row copy one way (gather from / scatter to a host table),
  * 1 an update that reads and writes host rows, 2 an update that only writes them.  blocks = 0
- * restores the default (16 / 128 / 64, or the HADES_HOST_LINK_BLOCKS, _RW, _WO environment
+ * restores the default (16 / 128 / 40, or the HADES_HOST_LINK_BLOCKS, _RW, _WO environment
  * variables, which are read once, at first use).  Process-wide; meant for tuning and measurement. */
 int hades_set_host_link_blocks(int use, int64_t blocks);
 int64_t hades_get_host_link_blocks(int use);
