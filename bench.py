@@ -216,7 +216,11 @@ class Workload:
                  ", %d trainer batches concatenated" % self.trainers if self.trainers > 1 else ""))
 
 
-def link_probe(dev, nbytes=256 << 20, reps=4):
+class WorkloadSetupError(RuntimeError):
+    """The tables of a workload could not be allocated on this host / GPU."""
+
+
+def link_probe(dev, nbytes=128 << 20, reps=4):
     """Pinned hipMemcpyAsync rates of this box, GB/s: host to device, device to host, and each
     direction while the other runs on a second stream."""
     import torch
@@ -407,7 +411,13 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
     from hades_amd import ops
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    wl = Workload(workload, args.batches, dev, args.optimizer, state_on_host=state_on_host)
+    try:
+        wl = Workload(workload, args.batches, dev, args.optimizer, state_on_host=state_on_host)
+    except (RuntimeError, MemoryError) as err:
+        msg = str(err).splitlines()[0][:300] if str(err) else type(err).__name__
+        if "memory" in msg.lower():
+            raise WorkloadSetupError(msg) from err
+        raise
     if args.sort is not None:
         ops.sort_config(one_sweep=args.sort == "one-sweep")
     opt = wl.opt
@@ -551,10 +561,18 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
     if with_gate:
         gate = parity_gate(wl, gate_step, average=average, rows_are_sums=keyed)
         log("parity gate passed: %s" % json.dumps(gate["max_rel_err"]))
-    link = link_probe(dev) if (with_link and wl.host_cold) else None
-    if link:
-        link["kernels"] = link_kernel_probe(wl)
-        log("host link: %s" % json.dumps(link))
+    link = None
+    if with_link and wl.host_cold:
+        # the probes need page-locked buffers of their own next to the 56.8 GB table: a host that
+        # has none left loses the probes, not the measurement
+        try:
+            link = link_probe(dev)
+            link["kernels"] = link_kernel_probe(wl)
+            log("host link: %s" % json.dumps(link))
+        except (RuntimeError, MemoryError) as err:
+            link = None
+            log("host-link probes skipped: %s" % (str(err).splitlines()[0][:200] if str(err) else type(err).__name__))
+            torch.cuda.empty_cache()
 
     for i in range(args.warmup):
         step(i)
@@ -1546,11 +1564,11 @@ def main():
     try:
         res = run_gpu(args, args.workload, args.schedule, reuse_rows=args.reuse_rows,
                       state_on_host=args.cold_state == "host")
-    except (RuntimeError, MemoryError) as err:
+    except WorkloadSetupError as err:
         # a host that refuses the 56.8 GB page-locked table (or lacks the HBM): say so and measure
         # the all-HBM configuration instead of printing nothing
-        msg = str(err).splitlines()[0][:300] if str(err) else type(err).__name__
-        if args.workload != "cfg3" or "memory" not in msg.lower():
+        msg = str(err)
+        if args.workload != "cfg3":
             raise
         if not args.allow_fallback:
             print("bench.py: cfg3 could not be set up on this host (%s).  Nothing was measured; "
@@ -1619,65 +1637,75 @@ def main():
     if fallback:
         line["config"]["fallback"] = fallback
     if args.workload == "cfg3" and not args.no_secondary:
-        log("secondary workload cfg2 (whole table in HBM)")
-        sec = run_gpu(args, "cfg2", None, with_gate=False, with_link=False)
-        line["secondary"] = {"cfg2": {
-            "workload": sec["workload"], "schedule": sec["schedule"],
-            "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
-            "step_us": sec["step_us"], "step_frac_hbm": sec["step_frac_hbm"],
-            "roofline": sec["roofline"], "kernels": sec["kernels"], "phases": sec["phases"]}}
-        if schedule == "keyed" and args.reuse_rows:
-            log("secondary: cfg3 again with the cold update re-reading the host table")
-            sec = run_gpu(args, "cfg3", "keyed", with_gate=True, with_link=False, reuse_rows=False)
-            line["secondary"]["cfg3_table_reread"] = {
-                "what": "the headline workload and schedule, but the cold update reads the old weight "
-                        "rows from the host table a second time (backward_keyed(fetched_rows=None), or "
-                        "an optimizer constructed with reuse_fetched_rows=False): what a table with "
-                        "writers the optimizer cannot see has to do.  Bit-identical results",
-                "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
-                "step_us": sec["step_us"], "phases": sec["phases"], "pcie": sec["pcie"],
-                "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
-                            for k, v in sec["kernels"].items()},
-                "parity_gate": sec["parity_gate"]}
-        if schedule == "keyed" and args.reuse_rows and args.cold_state == "hbm":
-            log("secondary: cfg3's batch on a half-size table with the cold Adagrad state in host memory")
+        line["secondary"] = {}
+
+        def secondary(key, what, build, **run_kw):
+            """One nested measurement.  A host or GPU that cannot hold it (allocation refused) leaves
+            a `skipped` entry instead of taking the headline down with it; a parity-gate failure is
+            not caught."""
+            log("secondary: " + key)
             try:
-                sec = run_gpu(args, "cfg3", "keyed", with_gate=True, with_link=False, reuse_rows=True,
-                              state_on_host=True)
-                line["secondary"]["cfg3_cold_state_in_host_memory"] = {
-                    "what": "the contract layout of the cold class: weights AND Adagrad state of the cold "
-                            "rows in pinned host memory, the two rows of an id side by side ([N, 2, D], "
-                            "1 KB per id), on a table cut to 55.5 M rows with 5.55 M hot so that the one "
-                            "page-locked allocation this box grants (56.8 GB) holds both; cfg3's batch "
-                            "size, skew and 10 % hot fraction",
-                    "workload": sec["workload"],
-                    "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
-                    "step_us": sec["step_us"], "phases": sec["phases"], "pcie": sec["pcie"],
-                    "hot_hit": sec["hot_hit"], "unique_per_step": sec["unique_per_step"],
+                sec = run_gpu(args, **run_kw)
+            except (RuntimeError, MemoryError) as err:
+                line["secondary"][key] = {"skipped": str(err).splitlines()[0][:300] if str(err)
+                                          else type(err).__name__}
+                import gc
+                import torch
+                gc.collect()
+                torch.cuda.empty_cache()
+                return
+            entry = {"what": what} if what else {}
+            entry.update(build(sec))
+            line["secondary"][key] = entry
+
+        def brief(sec):
+            return {"value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
+                    "step_us": sec["step_us"], "phases": sec["phases"], "pcie": sec.get("pcie"),
                     "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
                                 for k, v in sec["kernels"].items()},
                     "parity_gate": sec["parity_gate"]}
-            except (RuntimeError, MemoryError) as err:
-                line["secondary"]["cfg3_cold_state_in_host_memory"] = {
-                    "skipped": str(err).splitlines()[0][:300] if str(err) else type(err).__name__}
+
+        secondary("cfg2", None, lambda sec: {
+            "workload": sec["workload"], "schedule": sec["schedule"],
+            "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
+            "step_us": sec["step_us"], "step_frac_hbm": sec["step_frac_hbm"],
+            "roofline": sec["roofline"], "kernels": sec["kernels"], "phases": sec["phases"]},
+            workload="cfg2", schedule=None, with_gate=False, with_link=False)
         if schedule == "keyed" and args.reuse_rows:
-            log("secondary: cfg3 with two batches in flight (pipelined schedule, fetched rows reused)")
-            sec = run_gpu(args, "cfg3", "pipelined", with_gate=True, with_link=False, reuse_rows=True)
-            line["secondary"]["cfg3_pipelined"] = {
-                "what": "the headline workload with the next batch's forward half (lookup, partition, "
-                        "cold gather, key sort) running on side streams while this batch's cold update "
-                        "writes the host table, so that the link carries reads and writes at once; the "
-                        "cold rows that update wrote are read again afterwards, and every batch gets the "
-                        "rows and leaves the tables of the one-batch-at-a-time order, bit for bit.  Needs "
-                        "the ids of a batch one step ahead (prefetch_keyed / finish_prefetch) and, for the "
-                        "reuse of the fetched rows, one writer per table row",
-                "value": round(sec["n"] / (sec["ms_per_step"] * 1e-3), 1), "unit": "rows/s",
-                "step_us": sec["step_us"], "pcie": sec["pcie"],
-                "kernels": {k: {a: b for a, b in v.items() if a in ("us", "us_alone", "GB/s")}
-                            for k, v in sec["kernels"].items()},
-                "parity_gate": sec["parity_gate"]}
+            secondary("cfg3_table_reread",
+                      "the headline workload and schedule, but the cold update reads the old weight "
+                      "rows from the host table a second time (backward_keyed(fetched_rows=None), or "
+                      "an optimizer constructed with reuse_fetched_rows=False): what a table with "
+                      "writers the optimizer cannot see has to do.  Bit-identical results", brief,
+                      workload="cfg3", schedule="keyed", with_gate=True, with_link=False, reuse_rows=False)
+        if schedule == "keyed" and args.reuse_rows and args.cold_state == "hbm":
+            secondary("cfg3_cold_state_in_host_memory",
+                      "the contract layout of the cold class: weights AND Adagrad state of the cold "
+                      "rows in pinned host memory, the two rows of an id side by side ([N, 2, D], "
+                      "1 KB per id), on a table cut to 55.5 M rows with 5.55 M hot so that the one "
+                      "page-locked allocation this box grants (56.8 GB) holds both; cfg3's batch "
+                      "size, skew and 10 % hot fraction",
+                      lambda sec: dict(brief(sec), workload=sec["workload"], hot_hit=sec["hot_hit"],
+                                       unique_per_step=sec["unique_per_step"]),
+                      workload="cfg3", schedule="keyed", with_gate=True, with_link=False, reuse_rows=True,
+                      state_on_host=True)
+        if schedule == "keyed" and args.reuse_rows:
+            secondary("cfg3_pipelined",
+                      "the headline workload with the next batch's forward half (lookup, partition, "
+                      "cold gather, key sort) running on side streams while this batch's cold update "
+                      "writes the host table, so that the link carries reads and writes at once; the "
+                      "cold rows that update wrote are read again afterwards, and every batch gets the "
+                      "rows and leaves the tables of the one-batch-at-a-time order, bit for bit.  Needs "
+                      "the ids of a batch one step ahead (prefetch_keyed / finish_prefetch) and, for the "
+                      "reuse of the fetched rows, one writer per table row", brief,
+                      workload="cfg3", schedule="pipelined", with_gate=True, with_link=False, reuse_rows=True)
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = run_cpu_baseline(args.workload, args.cpu_seconds)
+        try:
+            line["cpu_baseline"] = run_cpu_baseline(args.workload, args.cpu_seconds)
+        except (RuntimeError, MemoryError) as err:
+            line["cpu_baseline"] = {"value": None, "unit": "rows/s", "cores": None, "kind": "port",
+                                    "sample": "not measured: %s" % (str(err).splitlines()[0][:200]
+                                                                    if str(err) else type(err).__name__)}
     print(json.dumps(line))
 
 
