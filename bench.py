@@ -489,9 +489,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
                 plan = ops.combine_plan(q, D, id_bound=N, workspace=opt._ws, out=out_ids)
             res = ops.combine_apply(plan, g, cmode, out=out_sum)
             if events: events[2].record()
-            if average:
-                ops.rows_div_count_(res[1], res[2], res[3], one_plus=average == "one_plus")
-            opt.update(res[0], res[1], res[3])
+            opt.update(res[0], res[1], res[3], cnts=res[2], average=average)
         if events: events[3].record()
         return rows, res
 
@@ -559,7 +557,7 @@ def run_gpu(args, workload, schedule, with_gate=True, with_link=True, reuse_rows
 
     gate = None
     if with_gate:
-        gate = parity_gate(wl, gate_step, average=average, rows_are_sums=keyed)
+        gate = parity_gate(wl, gate_step, average=average, rows_are_sums=not split)
         log("parity gate passed: %s" % json.dumps(gate["max_rel_err"]))
     link = None
     if with_link and wl.host_cold:

@@ -77,8 +77,8 @@ _SIGNATURES = {
     "hades_combine_plan": [_P, _L, _L, _L, _P, _P, _P, _P, c_size_t, _P],
     "hades_combine_apply": [_P, _L, _L, _L, c_int, _P, _P, _P, _P, c_size_t, _P],
     "hades_rows_div_count": [_P, _P, _P, _L, _L, c_int, _P],
-    "hades_adagrad_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, _P, c_float, c_float, _P],
-    "hades_adam_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P,
+    "hades_adagrad_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, _P, _P, c_int, c_float, c_float, _P],
+    "hades_adam_update": [_P, _P, _P, _L, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int,
                           c_float, ctypes.c_double, ctypes.c_double, c_float, _P],
     "hades_adam_update_listed": [_P, _P, _P, _P, _L, _L, _P, _P, _P, _P, _L, c_float,
                                  ctypes.c_double, ctypes.c_double, c_float, _P],

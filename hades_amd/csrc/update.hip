@@ -48,6 +48,9 @@ struct RowArgs {
   int64_t max_rows;
   int64_t dim;
   HotSet hs;
+  // averaging as in ListedRows below: 0 none, 1 divide row u by cnts[u], 2 by cnts[u] + 1
+  const int64_t* cnts;
+  int average;
 };
 
 struct AdagradArgs {
@@ -65,7 +68,8 @@ struct AdamArgs {
 
 // phase 1 shared by both optimizers: s_row[r] = element offset of the row in its table,
 // s_hot[r] = 1 if that table is the hot one.  Returns the number of live rows of this block.
-__device__ __forceinline__ int resolve_rows(const RowArgs& a, int64_t* s_row, uint8_t* s_hot) {
+__device__ __forceinline__ int resolve_rows(const RowArgs& a, int64_t* s_row, uint8_t* s_hot,
+                                            float* s_div) {
   const int64_t U = a.num_unique ? a.num_unique[0] : a.max_rows;
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRows;
   const int64_t left = (U < a.max_rows ? U : a.max_rows) - row0;
@@ -75,6 +79,7 @@ __device__ __forceinline__ int resolve_rows(const RowArgs& a, int64_t* s_row, ui
     const int64_t loc = a.hs.slot(id);
     s_row[r] = loc >= 0 ? loc : id;
     s_hot[r] = loc >= 0 ? 1 : 0;
+    if (a.average != 0) s_div[r] = static_cast<float>(a.cnts[row0 + r] + (a.average == 2 ? 1 : 0));
   }
   return rows_here;
 }
@@ -84,7 +89,8 @@ __global__ __launch_bounds__(kThreads) void adagrad_kernel(AdagradArgs a) {
   typedef typename Vf<VEC>::type V;
   __shared__ int64_t s_row[kRows];
   __shared__ uint8_t s_hot[kRows];
-  const int rows_here = resolve_rows(a.r, s_row, s_hot);
+  __shared__ float s_div[kRows];
+  const int rows_here = resolve_rows(a.r, s_row, s_hot, s_div);
   __syncthreads();
   if (rows_here == 0) return;
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRows;
@@ -114,6 +120,7 @@ __global__ __launch_bounds__(kThreads) void adagrad_kernel(AdagradArgs a) {
     for (int k = 0; k < kUnroll; ++k) {
       const int c = base + k * kThreads;
       if (c < total) {
+        if (a.r.average != 0) g[k] = vdiv(g[k], V(s_div[c / cpr]));
         const V s1 = s[k] + g[k] * g[k];
         const V std_ = vsqrt(s1) + a.eps;
         const V w1 = w[k] - vdiv(a.lr * g[k], std_);
@@ -401,7 +408,8 @@ __global__ __launch_bounds__(kThreads) void adam_kernel(AdamArgs a) {
   __shared__ uint8_t s_hot[kRows];
   __shared__ float s_c1[kRows];
   __shared__ float s_c2[kRows];
-  const int rows_here = resolve_rows(a.r, s_row, s_hot);
+  __shared__ float s_div[kRows];
+  const int rows_here = resolve_rows(a.r, s_row, s_hot, s_div);
   // per-row step counter and bias corrections (thread r owns row r in both loops)
   for (int r = threadIdx.x; r < rows_here; r += kThreads) {
     float* sp = (s_hot[r] ? a.hot_step : a.cold_step) + s_row[r];
@@ -444,6 +452,7 @@ __global__ __launch_bounds__(kThreads) void adam_kernel(AdamArgs a) {
     for (int k = 0; k < kUnroll; ++k) {
       const int c = base + k * kThreads;
       if (c < total) {
+        if (a.r.average != 0) g[k] = vdiv(g[k], V(s_div[c / cpr]));
         const V m1 = a.beta1 * m[k] + a.one_minus_beta1 * g[k];
         const V v1 = a.beta2 * v[k] + a.one_minus_beta2 * (g[k] * g[k]);
         const V mc = vdiv(m1, V(c1[k]));
@@ -555,14 +564,16 @@ extern "C" {
 
 int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                          int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,
-                         const void* hot_index, float* hot_w, float* hot_s, float* cold_w, float* cold_s, float lr,
-                         float eps, void* stream) {
+                         const void* hot_index, float* hot_w, float* hot_s, float* cold_w, float* cold_s,
+                         const int64_t* cnts, int average, float lr, float eps, void* stream) {
   int rc = check_rows(uids, grad, max_rows, dim, sorted_hot, num_hot);
   if (rc != HADES_OK) return rc;
+  HADES_REQUIRE(average >= 0 && average <= 2, "average must be 0, 1 or 2");
   if (max_rows == 0) return HADES_OK;
+  HADES_REQUIRE(average == 0 || cnts != nullptr, "averaging needs the occurrence counts of the rows (cnts)");
   HADES_REQUIRE(num_hot == 0 || (hot_w && hot_s), "hot tables are null but num_hot > 0");
   AdagradArgs a{{uids, grad, num_unique, max_rows, dim,
-              HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}},
+              HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}, cnts, average},
                 hot_w, hot_s, cold_w, cold_s, lr, eps};
   const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -685,11 +696,13 @@ int hades_adam_update_class(const int64_t* ukeys, const float* grad, const int64
 int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                       int64_t max_rows, int64_t dim, const int64_t* sorted_hot, int64_t num_hot,
                       const void* hot_index, float* hot_w, float* hot_step, float* hot_m, float* hot_v, float* cold_w,
-                      float* cold_step, float* cold_m, float* cold_v, float lr, double beta1,
-                      double beta2, float eps, void* stream) {
+                      float* cold_step, float* cold_m, float* cold_v, const int64_t* cnts,
+                      int average, float lr, double beta1, double beta2, float eps, void* stream) {
   int rc = check_rows(uids, grad, max_rows, dim, sorted_hot, num_hot);
   if (rc != HADES_OK) return rc;
+  HADES_REQUIRE(average >= 0 && average <= 2, "average must be 0, 1 or 2");
   if (max_rows == 0) return HADES_OK;
+  HADES_REQUIRE(average == 0 || cnts != nullptr, "averaging needs the occurrence counts of the rows (cnts)");
   HADES_REQUIRE(num_hot == 0 || (hot_w && hot_step && hot_m && hot_v),
                 "hot tables are null but num_hot > 0");
   // the betas arrive as doubles because the reference forms 1 - beta in Python double arithmetic
@@ -698,7 +711,7 @@ int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num
   const float omb1 = static_cast<float>(1.0 - beta1);
   const float omb2 = static_cast<float>(1.0 - beta2);
   AdamArgs a{{uids, grad, num_unique, max_rows, dim,
-              HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}},
+              HotSet{sorted_hot, num_hot, static_cast<const uint32_t*>(hot_index)}, cnts, average},
              hot_w, hot_step, hot_m, hot_v, cold_w, cold_step, cold_m, cold_v,
              lr, static_cast<float>(beta1), static_cast<float>(beta2), omb1, omb2, eps};
   const dim3 grid(static_cast<unsigned>(ceil_div(max_rows, kRows))), block(kThreads);

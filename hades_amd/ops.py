@@ -678,10 +678,15 @@ def rows_div_count_(sums, cnts, num_unique=None, one_plus=False):
 
 # ---- row optimizers -----------------------------------------------------------
 def adagrad_update_(uids, grad, hot_w, hot_s, cold_w, cold_s, sorted_hot, lr, eps,
-                    num_unique=None):
+                    num_unique=None, cnts=None, average=None):
     """Sparse Adagrad over the rows named by the duplicate-free `uids`, in place:
     s += g*g;  w -= lr * g / (sqrt(s) + eps), each row in the hot tables if its id is in
-    sorted_hot, else in the cold tables (device or pinned host)."""
+    sorted_hot, else in the cold tables (device or pinned host).  `average` = "mean" / "one_plus"
+    with `cnts` (the combine's counts) divides every row by its count (plus one) first."""
+    avg = _average_code(average)
+    if avg:
+        _check(cnts is not None, "averaging needs cnts")
+        _i64(cnts, "cnts")
     _i64(uids, "uids"); _dev(grad, "grad")
     _check(grad.dtype == torch.float32 and grad.dim() == 2, "grad must be a 2-D float32 tensor")
     dim = grad.size(1)
@@ -697,18 +702,24 @@ def adagrad_update_(uids, grad, hot_w, hot_s, cold_w, cold_s, sorted_hot, lr, ep
     _check(grad.size(0) >= uids.numel(), "grad has fewer rows than uids has entries")
     _lib.call("hades_adagrad_update", _ptr(uids), _ptr(grad), _opt(num_unique), uids.numel(), dim,
               hp, hn, hi, _opt(hot_w), _opt(hot_s), _opt(cold_w), _opt(cold_s),
-              float(lr), float(eps), _stream())
+              _opt(cnts if avg else None), avg, float(lr), float(eps), _stream())
 
 
-def adam_update_(uids, grad, hot, cold, sorted_hot, lr, beta1, beta2, eps, num_unique=None):
-    """SparseAdam row update in place.  `hot` and `cold` are (w, step, mem, power) tuples."""
+def adam_update_(uids, grad, hot, cold, sorted_hot, lr, beta1, beta2, eps, num_unique=None,
+                 cnts=None, average=None):
+    """SparseAdam row update in place.  `hot` and `cold` are (w, step, mem, power) tuples;
+    `cnts` / `average` as in adagrad_update_."""
+    avg = _average_code(average)
+    if avg:
+        _check(cnts is not None, "averaging needs cnts")
+        _i64(cnts, "cnts")
     _i64(uids, "uids"); _dev(grad, "grad")
     dim = grad.size(1)
     hp, hn, hi = _hot_args(sorted_hot)
     hot = hot if hot is not None else (None, None, None, None)
     _lib.call("hades_adam_update", _ptr(uids), _ptr(grad), _opt(num_unique), uids.numel(), dim,
               hp, hn, hi, _opt(hot[0]), _opt(hot[1]), _opt(hot[2]), _opt(hot[3]),
-              _opt(cold[0]), _opt(cold[1]), _opt(cold[2]), _opt(cold[3]),
+              _opt(cold[0]), _opt(cold[1]), _opt(cold[2]), _opt(cold[3]), _opt(cnts if avg else None), avg,
               float(lr), float(beta1), float(beta2), float(eps), _stream())
 
 

@@ -588,15 +588,17 @@ class _SparseRowOptimizer:
         self.update_split(uids, sums, nu, cnts=cnts, average=average)
         return uids, sums, cnts, nu
 
-    def step(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None):
+    def step(self, idx, grad, mode=ops.COMBINE_FAST, plan=None, out=None, average=None):
         """combine the per-occurrence gradients, then update every distinct row once.
-        No host synchronisation.  `plan` = what prepare(idx) returned, if it was called."""
+        No host synchronisation.  `plan` = what prepare(idx) returned, if it was called.
+        `average` = "mean" / "one_plus": the update divides every id's sum by its occurrences
+        (plus one) inside its kernel; the returned rows stay the sums."""
         if plan is None:
             plan = ops.combine_plan(idx, self.dim, id_bound=self.num_rows, workspace=self._ws)
         else:
             torch.cuda.current_stream().wait_event(plan.ready)
         uids, sums, cnts, nu = ops.combine_apply(plan, grad, mode, out=out)
-        self.update(uids, sums, nu)
+        self.update(uids, sums, nu, cnts=cnts, average=average)
         return uids, sums, cnts, nu
 
 
@@ -634,10 +636,10 @@ class SparseAdagrad(_SparseRowOptimizer):
                                   grad_rows=grad_rows, out=out if grad_rows is not None else None,
                                   average=average, cnts=out[1] if out is not None else None)
 
-    def update(self, uids, grad, num_unique=None):
+    def update(self, uids, grad, num_unique=None, cnts=None, average=None):
         self._epoch += 1
         ops.adagrad_update_(uids, grad, self.hot_w, self.hot_s, self.cold_w, self.cold_s,
-                            self.hot_set, self.lr, self.eps, num_unique)
+                            self.hot_set, self.lr, self.eps, num_unique, cnts=cnts, average=average)
 
 
 class SparseAdam(_SparseRowOptimizer):
@@ -670,11 +672,12 @@ class SparseAdam(_SparseRowOptimizer):
                                grad_rows=grad_rows, out=out if grad_rows is not None else None,
                                average=average, cnts=out[1] if out is not None else None)
 
-    def update(self, uids, grad, num_unique=None):
+    def update(self, uids, grad, num_unique=None, cnts=None, average=None):
         self._epoch += 1
         ops.adam_update_(uids, grad, (self.hot_w, self.hot_step, self.hot_m, self.hot_v),
                          (self.cold_w, self.cold_step, self.cold_m, self.cold_v), self.hot_set,
-                         self.lr, self.betas[0], self.betas[1], self.eps, num_unique)
+                         self.lr, self.betas[0], self.betas[1], self.eps, num_unique,
+                         cnts=cnts, average=average)
 
     def update_like_reference(self, idx, grad, cnt=None, is_unique=False, mode=ops.COMBINE_FAST):
         """The reference's SparseAdam.update(idx, grad, emb, cnt, is_unique)

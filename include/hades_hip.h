@@ -383,12 +383,15 @@ int hades_rows_div_count(float* sums, const int64_t* cnts, const int64_t* num_un
  *     (w, s) = loc >= 0 ? (hot_w[loc], hot_s[loc]) : (cold_w[id], cold_s[id])
  *     s += g*g;  w -= lr * g / (sqrt(s) + eps)          (each operation rounded to fp32, no FMA)
  * uids must be duplicate-free.  num_unique may be NULL (then all max_rows rows are live).
- * sorted_hot may be NULL with num_hot == 0 (everything in the cold tables). */
+ * sorted_hot may be NULL with num_hot == 0 (everything in the cold tables).
+ * average: 0 the rows of grad are applied as they are; 1 row u is first divided by cnts[u], its number
+ * of occurrences (the mean of unique_grads, python/EmbCache/sparse_optim.py:150-156); 2 by cnts[u] + 1
+ * (:145-148).  cnts (int64, the counts hades_combine wrote) may be NULL when average is 0. */
 int hades_adagrad_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                          int64_t max_rows, int64_t dim,
                          const int64_t* sorted_hot, int64_t num_hot, const void* hot_index,
                          float* hot_w, float* hot_s, float* cold_w, float* cold_s,
-                         float lr, float eps, void* stream);
+                         const int64_t* cnts, int average, float lr, float eps, void* stream);
 
 /* The same Adagrad arithmetic over one half of a split, against one table pair:
  *   for j < min(count[0], max_count): p = list[j]; r = row_index[p]; g = grad[p, :]
@@ -453,12 +456,14 @@ int hades_adagrad_update_class_summing(const int64_t* ukeys, const float* grad_r
 /* SparseAdam row update, same fusion (python/EmbCache/sparse_optim.py:632-657,681):
  *   step += 1; m = b1*m + (1-b1)*g; v = b2*v + (1-b2)*g*g
  *   w -= lr * (m / (1 - b1^step)) / (sqrt(v / (1 - b2^step)) + eps)
- * step: float[N] / float[H]; m, v, w: float[., dim]. */
+ * step: float[N] / float[H]; m, v, w: float[., dim].  cnts / average as in hades_adagrad_update
+ * (the reference's update always averages: sparse_optim.py:607-614). */
 int hades_adam_update(const int64_t* uids, const float* grad, const int64_t* num_unique,
                       int64_t max_rows, int64_t dim,
                       const int64_t* sorted_hot, int64_t num_hot, const void* hot_index,
                       float* hot_w, float* hot_step, float* hot_m, float* hot_v,
                       float* cold_w, float* cold_step, float* cold_m, float* cold_v,
+                      const int64_t* cnts, int average,
                       float lr, double beta1, double beta2, float eps, void* stream);
 
 /* The SparseAdam arithmetic of hades_adam_update over one half of a split, against one table

@@ -1385,7 +1385,7 @@ def test_library_pinned_allocation_through_the_c_abi(lib):
         _lib.call("hades_adagrad_update", ctypes.c_void_p(t_uq.data_ptr()), ctypes.c_void_p(t_g.data_ptr()), None,
                   uq.size, D, ctypes.c_void_p(t_hot_ids.data_ptr()), hot_ids.size, None,
                   ctypes.c_void_p(hot_w.data_ptr()), ctypes.c_void_p(hot_s.data_ptr()), raw,
-                  ctypes.c_void_p(cold_s.data_ptr()), 0.01, 1e-10, st)
+                  ctypes.c_void_p(cold_s.data_ptr()), None, 0, 0.01, 1e-10, st)
         torch.cuda.synchronize()
         hw, hs, cs = (want_tab[hot_ids] + 1.0).astype(np.float32), np.zeros((1500, D), np.float32), np.zeros((N, D), np.float32)
         O.sparse_adagrad_step(want_tab, cs, hw, hs, hot_ids, uq, g, 0.01, 1e-10)
@@ -1783,7 +1783,7 @@ def test_keyed_and_split_steps_that_average_like_the_reference(lib, kind, averag
         torch.cuda.synchronize()
         return [t.cpu().numpy().copy() for t in ts]
 
-    keyed, unfused, split = make(), make(), make()
+    keyed, unfused, split, serial = make(), make(), make(), make()
     unfused.fuse_cold_sums = False
     if kind == "adagrad":
         want = [cold.copy(), np.zeros_like(cold), cold[hot_ids].copy(), np.zeros((H, D), np.float32)]
@@ -1797,6 +1797,8 @@ def test_keyed_and_split_steps_that_average_like_the_reference(lib, kind, averag
             _, st = o.forward_keyed(t_q)
             uk, sums, cnts, nu, _ = o.backward_keyed(st, t_g, mode=ops.COMBINE_EXACT, average=average)
         split.step_split(t_q, t_g, mode=ops.COMBINE_EXACT, average=average)
+        if True:
+            serial.step(t_q, t_g, mode=ops.COMBINE_EXACT, average=average)      # one kernel, lookup inside
         if kind == "adagrad":
             wk, ws, wc, _ = O.keyed_step(want[0], want[1], want[2], want[3], hot_ids, q, g, 0.01, 1e-10, kb,
                                          average=average)
@@ -1807,9 +1809,9 @@ def test_keyed_and_split_steps_that_average_like_the_reference(lib, kind, averag
         # the returned rows stay the sums, the counts the occurrences
         assert np.array_equal(uk[:U].cpu().numpy(), wk) and np.array_equal(cnts[:U].cpu().numpy(), wc)
         assert np.array_equal(sums[:U].cpu().numpy(), ws)
-    tk, tu, tsp = tables(keyed), tables(unfused), tables(split)
-    for a, b, c, w in zip(tk, tu, tsp, want):
-        assert np.array_equal(a, b) and np.array_equal(a, c)
+    tk, tu, tsp, tse = tables(keyed), tables(unfused), tables(split), tables(serial)
+    for a, b, c, e, w in zip(tk, tu, tsp, tse, want):
+        assert np.array_equal(a, b) and np.array_equal(a, c) and np.array_equal(a, e)
         if kind == "adagrad":
             assert np.array_equal(a, w)
     if kind == "adam":      # the oracle's Adam is pinned to 1e-4 of one update only (device powf)
