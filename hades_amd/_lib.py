@@ -26,7 +26,7 @@ _L = c_int64
 KERNEL_NONE, KERNEL_CACHED_FETCH, KERNEL_SEG_SUM, KERNEL_ADAGRAD, KERNEL_RADIX_PASS = 0, 1, 2, 3, 4
 KERNEL_HASH_ACCUMULATE = 5
 KERNEL_ADAM = 6
-ABI_VERSION = 130      # HADES_ABI_VERSION of include/hades_hip.h
+ABI_VERSION = 131      # HADES_ABI_VERSION of include/hades_hip.h
 
 _SIGNATURES = {
     "hades_profile_kernel": [c_int, _P, _P],
@@ -106,6 +106,7 @@ _SIZE_QUERIES = {
     "hades_split_compact_workspace_bytes": [_L],
     "hades_hot_index_bytes": [_L],
     "hades_combine_workspace_bytes": [_L, _L],
+    "hades_combine_workspace_bytes_min": [_L, _L],
     "hades_hash_flush_workspace_bytes": [_L, _L],
     "hades_bucket_workspace_bytes": [_L],
     "hades_sacache_workspace_bytes": [_L],

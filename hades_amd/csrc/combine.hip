@@ -794,6 +794,7 @@ struct RowVec<1> {
   static __device__ __forceinline__ type zero() { return 0.f; }
 };
 
+constexpr int kLongRun = 64;     // EXACT: shortest run that is summed by a block of its own
 constexpr int kChunk = 32;       // sorted positions per lane group
 constexpr int kMinGroup = 4;     // lanes per group: power of two in [4, 64]
 constexpr int kMaxGroups = kThreads / kMinGroup;
@@ -817,6 +818,9 @@ struct SegArgs {
   // position, first run} of the upper class; which = 0 lower class, 1 upper class, -1 everything
   const int64_t* class_split;
   int which;
+  // EXACT with a staging area (else null): see seg_stage_kernel
+  float* stage = nullptr;
+  uint32_t* long_list = nullptr;
 };
 
 // [*pos_lo, *pos_hi) sorted positions and [*run_lo, *run_hi) runs of the class a launch works on
@@ -1048,17 +1052,16 @@ __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
 // EXACT: strictly left to right from +0.0f, one accumulator chain per id.
 // Runs shorter than kLongRun: one lane group per distinct id.  Longer runs (a heavy-hitter id can
 // have tens of thousands of occurrences) are left to seg_exact_long_kernel.
-constexpr int kLongRun = 64;    // shortest run the long-run kernel takes
 constexpr int kLongThreads = 1024;  // the long-run kernel's block: one CU has to pull a whole run
                                     // through, so it keeps as many row loads in flight as it can
 constexpr int kLongRows = 8;    // rows every lane group stages per batch in the long-run kernel
 constexpr int kLongSlice = 32;  // floats of a row one block of the long-run kernel sums (128 bytes)
 
 template <int VEC>
-__global__ __launch_bounds__(kThreads) void seg_exact_kernel(SegArgs a) {
+__device__ __forceinline__ void exact_short_runs(const SegArgs& a, int64_t block) {
   typedef typename RowVec<VEC>::type V;
   const int64_t U = a.num_unique[0];
-  const int64_t gtid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t gtid = block * kThreads + threadIdx.x;
   const int64_t u = gtid / a.group;
   const int gl = static_cast<int>(gtid & (a.group - 1));
   int64_t pos_lo, pos_hi, run_lo, run_hi;
@@ -1088,6 +1091,11 @@ __global__ __launch_bounds__(kThreads) void seg_exact_kernel(SegArgs a) {
     }
     *reinterpret_cast<V*>(a.sums + u * a.dim + col) = acc;
   }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void seg_exact_kernel(SegArgs a) {
+  exact_short_runs<VEC>(a, blockIdx.x);
 }
 
 // EXACT, long runs: block c takes the run that begins inside positions [c*kLongRun, (c+1)*kLongRun)
@@ -1178,6 +1186,158 @@ __global__ __launch_bounds__(kLongThreads) void seg_exact_long_kernel(SegArgs a)
     const int64_t c_out = static_cast<int64_t>(blockIdx.y) * kLongSlice + threadIdx.x;
     if (c_out < a.dim) a.sums[static_cast<int64_t>(u) * a.dim + c_out] = accf;
   }
+}
+
+// EXACT, long runs, with a staging area.  One compute unit pulls random rows out of HBM at about a
+// hundred cache lines a microsecond, a chain of dependent adds could take five times as many rows:
+// a block that fetches the rows of its run itself (seg_exact_long_kernel) is bound by its loads,
+// however many it keeps in flight.  So the rows of all long runs are first copied by the whole
+// chip, in sorted order, into column slices of four floats: stage[s][j] (16 bytes) = columns
+// 4s .. 4s + 3 of the row at sorted position j.  A (run, slice) pair is then one contiguous stream
+// in which a cache line carries eight rows, and the block that sums it is bound by its adds.
+// The kernel also lists the long runs: long_list[0] runs of kVeryLongRun rows or more from entry 2
+// upwards, long_list[1] shorter ones from the last entry downwards, each in no particular order
+// (every run is summed on its own).  seg_chain_kernel's blocks take the entries in that order, so
+// the runs that decide its length are begun first.
+constexpr int64_t kVeryLongRun = 2048;
+
+__global__ __launch_bounds__(kThreads) void seg_stage_kernel(SegArgs a) {
+  const int64_t pieces = a.dim / 4;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t j = gid / pieces;
+  const int64_t sl = gid - j * pieces;
+  int64_t pos_lo, pos_hi, run_lo, run_hi;
+  class_range(a, a.num_unique[0], &pos_lo, &pos_hi, &run_lo, &run_hi);
+  if (j < pos_lo || j >= pos_hi) return;
+  const uint32_t u = a.seg_of[j];
+  const int64_t start = a.seg_start[u], end = a.seg_start[u + 1];
+  if (end - start < kLongRun) return;
+  const f32x4 v = __builtin_nontemporal_load(
+      reinterpret_cast<const f32x4*>(a.grad + static_cast<int64_t>(a.perm[j]) * a.dim) + sl);
+  reinterpret_cast<f32x4*>(a.stage)[sl * a.n + j] = v;
+  if (sl == 0 && j == start) {
+    if (end - start >= kVeryLongRun) {
+      a.long_list[2 + atomicAdd(&a.long_list[0], 1u)] = u;
+    } else {
+      const int64_t last_entry = 1 + (a.n + kLongRun - 1) / kLongRun;
+      a.long_list[last_entry - atomicAdd(&a.long_list[1], 1u)] = u;
+    }
+  }
+}
+
+// Sums the staged slice `sl` of the long runs `first`, `first + stride`, ... of the list, in order of
+// occurrence from +0.0f.  All threads copy the stream into LDS, transposed (one array per column),
+// 512 rows a batch, two batches of loads in flight and two LDS buffers; threads 0..3 own a column
+// each and add it with 16-byte LDS loads (four rows), the loads of the next 32 rows in flight
+// while 32 are added.  While they add batch b the others already write batch b + 1.
+constexpr int kChainRows = 2;                        // rows per thread and batch
+constexpr int kChainBatch = kThreads * kChainRows;   // 512
+constexpr int kChainStride = kChainBatch + 4;        // floats between the columns of a buffer
+
+__device__ __forceinline__ void exact_chain_runs(const SegArgs& a, float (&s_buf)[2][4 * kChainStride],
+                                                 int64_t sl, uint32_t first, uint32_t stride) {
+  const uint32_t very_long = a.long_list[0], count = very_long + a.long_list[1];
+  const int64_t last_entry = 1 + (a.n + kLongRun - 1) / kLongRun;
+  const f32x4* slice = reinterpret_cast<const f32x4*>(a.stage) + sl * a.n;
+  const bool adder = threadIdx.x < 4;
+  for (uint32_t li = first; li < count; li += stride) {
+    const uint32_t u = li < very_long ? a.long_list[2 + li] : a.long_list[last_entry - (li - very_long)];
+    const int64_t start = a.seg_start[u];
+    const int64_t len = a.seg_start[u + 1] - start;
+    const f32x4* src = slice + start;
+    float accf = 0.f;
+    f32x4 rows_a[kChainRows], rows_b[kChainRows];
+    auto issue_rows = [&](f32x4 (&rows)[kChainRows], int64_t base) {
+#pragma unroll
+      for (int k = 0; k < kChainRows; ++k) {
+        const int64_t r = base + k * kThreads + threadIdx.x;
+        rows[k] = r < len ? __builtin_nontemporal_load(src + r) : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+    };
+    auto stage = [&](const f32x4 (&rows)[kChainRows], float* buf) {
+#pragma unroll
+      for (int k = 0; k < kChainRows; ++k) {
+        const int r = k * kThreads + threadIdx.x;
+        buf[0 * kChainStride + r] = rows[k].x;
+        buf[1 * kChainStride + r] = rows[k].y;
+        buf[2 * kChainStride + r] = rows[k].z;
+        buf[3 * kChainStride + r] = rows[k].w;
+      }
+    };
+    auto add_batch = [&](const float* buf, int rows_here) {
+      const float* colp = buf + threadIdx.x * kChainStride;
+      constexpr int kUnits = 8;                  // 16-byte loads (four rows each) per register set
+      f32x4 qa[kUnits], qb[kUnits];
+      auto rd = [&](f32x4 (&q)[kUnits], int row0) {
+#pragma unroll
+        for (int k = 0; k < kUnits; ++k) q[k] = *reinterpret_cast<const f32x4*>(colp + row0 + 4 * k);
+      };
+      auto ad = [&](const f32x4 (&q)[kUnits]) {
+#pragma unroll
+        for (int k = 0; k < kUnits; ++k) {
+          accf += q[k].x;
+          accf += q[k].y;
+          accf += q[k].z;
+          accf += q[k].w;
+        }
+      };
+      const int nsets = rows_here / (4 * kUnits);   // whole register sets: 32 rows each
+      int sidx = 0;
+      if (nsets > 0) rd(qa, 0);
+      while (sidx < nsets) {
+        if (sidx + 1 < nsets) rd(qb, (sidx + 1) * 4 * kUnits);
+        ad(qa);
+        if (++sidx >= nsets) break;
+        if (sidx + 1 < nsets) rd(qa, (sidx + 1) * 4 * kUnits);
+        ad(qb);
+        ++sidx;
+      }
+      for (int r = nsets * 4 * kUnits; r < rows_here; ++r) accf += colp[r];
+    };
+    // step b: batch b (loaded two steps earlier) goes to LDS buffer b & 1, the loads of batch
+    // b + 2 are issued, and after the barrier the column threads add batch b - while the others
+    // go on to write batch b + 1 into the other buffer, which the column threads left before
+    // they reached this barrier
+    auto step = [&](f32x4 (&rows)[kChainRows], float* buf, int64_t base) {
+      stage(rows, buf);
+      if (base + 2 * kChainBatch < len) issue_rows(rows, base + 2 * kChainBatch);
+      __syncthreads();
+      if (adder) {
+        const int64_t left = len - base;
+        add_batch(buf, left < kChainBatch ? static_cast<int>(left) : kChainBatch);
+      }
+    };
+    issue_rows(rows_a, 0);
+    issue_rows(rows_b, kChainBatch);
+    for (int64_t base = 0; base < len; base += 2 * kChainBatch) {
+      step(rows_a, s_buf[0], base);
+      if (base + kChainBatch < len) step(rows_b, s_buf[1], base + kChainBatch);
+    }
+    if (adder)
+      a.sums[static_cast<int64_t>(u) * a.dim + sl * 4 + threadIdx.x] = accf;
+    __syncthreads();   // the buffers are rewritten for the next run of the list
+  }
+}
+
+// The last kernel of the staged EXACT sum.  Its first pieces * chain_blocks blocks sum the long
+// runs: block b takes slice b % pieces of the list entries b / pieces, b / pieces + chain_blocks,
+// ... - blocks are handed out in the order of their index, so all slices of the first (longest)
+// runs start before anything else.  The blocks after them sum the short runs, one lane group per
+// run, on the compute units that the few long chains leave idle.
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void seg_exact_staged_kernel(SegArgs a, uint32_t pieces,
+                                                                   uint32_t chain_blocks) {
+  __shared__ __align__(16) float s_buf[2][4 * kChainStride];
+  const uint32_t nchain = pieces * chain_blocks;
+  if (blockIdx.x < nchain) {
+    exact_chain_runs(a, s_buf, blockIdx.x % pieces, blockIdx.x / pieces, chain_blocks);
+  } else {
+    exact_short_runs<VEC>(a, static_cast<int64_t>(blockIdx.x - nchain));
+  }
+}
+
+__global__ void clear_u32x2_kernel(uint32_t* p) {
+  if (blockIdx.x == 0 && threadIdx.x < 2) p[threadIdx.x] = 0;
 }
 
 __global__ __launch_bounds__(kThreads) void rows_div_kernel(float* __restrict__ sums,
@@ -1279,7 +1439,12 @@ struct Ws {
   uint32_t* seg_of;
   uint32_t* seg_start;
   float* partial;
-  size_t bytes;
+  uint32_t* long_list;  // [2][2 + ceil(n / kLongRun)]: the long runs of the EXACT sum, see
+                        // seg_stage_kernel; the lower class of a classed plan has the second list
+  size_t bytes_min;     // what every entry point needs
+  float* stage;         // [n * dim]: the rows of the long runs in column slices (EXACT sum); last,
+                        // so that a workspace of bytes_min simply lacks it
+  size_t bytes;         // with the staging area
 };
 
 Ws carve(void* ws, int64_t n, int64_t dim) {
@@ -1292,6 +1457,9 @@ Ws carve(void* ws, int64_t n, int64_t dim) {
   w.seg_start = c.take<uint32_t>(nn + 1);
   // at most two partial rows per block of the FAST sum; the smallest block span is 128 positions
   w.partial = c.take<float>(2 * ceil_div(nn, (kThreads / 64) * kChunk) * dim);
+  w.long_list = c.take<uint32_t>(2 * (2 + ceil_div(nn, kLongRun)));
+  w.bytes_min = c.total();
+  w.stage = c.take<float>(static_cast<size_t>(nn) * dim);
   w.bytes = c.total();
   return w;
 }
@@ -1482,9 +1650,9 @@ int combine_plan_views(void* workspace, size_t workspace_bytes, int64_t n, int64
   HADES_REQUIRE(n >= 1 && n < (int64_t(1) << 30) && dim >= 1 && id_bound >= 0, "bad plan shape");
   const Plan p = make_plan(n, dim, id_bound, true);
   const Ws w = carve(workspace, n, dim);
-  if (workspace == nullptr || workspace_bytes < w.bytes)
+  if (workspace == nullptr || workspace_bytes < w.bytes_min)
     return set_error(HADES_ERR_WORKSPACE, "combine workspace too small: need %zu bytes, got %zu",
-                     w.bytes, workspace_bytes);
+                     w.bytes_min, workspace_bytes);
   HADES_REQUIRE((align_of_ptr(workspace) & 255) == 0, "workspace must be 256-byte aligned");
   *perm = w.sort.vals[(p.passes - 1) & 1];   // where the last pass of the plan left the positions
   *seg_start = w.seg_start;
@@ -1511,6 +1679,11 @@ int hades_sort_mode(void) { return g_one_sweep.load(std::memory_order_relaxed); 
 size_t hades_combine_workspace_bytes(int64_t n, int64_t dim) {
   if (n < 0 || dim < 1) return 0;
   return carve(nullptr, n, dim).bytes;
+}
+
+size_t hades_combine_workspace_bytes_min(int64_t n, int64_t dim) {
+  if (n < 0 || dim < 1) return 0;
+  return carve(nullptr, n, dim).bytes_min;
 }
 
 namespace {
@@ -1540,9 +1713,9 @@ int combine_plan_impl(const int64_t* idx, int64_t n, int64_t dim, int64_t id_bou
   HADES_REQUIRE(idx && uids, "null pointer argument");
   const Plan p = make_plan(n, dim, id_bound, true);
   const Ws w = carve(workspace, n, dim);
-  if (workspace == nullptr || workspace_bytes < w.bytes)
+  if (workspace == nullptr || workspace_bytes < w.bytes_min)
     return set_error(HADES_ERR_WORKSPACE, "combine workspace too small: need %zu bytes, got %zu",
-                     w.bytes, workspace_bytes);
+                     w.bytes_min, workspace_bytes);
   HADES_REQUIRE((align_of_ptr(workspace) & 255) == 0, "workspace must be 256-byte aligned");
 
   const uint32_t* perm = nullptr;
@@ -1596,11 +1769,13 @@ int combine_apply_impl(const float* grad, int64_t n, int64_t dim, int64_t id_bou
   const bool aligned = (align_of_ptr(grad) % 16) == 0 && (align_of_ptr(sums) % 16) == 0;
   const Plan p = make_plan(n, dim, id_bound, aligned);
   const Ws w = carve(workspace, n, dim);
-  if (workspace == nullptr || workspace_bytes < w.bytes)
+  if (workspace == nullptr || workspace_bytes < w.bytes_min)
     return set_error(HADES_ERR_WORKSPACE, "combine workspace too small: need %zu bytes, got %zu",
-                     w.bytes, workspace_bytes);
+                     w.bytes_min, workspace_bytes);
   HADES_REQUIRE((align_of_ptr(workspace) & 255) == 0, "workspace must be 256-byte aligned");
 
+  // a workspace of the full size has the staging area of the EXACT sum behind everything else
+  const bool staged = workspace_bytes >= w.bytes;
   SegArgs a;
   a.grad = grad;
   a.perm = w.sort.vals[(p.passes - 1) & 1];  // where the last pass of the plan left the positions
@@ -1624,7 +1799,23 @@ int combine_apply_impl(const float* grad, int64_t n, int64_t dim, int64_t id_bou
     if (timed) HADES_HIP_TRY(hipEventRecord(g_profile.start, st));
     const dim3 lgrid(static_cast<unsigned>(ceil_div(n, kLongRun)),
                      static_cast<unsigned>(ceil_div(dim, kLongSlice)));
-    if (p.vec == 4) {
+    if (p.vec == 4 && staged) {
+      // the rows of the long runs into column slices (and the runs into a list), then one kernel
+      // with a chain of adds per long run and slice, and the short runs beside them
+      a.stage = w.stage;   // indexed by sorted position: the classes of a classed plan do not meet
+      a.long_list = w.long_list + (a.which == 0 ? 2 + ceil_div(n, kLongRun) : 0);
+      const int64_t pieces = dim / 4;
+      const int64_t sblocks = ceil_div(n * pieces, kThreads);
+      int64_t cblocks = ceil_div(n, kLongRun);   // no more long runs than this
+      if (cblocks > 512) cblocks = 512;
+      HADES_REQUIRE(sblocks < (int64_t(1) << 31) && blocks + pieces * cblocks < (int64_t(1) << 31),
+                    "combine: too many rows");
+      HADES_LAUNCH(clear_u32x2_kernel, dim3(1), dim3(64), 0, st, a.long_list);
+      HADES_LAUNCH(seg_stage_kernel, dim3((unsigned)sblocks), dim3(kThreads), 0, st, a);
+      HADES_LAUNCH((seg_exact_staged_kernel<4>), dim3((unsigned)(blocks + pieces * cblocks)),
+                   dim3(kThreads), 0, st, a, static_cast<uint32_t>(pieces),
+                   static_cast<uint32_t>(cblocks));
+    } else if (p.vec == 4) {
       // 128 KB of dynamic LDS: above the default limit, which has to be raised once per device
       constexpr int kLongLds = kLongThreads * kLongRows * sizeof(f32x4);  // a batch of row slices
       static std::atomic<uint64_t> raised{0};  // bit d: done on device d
@@ -1702,7 +1893,7 @@ int hades_combine_static(const int64_t* idx, const float* grad, int64_t n, int64
                          int64_t id_bound, int mode, int64_t* uids, float* sums, int64_t* cnts,
                          int64_t* num_unique, int32_t* inverse, void* stream) {
   HADES_REQUIRE(n >= 0 && dim >= 1, "n must be >= 0 and dim >= 1");
-  const size_t need = hades_combine_workspace_bytes(n, dim);
+  const size_t need = hades_combine_workspace_bytes_min(n, dim);
   HADES_REQUIRE(need <= size_t(HADES_COMBINE_STATIC_SCRATCH_BYTES),
                 "hades_combine_static: n=%lld rows of dim=%lld need %zu bytes of scratch, the "
                 "library holds %zu; use hades_combine with a workspace of your own",

@@ -55,7 +55,7 @@ extern "C" {
 const char* hades_last_error(void);
 /* Version of this interface; raised whenever a signature changes, so that a binding can refuse a
  * library built from other sources. */
-#define HADES_ABI_VERSION 130
+#define HADES_ABI_VERSION 131
 int hades_version(void);
 
 /* Kernel timing hook (no counterpart in the reference, whose scripts time whole calls from the
@@ -297,8 +297,15 @@ int hades_fetch_listed_in_set(const void* src, int64_t src_stride, const int64_t
  * Optional output (may be NULL): inverse[i] = index of idx[i] in uids (int32[n]).
  * If an id violates id_bound, num_unique[0] is set to -1 and the other outputs are unspecified;
  * every operator of this library that takes num_unique treats a negative value as "no live rows",
- * so nothing is read or written out of range downstream.  The workspace needs no initialisation. */
+ * so nothing is read or written out of range downstream.  The workspace needs no initialisation.
+ * hades_combine_workspace_bytes is the size to allocate; its tail (n x dim floats) is a staging
+ * area in which HADES_COMBINE_EXACT lays out the rows of ids that occur 64 times or more, so that
+ * their sums are bound by the chain of adds and not by one compute unit's row loads.  A workspace
+ * of hades_combine_workspace_bytes_min (everything but that area) is accepted by every entry point
+ * that takes a combine workspace; EXACT then sums such ids about three times more slowly, with
+ * the same result. */
 size_t hades_combine_workspace_bytes(int64_t n, int64_t dim);
+size_t hades_combine_workspace_bytes_min(int64_t n, int64_t dim);
 int hades_combine(const int64_t* idx, const float* grad, int64_t n, int64_t dim, int64_t id_bound,
                   int mode, int64_t* uids, float* sums, int64_t* cnts, int64_t* num_unique,
                   int32_t* inverse, void* workspace, size_t workspace_bytes, void* stream);
@@ -359,7 +366,7 @@ int hades_combine_apply_class(const float* grad, int64_t n, int64_t dim, int64_t
  * capture, tight serving loops, harnesses that forbid hipMalloc.  The call allocates and frees
  * nothing; its scratch is a fixed array of HADES_COMBINE_STATIC_SCRATCH_BYTES that every GPU the
  * library runs on holds until the process ends.  Same arguments and results as hades_combine
- * without the workspace pair.  A batch whose hades_combine_workspace_bytes(n, dim) exceeds the
+ * without the workspace pair.  A batch whose hades_combine_workspace_bytes_min(n, dim) exceeds the
  * array is refused with HADES_ERR_ARG (the limit admits e.g. 262 144 ids of dim 128).  All calls
  * on one GPU share that GPU's array: two calls that overlap in time on one GPU (different streams
  * or threads) race, and the array must not be relied on between calls.  The first call on a

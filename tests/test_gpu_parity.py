@@ -619,6 +619,51 @@ def test_combine(lib, sort_form, n, dim, space, kind, bounded):
         assert np.array_equal(got[short], ws[short])
 
 
+@pytest.mark.parametrize("dim", [4, 20, 64, 128, 7])
+def test_exact_combine_long_runs_with_and_without_the_staging_area(lib, dim):
+    """Deterministic-order sums of ids that occur 64 times or more: run lengths around the 64-row
+    threshold and around the 1 024-row batches of the staged chain (one and two batches, one row
+    more and less), a run of 40 000 rows, short runs between them, rows in shuffled batch order.
+    With the full workspace the rows of the long runs are staged in column slices and summed by
+    one chain per slice; with a workspace of hades_combine_workspace_bytes_min the block of a run
+    fetches its rows itself.  Both equal the oracle's left-to-right sums bit for bit (dim 7: rows
+    that cannot be read 16 bytes at a time take the second way whatever the workspace)."""
+    from hades_amd import _lib
+    _, ops = lib
+    rng = np.random.default_rng(dim)
+    lens = [63, 64, 65, 1, 1023, 1024, 1025, 7, 2047, 2048, 2049, 3, 3000, 40_000, 2, 100, 5000]
+    idx = np.repeat(np.arange(len(lens), dtype=np.int64) * 11 + 5, lens)
+    rng.shuffle(idx)
+    n = idx.size
+    grad = (rng.standard_normal((n, dim)) * 1e-3).astype(np.float32)
+    wu, ws, wc = O.combine_sequential(idx, grad)
+    t_idx, t_grad = dev(idx), dev(grad)
+    full = _lib.query("hades_combine_workspace_bytes", n, dim)
+    least = _lib.query("hades_combine_workspace_bytes_min", n, dim)
+    assert full - least >= n * dim * 4
+    st = torch.cuda.current_stream().cuda_stream
+    for nbytes in (full, least):
+        wsb = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        uids = torch.empty(n, dtype=torch.int64, device="cuda")
+        sums = torch.full((n, dim), float("nan"), device="cuda")
+        cnts = torch.empty(n, dtype=torch.int64, device="cuda")
+        nu = torch.empty(1, dtype=torch.int64, device="cuda")
+        for _ in range(2):      # the second call finds the list of long runs of the first one
+            _lib.call("hades_combine", t_idx.data_ptr(), t_grad.data_ptr(), n, dim, 1000, ops.COMBINE_EXACT,
+                      uids.data_ptr(), sums.data_ptr(), cnts.data_ptr(), nu.data_ptr(), None,
+                      wsb.data_ptr(), nbytes, st)
+        torch.cuda.synchronize()
+        U = int(nu.item())
+        assert U == wu.size and np.array_equal(uids[:U].cpu().numpy(), wu)
+        assert np.array_equal(cnts[:U].cpu().numpy(), wc)
+        assert np.array_equal(sums[:U].cpu().numpy(), ws)
+    # one byte less than the minimum is refused
+    rc = _lib.load().hades_combine(t_idx.data_ptr(), t_grad.data_ptr(), n, dim, 1000, ops.COMBINE_EXACT,
+                                   uids.data_ptr(), sums.data_ptr(), cnts.data_ptr(), nu.data_ptr(), None,
+                                   wsb.data_ptr(), least - 1, st)
+    assert rc != 0
+
+
 @pytest.mark.parametrize("n,space,bounded", [(5000, 300, True), (70_001, 5000, True), (262_145, 3_000_000, True),
                                              (150_000, 40, True), (100_000, 2_400_000, False)])
 def test_one_sweep_sort_when_its_waits_run_out(lib, n, space, bounded):

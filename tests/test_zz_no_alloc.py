@@ -75,11 +75,11 @@ def test_combine_static_limits_and_bound_flag(cuda_device):
     lib = _lib.load()
     # a batch that needs more scratch than the library holds is refused, nothing is launched
     n, dim = 1_000_000, 128
-    assert _lib.query("hades_combine_workspace_bytes", n, dim) > _lib.COMBINE_STATIC_SCRATCH_BYTES
+    assert _lib.query("hades_combine_workspace_bytes_min", n, dim) > _lib.COMBINE_STATIC_SCRATCH_BYTES
     rc = lib.hades_combine_static(None, None, n, dim, 0, 0, None, None, None, None, None, None)
     assert rc == 1 and b"scratch" in lib.hades_last_error()
     # the largest single-trainer batch of the benchmark configurations fits
-    assert _lib.query("hades_combine_workspace_bytes", 262_144, 128) <= _lib.COMBINE_STATIC_SCRATCH_BYTES
+    assert _lib.query("hades_combine_workspace_bytes_min", 262_144, 128) <= _lib.COMBINE_STATIC_SCRATCH_BYTES
     # an id beyond id_bound: -1 distinct ids on this call, and no trace of it on the next one
     idx = torch.arange(5000, dtype=torch.int64, device="cuda") % 100
     grad = torch.ones((5000, 8), device="cuda")
