@@ -15,9 +15,12 @@
 //      reads five count rows whatever the batch size.
 //   2. run boundaries -> uids, seg_start, seg_of (index of the run every sorted position is in).
 //   3. segmented sum of the gradient rows:
-//        EXACT: one lane group per distinct id walks its rows left to right; a run of 64 rows or
-//               more is staged through LDS by 1024-thread blocks, one per 32-float column slice,
-//               and added in the same order by one thread per column.
+//        EXACT: one lane group per distinct id walks its rows left to right.  The rows of a run
+//               of 64 rows or more are first copied, by the whole chip, into four-float column
+//               slices of a staging area at the end of the workspace; a block per run and slice
+//               then streams its slice through LDS and one thread per column adds it in the same
+//               order (without the staging area: 1024-thread blocks fetch the rows of their run
+//               themselves, one block per 32-float column slice).
 //        FAST : the sorted sequence is cut into fixed chunks of 32 positions per lane group; a
 //               block stages the sort permutation of its groups in LDS, every group sums its
 //               runs left to right with 16 row loads in flight, runs that cross group borders
