@@ -1810,7 +1810,7 @@ int combine_apply_impl(const float* grad, int64_t n, int64_t dim, int64_t id_bou
       const int64_t pieces = dim / 4;
       const int64_t sblocks = ceil_div(n * pieces, kThreads);
       int64_t cblocks = ceil_div(n, kLongRun);   // no more long runs than this
-      if (cblocks > 512) cblocks = 512;
+      if (cblocks > 128) cblocks = 128;
       HADES_REQUIRE(sblocks < (int64_t(1) << 31) && blocks + pieces * cblocks < (int64_t(1) << 31),
                     "combine: too many rows");
       HADES_LAUNCH(clear_u32x2_kernel, dim3(1), dim3(64), 0, st, a.long_list);
