@@ -1204,28 +1204,49 @@ __global__ __launch_bounds__(kLongThreads) void seg_exact_long_kernel(SegArgs a)
 // the runs that decide its length are begun first.
 constexpr int64_t kVeryLongRun = 2048;
 
+constexpr int kStagePieces = 4;   // 16-byte pieces per thread: four chains of dependent loads in flight
+
 __global__ __launch_bounds__(kThreads) void seg_stage_kernel(SegArgs a) {
   const int64_t pieces = a.dim / 4;
-  const int64_t gid = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  const int64_t j = gid / pieces;
-  const int64_t sl = gid - j * pieces;
   int64_t pos_lo, pos_hi, run_lo, run_hi;
   class_range(a, a.num_unique[0], &pos_lo, &pos_hi, &run_lo, &run_hi);
-  if (j < pos_lo || j >= pos_hi) return;
-  const uint32_t u = a.seg_of[j];
-  const int64_t start = a.seg_start[u], end = a.seg_start[u + 1];
-  if (end - start < kLongRun) return;
-  const f32x4 v = __builtin_nontemporal_load(
-      reinterpret_cast<const f32x4*>(a.grad + static_cast<int64_t>(a.perm[j]) * a.dim) + sl);
-  reinterpret_cast<f32x4*>(a.stage)[sl * a.n + j] = v;
-  if (sl == 0 && j == start) {
-    if (end - start >= kVeryLongRun) {
-      a.long_list[2 + atomicAdd(&a.long_list[0], 1u)] = u;
-    } else {
-      const int64_t last_entry = 1 + (a.n + kLongRun - 1) / kLongRun;
-      a.long_list[last_entry - atomicAdd(&a.long_list[1], 1u)] = u;
+  const int64_t gid0 = static_cast<int64_t>(blockIdx.x) * (kThreads * kStagePieces) + threadIdx.x;
+  int64_t j[kStagePieces], sl[kStagePieces];
+  uint32_t u[kStagePieces], p[kStagePieces];
+  bool live[kStagePieces];
+#pragma unroll
+  for (int k = 0; k < kStagePieces; ++k) {
+    const int64_t gid = gid0 + k * kThreads;
+    j[k] = gid / pieces;
+    sl[k] = gid - j[k] * pieces;
+    live[k] = j[k] >= pos_lo && j[k] < pos_hi;
+    u[k] = live[k] ? a.seg_of[j[k]] : 0u;
+    p[k] = live[k] ? a.perm[j[k]] : 0u;
+  }
+  int64_t start[kStagePieces];
+#pragma unroll
+  for (int k = 0; k < kStagePieces; ++k) {
+    start[k] = live[k] ? a.seg_start[u[k]] : 0;
+    const int64_t end = live[k] ? a.seg_start[u[k] + 1] : 0;
+    live[k] = live[k] && end - start[k] >= kLongRun;
+    if (live[k] && sl[k] == 0 && j[k] == start[k]) {
+      if (end - start[k] >= kVeryLongRun) {
+        a.long_list[2 + atomicAdd(&a.long_list[0], 1u)] = u[k];
+      } else {
+        const int64_t last_entry = 1 + (a.n + kLongRun - 1) / kLongRun;
+        a.long_list[last_entry - atomicAdd(&a.long_list[1], 1u)] = u[k];
+      }
     }
   }
+  f32x4 v[kStagePieces];
+#pragma unroll
+  for (int k = 0; k < kStagePieces; ++k)
+    if (live[k])
+      v[k] = __builtin_nontemporal_load(
+          reinterpret_cast<const f32x4*>(a.grad + static_cast<int64_t>(p[k]) * a.dim) + sl[k]);
+#pragma unroll
+  for (int k = 0; k < kStagePieces; ++k)
+    if (live[k]) reinterpret_cast<f32x4*>(a.stage)[sl[k] * a.n + j[k]] = v[k];
 }
 
 // Sums the staged slice `sl` of the long runs `first`, `first + stride`, ... of the list, in order of
@@ -1808,7 +1829,7 @@ int combine_apply_impl(const float* grad, int64_t n, int64_t dim, int64_t id_bou
       a.stage = w.stage;   // indexed by sorted position: the classes of a classed plan do not meet
       a.long_list = w.long_list + (a.which == 0 ? 2 + ceil_div(n, kLongRun) : 0);
       const int64_t pieces = dim / 4;
-      const int64_t sblocks = ceil_div(n * pieces, kThreads);
+      const int64_t sblocks = ceil_div(n * pieces, kThreads * kStagePieces);
       int64_t cblocks = ceil_div(n, kLongRun);   // no more long runs than this
       if (cblocks > 128) cblocks = 128;
       HADES_REQUIRE(sblocks < (int64_t(1) << 31) && blocks + pieces * cblocks < (int64_t(1) << 31),
