@@ -798,7 +798,7 @@ struct RowVec<1> {
 };
 
 constexpr int kLongRun = 64;     // EXACT: shortest run that is summed by a block of its own
-constexpr int kChunk = 32;       // sorted positions per lane group
+constexpr int kChunk = 32;       // sorted positions per lane group (large batches; see seg_chunk_for)
 constexpr int kMinGroup = 4;     // lanes per group: power of two in [4, 64]
 constexpr int kMaxGroups = kThreads / kMinGroup;
 constexpr int kSegUnroll = 16;   // row loads in flight per lane
@@ -837,19 +837,20 @@ __device__ __forceinline__ void class_range(const SegArgs& a, int64_t U, int64_t
   }
 }
 
-// FAST, kernel 1.  A block covers (kThreads / group) * kChunk consecutive sorted positions.
-template <int VEC>
+// FAST, kernel 1.  A block covers (kThreads / group) * CH consecutive sorted positions.
+template <int VEC, int CH>
 __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
   typedef typename RowVec<VEC>::type V;
-  __shared__ uint32_t s_perm[kMaxGroups * kChunk];
-  __shared__ uint32_t s_seg[kMaxGroups * kChunk + 2];   // s_seg[1 + t] = run of position B0 + t
+  constexpr int kUnroll = CH < kSegUnroll ? CH : kSegUnroll;   // row loads in flight per lane
+  __shared__ uint32_t s_perm[kMaxGroups * CH];
+  __shared__ uint32_t s_seg[kMaxGroups * CH + 2];   // s_seg[1 + t] = run of position B0 + t
   __shared__ V s_part[kThreads * 2];                    // [group][first|last][lane]
   __shared__ uint32_t s_first[kMaxGroups], s_last[kMaxGroups];
   __shared__ uint8_t s_flags[kMaxGroups];               // 1 head open, 2 tail open, 4 active
 
   const int G = a.group;
   const int ngroups = kThreads / G;
-  const int bp = ngroups * kChunk;
+  const int bp = ngroups * CH;
   const int64_t B0 = static_cast<int64_t>(blockIdx.x) * bp;
   // runs [run_lo, run_hi) are this launch's to write
   uint32_t run_lo = 0, run_hi = kNoRun;
@@ -874,9 +875,9 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
 
   const int g = threadIdx.x / G;
   const int gl = threadIdx.x & (G - 1);
-  const int t0 = g * kChunk;                       // block-relative first position of the group
+  const int t0 = g * CH;                       // block-relative first position of the group
   const int64_t left = a.n - (B0 + t0);
-  const int len = left >= kChunk ? kChunk : (left > 0 ? static_cast<int>(left) : 0);
+  const int len = left >= CH ? CH : (left > 0 ? static_cast<int>(left) : 0);
   const bool active = len > 0;
   const uint32_t first_run = s_seg[1 + t0];
   const uint32_t last_run = active ? s_seg[t0 + len] : kNoRun;
@@ -893,10 +894,10 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
     const bool col_ok = col < a.dim;
     V acc = RowVec<VEC>::zero();
     uint32_t cur = first_run;
-    for (int tt = 0; tt < len; tt += kSegUnroll) {
-      V row[kSegUnroll];
+    for (int tt = 0; tt < len; tt += kUnroll) {
+      V row[kUnroll];
 #pragma unroll
-      for (int k = 0; k < kSegUnroll; ++k) {
+      for (int k = 0; k < kUnroll; ++k) {
         // clamped, so that every slot loads a valid row and the loads form one straight run of
         // instructions; gradient rows are read exactly once: non-temporal loads keep them from
         // displacing the table rows the neighbouring kernels reuse (measured 41.6 -> 32.0 us)
@@ -907,7 +908,7 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
                         : RowVec<VEC>::zero();
       }
 #pragma unroll
-      for (int k = 0; k < kSegUnroll; ++k) {
+      for (int k = 0; k < kUnroll; ++k) {
         if (tt + k < len) {
           const uint32_t seg = s_seg[1 + t0 + tt + k];
           if (seg != cur) {
@@ -990,7 +991,7 @@ __global__ __launch_bounds__(kThreads) void seg_chunk_kernel(SegArgs a) {
 // FAST, kernel 2: block c finishes the run that begins in block c's span and crosses into the
 // next one, adding the per-block partial rows in block order (lane groups take partials
 // round-robin, then group 0 adds the per-group sums in group order).  Also writes the counts.
-template <int VEC>
+template <int VEC, int CH>
 __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
   typedef typename RowVec<VEC>::type V;
   __shared__ V s_part[kThreads];
@@ -1003,7 +1004,7 @@ __global__ __launch_bounds__(kThreads) void seg_fixup_kernel(SegArgs a) {
 
   const int G = a.group;
   const int ngroups = kThreads / G;
-  const int64_t span = static_cast<int64_t>(ngroups) * kChunk;
+  const int64_t span = static_cast<int64_t>(ngroups) * CH;
   const int64_t c = blockIdx.x;
   const int64_t border = (c + 1) * span;
   if (border >= a.n) return;
@@ -1389,8 +1390,18 @@ struct Plan {
   int col_tiles;
   int64_t ntiles;        // radix tiles
   int64_t nblocks_runs;
+  int chunk;             // sorted positions per lane group of the FAST segmented sum
   int64_t nblocks_seg;   // blocks of the FAST segmented sum
 };
+
+// Sorted positions per lane group of the FAST sum.  A small batch gives a chunk of 32 only a
+// hundred-odd blocks, each a chain of two rounds of row loads: shorter chunks make more and
+// shorter blocks.  The shape of the sum stays a function of (n, dim) alone.
+int seg_chunk_for(int64_t n) {
+  static const int env = [] { const char* e = getenv("HADES_SEG_CHUNK"); return e ? atoi(e) : 0; }();
+  if (env == 8 || env == 16 || env == 32) return env;
+  return n <= (int64_t(1) << 17) ? 8 : kChunk;
+}
 
 Plan make_plan(int64_t n, int64_t dim, int64_t id_bound, bool grad_aligned) {
   Plan p;
@@ -1415,7 +1426,8 @@ Plan make_plan(int64_t n, int64_t dim, int64_t id_bound, bool grad_aligned) {
   p.group = g;
   p.col_tiles = static_cast<int>((lanes + g - 1) / g);
   p.nblocks_runs = ceil_div(nn, kUTile);
-  p.nblocks_seg = ceil_div(nn, static_cast<int64_t>(kThreads / g) * kChunk);
+  p.chunk = seg_chunk_for(nn);
+  p.nblocks_seg = ceil_div(nn, static_cast<int64_t>(kThreads / g) * p.chunk);
   return p;
 }
 
@@ -1479,8 +1491,8 @@ Ws carve(void* ws, int64_t n, int64_t dim) {
   w.run_cnt = c.take<uint32_t>(ceil_div(nn, kUTile) + 1);
   w.seg_of = c.take<uint32_t>(nn);
   w.seg_start = c.take<uint32_t>(nn + 1);
-  // at most two partial rows per block of the FAST sum; the smallest block span is 128 positions
-  w.partial = c.take<float>(2 * ceil_div(nn, (kThreads / 64) * kChunk) * dim);
+  // at most two partial rows per block of the FAST sum; the smallest block span is four chunks
+  w.partial = c.take<float>(2 * ceil_div(nn, (kThreads / 64) * seg_chunk_for(nn)) * dim);
   w.long_list = c.take<uint32_t>(2 * (2 + ceil_div(nn, kLongRun)));
   w.bytes_min = c.total();
   w.stage = c.take<float>(static_cast<size_t>(nn) * dim);
@@ -1862,20 +1874,26 @@ int combine_apply_impl(const float* grad, int64_t n, int64_t dim, int64_t id_bou
   } else {
     HADES_REQUIRE(p.nblocks_seg < (int64_t(1) << 31), "combine: too many rows");
     const dim3 grid(static_cast<unsigned>(p.nblocks_seg));
-    if (p.vec == 4)
-      HADES_LAUNCH_TIMED(HADES_KERNEL_SEG_SUM, st, (seg_chunk_kernel<4>), grid, dim3(kThreads), 0,
-                         st, a);
-    else
-      HADES_LAUNCH_TIMED(HADES_KERNEL_SEG_SUM, st, (seg_chunk_kernel<1>), grid, dim3(kThreads), 0,
-                         st, a);
-    HADES_LAUNCH_CHECK();
-    // one block per span of the chunk kernel, and at least one thread per sorted position so that
-    // every u < U <= n gets its count written
+    // one block of the second kernel per span of the first, and at least one thread per sorted
+    // position so that every u < U <= n gets its count written
     const int64_t fblocks = p.nblocks_seg > ceil_div(n, kThreads) ? p.nblocks_seg : ceil_div(n, kThreads);
-    if (p.vec == 4)
-      HADES_LAUNCH((seg_fixup_kernel<4>), dim3((unsigned)fblocks), dim3(kThreads), 0, st, a);
-    else
-      HADES_LAUNCH((seg_fixup_kernel<1>), dim3((unsigned)fblocks), dim3(kThreads), 0, st, a);
+#define HADES_FAST_SUM(VEC_, CH_)                                                                   \
+  do {                                                                                              \
+    HADES_LAUNCH_TIMED(HADES_KERNEL_SEG_SUM, st, (seg_chunk_kernel<VEC_, CH_>), grid,               \
+                       dim3(kThreads), 0, st, a);                                                   \
+    HADES_LAUNCH_CHECK();                                                                           \
+    HADES_LAUNCH((seg_fixup_kernel<VEC_, CH_>), dim3((unsigned)fblocks), dim3(kThreads), 0, st, a); \
+  } while (0)
+    if (p.vec == 4) {
+      if (p.chunk == 8) HADES_FAST_SUM(4, 8);
+      else if (p.chunk == 16) HADES_FAST_SUM(4, 16);
+      else HADES_FAST_SUM(4, 32);
+    } else {
+      if (p.chunk == 8) HADES_FAST_SUM(1, 8);
+      else if (p.chunk == 16) HADES_FAST_SUM(1, 16);
+      else HADES_FAST_SUM(1, 32);
+    }
+#undef HADES_FAST_SUM
     HADES_LAUNCH_CHECK();
   }
   return HADES_OK;
