@@ -50,7 +50,12 @@ constexpr int kBins = 1 << kRadixBits;
 constexpr int kMaxPasses = 8;
 constexpr int kGroup = 4;  // tiles counted by one block of the count kernel
 constexpr int kIpt = 4;    // keys per thread in a radix tile: tiles of 1024 keys
+constexpr int kIptSmall = 2;             // ... tiles of 512 keys for batches of up to kSmallBatch ids:
+constexpr int64_t kSmallBatch = 1 << 17; // they would leave three quarters of the chip without a tile
 constexpr int kScanFrom = 64;  // groups of tiles from which the group counts get their own scan
+
+// keys per thread of a tile of the three-kernel radix passes
+inline int radix_ipt_for(int64_t n) { return n <= kSmallBatch ? kIptSmall : kIpt; }
 
 // ---- key transforms ---------------------------------------------------------
 template <typename KeyT>
@@ -100,7 +105,7 @@ template <typename KeyT, bool FIRST, int IPT>
 __global__ __launch_bounds__(kGroup * kThreads) void radix_count_kernel(
     const void* __restrict__ keys_in, int64_t n, int shift, uint32_t mask,
     uint32_t* __restrict__ cnt, uint32_t* __restrict__ gcnt, int64_t ntiles, int64_t id_bound,
-    int32_t* __restrict__ bad_blk) {
+    int32_t* __restrict__ bad_blk, int64_t nbad) {
   __shared__ uint32_t s_hist[kGroup][kBins];
   const int g = threadIdx.x / kThreads;  // the tile of the group this thread counts
   const int t = threadIdx.x % kThreads;  // kThreads == kBins: also the digit it writes out
@@ -141,6 +146,9 @@ __global__ __launch_bounds__(kGroup * kThreads) void radix_count_kernel(
   // every block on every call, so the flags need no clearing and are never stale
   const int any_bad = __syncthreads_or(FIRST && bad ? 1 : 0);
   if (FIRST && threadIdx.x == 0) bad_blk[blockIdx.x] = any_bad;
+  // the flags of the blocks a launch with larger tiles would have had: block 0 clears them
+  if (FIRST && blockIdx.x == 0)
+    for (int64_t f = gridDim.x + threadIdx.x; f < nbad; f += kGroup * kThreads) bad_blk[f] = 0;
   if (tile < ntiles) cnt[tile * kBins + t] = s_hist[g][t];
   if (g == 0) {
     uint32_t sum = 0;
@@ -1456,7 +1464,7 @@ void carve_sort(Carver& c, int64_t n, SortWs* w) {
   w->status = c.take<uint32_t>(kSweepStatusWords);
   for (int i = 0; i < 2; ++i) w->keys[i] = c.take<uint64_t>(nn);  // sized for 64-bit keys
   for (int i = 0; i < 2; ++i) w->vals[i] = c.take<uint32_t>(nn);
-  w->cnt_len = make_plan(nn, 1, 0, true).ntiles * kBins;  // the tile count depends on n only
+  w->cnt_len = ceil_div(nn, kThreads * radix_ipt_for(nn)) * kBins;  // the tile count depends on n only
   w->nchunks = ceil_div(nn, kHistChunk);
   const int64_t ngroups = ceil_div(w->cnt_len / kBins, kGroup);
   w->nbad = ngroups > w->nchunks ? ngroups : w->nchunks;
@@ -1512,12 +1520,16 @@ template <typename KeyT>
 int run_sort_three_kernels(const int64_t* idx, int64_t n, int64_t id_bound, const Plan& p,
                            const SortWs& w, hipStream_t st, const void** keys_out,
                            const uint32_t** perm_out) {
-  const int64_t ngroups = ceil_div(p.ntiles, kGroup);
-  HADES_REQUIRE(p.ntiles * kBins <= w.cnt_len, "internal: radix count buffer too small");
-  constexpr int IPT = kIpt;
-  const dim3 grid(static_cast<unsigned>(p.ntiles)), cgrid(static_cast<unsigned>(ngroups)),
+  // 65 536 keys in tiles of 1 024 are 64 blocks a kernel; in tiles of 512 every block's chain of
+  // ranking rounds is half as long and twice as many compute units work (whole cfg1 step 76.5 ->
+  // 71.3 us; at 200 000 keys the smaller tiles lose: 159.7 -> 163.2 us, tiles of 256: 173.6 us)
+  const int ipt = radix_ipt_for(n);
+  const int64_t ntiles = ceil_div(n, static_cast<int64_t>(kThreads) * ipt);
+  const int64_t ngroups = ceil_div(ntiles, kGroup);
+  HADES_REQUIRE(ntiles * kBins <= w.cnt_len && ngroups <= w.nbad, "internal: radix count buffer too small");
+  const dim3 grid(static_cast<unsigned>(ntiles)), cgrid(static_cast<unsigned>(ngroups)),
       block(kThreads), cblock(kGroup * kThreads), sgrid(kBins / kWaves);
-  const int scanned = p.scan ? 1 : 0;
+  const int scanned = ngroups > kScanFrom ? 1 : 0;
   const int base = p.key_bits / p.passes, extra = p.key_bits % p.passes;
   int bits_of[kMaxPasses], shift_of[kMaxPasses + 1];
   shift_of[0] = 0;
@@ -1532,21 +1544,23 @@ int run_sort_three_kernels(const int64_t* idx, int64_t n, int64_t id_bound, cons
     const uint32_t mask = (1u << bits_of[pass]) - 1u;
     KeyT* kout = static_cast<KeyT*>(w.keys[cur]);
     uint32_t* vout = w.vals[cur];
+#define HADES_RADIX_PASS(FIRST_, IPT_)                                                              \
+  do {                                                                                              \
+    HADES_LAUNCH((radix_count_kernel<KeyT, FIRST_, IPT_>), cgrid, cblock, 0, st, kin, n,            \
+                 shift_of[pass], mask, w.cnt, w.gcnt, ntiles, id_bound, w.bad, w.nbad);             \
+    if (scanned) HADES_LAUNCH(radix_group_scan_kernel, sgrid, block, 0, st, w.gcnt, ngroups);       \
+    HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, FIRST_, IPT_>), grid,  \
+                       block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,       \
+                       w.gcnt, ngroups, scanned, kout, vout);                                       \
+  } while (0)
     if (pass == 0) {
-      HADES_LAUNCH((radix_count_kernel<KeyT, true, IPT>), cgrid, cblock, 0, st, kin, n,
-                   shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.bad);
-      if (scanned) HADES_LAUNCH(radix_group_scan_kernel, sgrid, block, 0, st, w.gcnt, ngroups);
-      HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, true, IPT>), grid,
-                         block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
-                         w.gcnt, ngroups, scanned, kout, vout);
+      if (ipt == kIptSmall) HADES_RADIX_PASS(true, kIptSmall);
+      else HADES_RADIX_PASS(true, kIpt);
     } else {
-      HADES_LAUNCH((radix_count_kernel<KeyT, false, IPT>), cgrid, cblock, 0, st, kin, n,
-                   shift_of[pass], mask, w.cnt, w.gcnt, p.ntiles, id_bound, w.bad);
-      if (scanned) HADES_LAUNCH(radix_group_scan_kernel, sgrid, block, 0, st, w.gcnt, ngroups);
-      HADES_LAUNCH_TIMED(HADES_KERNEL_RADIX_PASS, st, (radix_pass_kernel<KeyT, false, IPT>), grid,
-                         block, 0, st, kin, vin, n, shift_of[pass], mask, bits_of[pass], w.cnt,
-                         w.gcnt, ngroups, scanned, kout, vout);
+      if (ipt == kIptSmall) HADES_RADIX_PASS(false, kIptSmall);
+      else HADES_RADIX_PASS(false, kIpt);
     }
+#undef HADES_RADIX_PASS
     kin = kout;
     vin = vout;
     cur ^= 1;
