@@ -555,20 +555,26 @@ __global__ __launch_bounds__(kThreads) void sweep_pass_kernel(
 }
 
 // ---- run boundaries ---------------------------------------------------------
-constexpr int kUItems = 8;
+constexpr int kUItems = 8;         // sorted positions per thread of the run kernels ...
+constexpr int kUItemsSmall = 2;    // ... and for batches of up to kRunsSmallBatch ids: more and shorter
+                                   // blocks (whole step with 8 / 4 / 2 positions per thread: cfg1 71.6 /
+                                   // 69.9 / 69.3 us, cfg2 159.8 / 158.3 / 158.0, cfg5 331.7 / 323.5 / 319.3).
+                                   // Every block adds up the counts of the tiles before it, which is
+                                   // quadratic in the number of tiles: larger batches keep larger tiles.
+constexpr int64_t kRunsSmallBatch = 1 << 21;
 constexpr int kUTile = kThreads * kUItems;
 
-template <typename KeyT>
+template <typename KeyT, int ITEMS>
 __global__ __launch_bounds__(kThreads) void run_count_kernel(const KeyT* __restrict__ keys,
                                                             int64_t n,
                                                             uint32_t* __restrict__ blk_cnt) {
   __shared__ uint32_t smem[kWaves + 1];
-  const int64_t j0 = static_cast<int64_t>(blockIdx.x) * kUTile + threadIdx.x * kUItems;
+  const int64_t j0 = static_cast<int64_t>(blockIdx.x) * (kThreads * ITEMS) + threadIdx.x * ITEMS;
   uint32_t c = 0;
   if (j0 < n) {
     KeyT prev = j0 > 0 ? keys[j0 - 1] : KeyT(0);
 #pragma unroll
-    for (int k = 0; k < kUItems; ++k) {
+    for (int k = 0; k < ITEMS; ++k) {
       const int64_t j = j0 + k;
       if (j < n) {
         const KeyT cur = keys[j];
@@ -582,7 +588,7 @@ __global__ __launch_bounds__(kThreads) void run_count_kernel(const KeyT* __restr
   if (threadIdx.x == 0) blk_cnt[blockIdx.x] = total;
 }
 
-template <typename KeyT>
+template <typename KeyT, int ITEMS>
 __global__ __launch_bounds__(kThreads) void run_emit_kernel(
     const KeyT* __restrict__ keys, const uint32_t* __restrict__ perm, int64_t n,
     const uint32_t* __restrict__ blk_cnt, int64_t* __restrict__ uids,
@@ -605,14 +611,14 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
   uint32_t blk_base;
   (void)block_exclusive_sum<uint32_t, kThreads>(before, smem, &blk_base);
 
-  const int64_t j0 = static_cast<int64_t>(blockIdx.x) * kUTile + threadIdx.x * kUItems;
-  uint32_t flag[kUItems];
-  KeyT kk[kUItems];
+  const int64_t j0 = static_cast<int64_t>(blockIdx.x) * (kThreads * ITEMS) + threadIdx.x * ITEMS;
+  uint32_t flag[ITEMS];
+  KeyT kk[ITEMS];
   uint32_t c = 0;
   if (j0 < n) {
     KeyT prev = j0 > 0 ? keys[j0 - 1] : KeyT(0);
 #pragma unroll
-    for (int k = 0; k < kUItems; ++k) {
+    for (int k = 0; k < ITEMS; ++k) {
       const int64_t j = j0 + k;
       flag[k] = 0;
       if (j < n) {
@@ -628,7 +634,7 @@ __global__ __launch_bounds__(kThreads) void run_emit_kernel(
   // u = number of runs that begin before j0
   if (j0 < n) {
 #pragma unroll
-    for (int k = 0; k < kUItems; ++k) {
+    for (int k = 0; k < ITEMS; ++k) {
       const int64_t j = j0 + k;
       if (j < n) {
         u += flag[k];
@@ -1496,7 +1502,7 @@ Ws carve(void* ws, int64_t n, int64_t dim) {
   Ws w;
   const int64_t nn = n > 0 ? n : 1;
   carve_sort(c, n, &w.sort);
-  w.run_cnt = c.take<uint32_t>(ceil_div(nn, kUTile) + 1);
+  w.run_cnt = c.take<uint32_t>(ceil_div(nn, kThreads * kUItemsSmall) + 1);
   w.seg_of = c.take<uint32_t>(nn);
   w.seg_start = c.take<uint32_t>(nn + 1);
   // at most two partial rows per block of the FAST sum; the smallest block span is four chunks
@@ -1647,12 +1653,23 @@ int run_runs(const void* sorted_keys, const uint32_t* perm, int64_t n, const Pla
                  key_from_id<KeyT>(threshold), class_split, first_pos);
     return HADES_OK;
   }
-  HADES_LAUNCH((run_count_kernel<KeyT>), rgrid, block, 0, st, keys, n, w.run_cnt);
-  HADES_LAUNCH_CHECK();
-  HADES_LAUNCH((run_emit_kernel<KeyT>), rgrid, block, 0, st, keys, perm, n, w.run_cnt, uids,
-                     w.seg_start, w.seg_of, num_unique, inverse, w.sort.bad, w.sort.nbad,
-                     key_from_id<KeyT>(threshold), class_split, first_pos);
-  HADES_LAUNCH_CHECK();
+  static const int items_env = [] { const char* e = getenv("HADES_RUN_ITEMS"); return e ? atoi(e) : 0; }();
+  int items = n <= kRunsSmallBatch ? kUItemsSmall : kUItems;
+  if (items_env == 2 || items_env == 4 || items_env == 8) items = items_env;
+  const dim3 sgrid(static_cast<unsigned>(ceil_div(n, static_cast<int64_t>(kThreads) * items)));
+#define HADES_RUNS(ITEMS_)                                                                          \
+  do {                                                                                              \
+    HADES_LAUNCH((run_count_kernel<KeyT, ITEMS_>), sgrid, block, 0, st, keys, n, w.run_cnt);        \
+    HADES_LAUNCH_CHECK();                                                                           \
+    HADES_LAUNCH((run_emit_kernel<KeyT, ITEMS_>), sgrid, block, 0, st, keys, perm, n, w.run_cnt,    \
+                 uids, w.seg_start, w.seg_of, num_unique, inverse, w.sort.bad, w.sort.nbad,         \
+                 key_from_id<KeyT>(threshold), class_split, first_pos);                             \
+    HADES_LAUNCH_CHECK();                                                                           \
+  } while (0)
+  if (items == 2) HADES_RUNS(2);
+  else if (items == 4) HADES_RUNS(4);
+  else HADES_RUNS(8);
+#undef HADES_RUNS
   return HADES_OK;
 }
 
