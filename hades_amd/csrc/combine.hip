@@ -52,10 +52,14 @@ constexpr int kGroup = 4;  // tiles counted by one block of the count kernel
 constexpr int kIpt = 4;    // keys per thread in a radix tile: tiles of 1024 keys
 constexpr int kIptSmall = 2;             // ... tiles of 512 keys for batches of up to kSmallBatch ids:
 constexpr int64_t kSmallBatch = 1 << 17; // they would leave three quarters of the chip without a tile
+constexpr int kIptLarge = 8;             // ... and tiles of 2 048 keys for batches above kLargeBatch ids
+constexpr int64_t kLargeBatch = 1 << 19;
 constexpr int kScanFrom = 64;  // groups of tiles from which the group counts get their own scan
 
 // keys per thread of a tile of the three-kernel radix passes
-inline int radix_ipt_for(int64_t n) { return n <= kSmallBatch ? kIptSmall : kIpt; }
+inline int radix_ipt_for(int64_t n) {
+  return n <= kSmallBatch ? kIptSmall : (n > kLargeBatch ? kIptLarge : kIpt);
+}
 
 // ---- key transforms ---------------------------------------------------------
 template <typename KeyT>
@@ -1470,7 +1474,9 @@ void carve_sort(Carver& c, int64_t n, SortWs* w) {
   w->status = c.take<uint32_t>(kSweepStatusWords);
   for (int i = 0; i < 2; ++i) w->keys[i] = c.take<uint64_t>(nn);  // sized for 64-bit keys
   for (int i = 0; i < 2; ++i) w->vals[i] = c.take<uint32_t>(nn);
-  w->cnt_len = ceil_div(nn, kThreads * radix_ipt_for(nn)) * kBins;  // the tile count depends on n only
+  // the tile count depends on n only; the one-sweep form keeps its tile states here, kIpt keys per thread
+  const int ipt_min = radix_ipt_for(nn) < kIpt ? radix_ipt_for(nn) : kIpt;
+  w->cnt_len = ceil_div(nn, kThreads * ipt_min) * kBins;
   w->nchunks = ceil_div(nn, kHistChunk);
   const int64_t ngroups = ceil_div(w->cnt_len / kBins, kGroup);
   w->nbad = ngroups > w->nchunks ? ngroups : w->nchunks;
@@ -1529,6 +1535,7 @@ int run_sort_three_kernels(const int64_t* idx, int64_t n, int64_t id_bound, cons
   // 65 536 keys in tiles of 1 024 are 64 blocks a kernel; in tiles of 512 every block's chain of
   // ranking rounds is half as long and twice as many compute units work (whole cfg1 step 76.5 ->
   // 71.3 us; at 200 000 keys the smaller tiles lose: 159.7 -> 163.2 us, tiles of 256: 173.6 us)
+  // (one million keys: tiles of 2 048 take 5 us off the sort, 194 -> 189 us for cfg5's combine)
   const int ipt = radix_ipt_for(n);
   const int64_t ntiles = ceil_div(n, static_cast<int64_t>(kThreads) * ipt);
   const int64_t ngroups = ceil_div(ntiles, kGroup);
@@ -1561,9 +1568,11 @@ int run_sort_three_kernels(const int64_t* idx, int64_t n, int64_t id_bound, cons
   } while (0)
     if (pass == 0) {
       if (ipt == kIptSmall) HADES_RADIX_PASS(true, kIptSmall);
+      else if (ipt == kIptLarge) HADES_RADIX_PASS(true, kIptLarge);
       else HADES_RADIX_PASS(true, kIpt);
     } else {
       if (ipt == kIptSmall) HADES_RADIX_PASS(false, kIptSmall);
+      else if (ipt == kIptLarge) HADES_RADIX_PASS(false, kIptLarge);
       else HADES_RADIX_PASS(false, kIpt);
     }
 #undef HADES_RADIX_PASS
