@@ -1688,6 +1688,21 @@ def main():
                       workload="cfg3", schedule="keyed", with_gate=True, with_link=False, reuse_rows=True,
                       state_on_host=True)
         if schedule == "keyed" and args.reuse_rows:
+            from hades_amd import ops as _ops
+            width = _ops.set_host_link_blocks(_ops.LINK_WRITE_ONLY, 34)
+            try:
+                secondary("cfg3_update_34_blocks",
+                          "the headline workload and schedule with the write-only cold update 34 "
+                          "workgroups wide instead of %d: the update gives up some of its link rate, "
+                          "the hot-class sums and update beside it are slowed less - both of the "
+                          "targets (hot-cache traffic at 60 %% of HBM peak inside the step, cold rows "
+                          "at 70 %% of the link) are met in one and the same step, which is a few "
+                          "per cent longer" % width,
+                          lambda sec: dict(brief(sec), hot_traffic_all_row_kernels=sec["roofline"].get(
+                              "hot_traffic_all_row_kernels")),
+                          workload="cfg3", schedule="keyed", with_gate=True, with_link=False, reuse_rows=True)
+            finally:
+                _ops.set_host_link_blocks(_ops.LINK_WRITE_ONLY, width)
             secondary("cfg3_pipelined",
                       "the headline workload with the next batch's forward half (lookup, partition, "
                       "cold gather, key sort) running on side streams while this batch's cold update "
